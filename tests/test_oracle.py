@@ -1,0 +1,449 @@
+"""Pins the CPU checker (oracle/) before anything is compared against it.
+
+Each test checks the restatement against something it does not itself define:
+published known-answer vectors, the fixture the reference's own harness holds,
+exact rational arithmetic on tiny inputs, library routines (numpy / scipy /
+torch) or invariants that a plausible mistake (dropped term, wrong index,
+transposed operand) breaks.
+"""
+import ctypes as C
+import os
+from fractions import Fraction
+
+import numpy as np
+import pytest
+
+from helpers import QB, block_amax, block_view, expand_scales, rand_codes, rand_scales
+
+GOLD = os.path.join(os.path.dirname(__file__), "golden")
+
+
+# ----------------------------------------------------------------------------- Philox
+# Random123 known-answer vectors for philox4x32-10 (kat_vectors of the Random123 distribution).
+PHILOX_KAT = [
+    ([0, 0, 0, 0], [0, 0], [0x6627E8D5, 0xE169C58D, 0xBC57AC4C, 0x9B00DBD8]),
+    ([0xFFFFFFFF] * 4, [0xFFFFFFFF] * 2, [0x408F276D, 0x41C83B0E, 0xA20BC7C6, 0x6D5451FD]),
+    ([0x243F6A88, 0x85A308D3, 0x13198A2E, 0x03707344], [0xA4093822, 0x299F31D0],
+     [0xD16CFE09, 0x94FDCCEB, 0x5001E420, 0x24126EA1]),
+]
+
+
+@pytest.mark.parametrize("ctr,key,want", PHILOX_KAT)
+def test_philox_known_answers(oracle, ctr, key, want):
+    assert oracle.philox4x32_10(ctr, key).tolist() == want
+
+
+def test_sr_noise_layout_and_range(oracle):
+    # 8 consecutive elements share one Philox call, 16 bits each, low half first.
+    seed, offset = 0x0123456789ABCDEF, 5
+    for base in (0, 8, 8 * 12345):
+        c = offset + base // 8
+        words = oracle.philox4x32_10([c & 0xFFFFFFFF, c >> 32, 0, 0], [seed & 0xFFFFFFFF, seed >> 32])
+        for lane in range(8):
+            w = int(words[lane // 2])
+            h = (w >> 16) if lane & 1 else (w & 0xFFFF)
+            want = np.float32((h + 0.5) / 65536.0 - 0.5)
+            assert oracle.sr_noise(seed, offset, base + lane) == want
+    n = np.array([oracle.sr_noise(1, 0, e) for e in range(40000)])
+    assert n.min() > -0.5 and n.max() < 0.5
+    assert abs(n.mean()) < 4 * (1 / np.sqrt(12)) / np.sqrt(n.size)
+    hist, _ = np.histogram(n, bins=16, range=(-0.5, 0.5))
+    chi2 = ((hist - n.size / 16) ** 2 / (n.size / 16)).sum()
+    assert chi2 < 45.0  # 15 dof, p ~ 1e-4
+
+
+def test_f16_conversion_matches_numpy(oracle):
+    rng = np.random.default_rng(1)
+    vals = np.concatenate([
+        (rng.standard_normal(20000) * np.exp2(rng.integers(-30, 18, 20000))).astype(np.float32),
+        np.array([0.0, -0.0, 65504.0, 65519.9, 65520.0, 1e9, 5.96e-8, 2.98e-8, 2.9802322e-8, 6.1e-5,
+                  6.0975552e-5, 1.0, 1.00048828125, 1.0009765625], dtype=np.float32),
+    ])
+    want = vals.astype(np.float16).view(np.uint16)
+    got = np.array([oracle.f32_to_f16_bits(v) for v in vals], dtype=np.uint16)
+    assert np.array_equal(got, want)
+    L = oracle.lib()
+    back = np.array([L.jfo_f16_bits_to_f32(int(b)) for b in want], dtype=np.float32)
+    assert np.array_equal(back.view(np.uint32), want.view(np.float16).astype(np.float32).view(np.uint32))
+
+
+# ----------------------------------------------------------------------------- integer GEMM
+def _load_txt(name, shape):
+    return np.loadtxt(os.path.join(GOLD, name), dtype=np.int64).reshape(shape)
+
+
+def test_igemm_s32_reference_fixture(oracle):
+    """The A/B/CPU dump of JetfireGEMMKernel/cppsrc/igemm/igemm_BasicInt8Gemm_128_128_32."""
+    A = _load_txt("basic_int8_gemm_128_128_32_A.txt", (128, 32))
+    B = _load_txt("basic_int8_gemm_128_128_32_B.txt", (32, 128))
+    Cw = _load_txt("basic_int8_gemm_128_128_32_C.txt", (128, 128))
+    assert np.array_equal(A @ B, Cw)
+    got = oracle.igemm_s32(A.astype(np.int8), B.astype(np.int8), b_layout=1)
+    assert np.array_equal(got, Cw)
+    got_nk = oracle.igemm_s32(A.astype(np.int8), np.ascontiguousarray(B.T).astype(np.int8), b_layout=0)
+    assert np.array_equal(got_nk, Cw)
+
+
+@pytest.mark.parametrize("M,N,K", [(32, 32, 32), (64, 96, 160), (128, 256, 32), (96, 160, 224)])
+def test_igemm_s32_and_block_acc_vs_numpy(oracle, M, N, K):
+    rng = np.random.default_rng(M + N + K)
+    A = rand_codes(rng, (M, K))
+    Bkn = rand_codes(rng, (K, N))
+    want = A.astype(np.int64) @ Bkn.astype(np.int64)
+    assert np.array_equal(oracle.igemm_s32(A, Bkn, 1), want)
+    assert np.array_equal(oracle.igemm_s32(A, np.ascontiguousarray(Bkn.T), 0), want)
+    acc = oracle.igemm_block_acc(A, Bkn, 1)
+    assert acc.shape == (K // QB, M, N)
+    for kb in range(K // QB):
+        w = A[:, kb * QB:(kb + 1) * QB].astype(np.int64) @ Bkn[kb * QB:(kb + 1) * QB].astype(np.int64)
+        assert np.array_equal(acc[kb], w)
+    assert np.abs(acc).max() <= 32 * 127 * 127
+    assert np.array_equal(acc.astype(np.int64).sum(axis=0), want)
+    assert np.array_equal(oracle.igemm_block_acc(A, np.ascontiguousarray(Bkn.T), 0), acc)
+
+
+def test_igemm_extreme_codes(oracle):
+    A = np.full((32, 64), -127, np.int8)
+    B = np.full((64, 32), 127, np.int8)
+    acc = oracle.igemm_block_acc(A, B, 1)
+    assert np.all(acc == -32 * 127 * 127)
+
+
+# ----------------------------------------------------------------------------- dequantise-accumulate
+def _round_f32(fr):
+    """Correctly rounded (ties-to-even) binary32 value of a Fraction, as a Fraction."""
+    if fr == 0:
+        return Fraction(0)
+    sign = -1 if fr < 0 else 1
+    a = abs(fr)
+    e = 0
+    while a >= 2 ** 24:
+        a /= 2
+        e += 1
+    while a < 2 ** 23:
+        a *= 2
+        e -= 1
+    n = round(a)  # Fraction.__round__ is half-even
+    return sign * Fraction(n) * (Fraction(2) ** e)
+
+
+def test_block_f32_is_ascending_fma_chain_exact_rational(oracle):
+    """Brute force with exact rationals: acc <- RN(sa*sb*d + acc), kb ascending."""
+    rng = np.random.default_rng(7)
+    M, N, K = 32, 64, 96
+    A = rand_codes(rng, (M, K))
+    Bkn = rand_codes(rng, (K, N))
+    sa = rand_scales(rng, (K // QB, M // QB))
+    sb = rand_scales(rng, (K // QB, N // QB))
+    got = oracle.igemm_block_f32(A, Bkn, sa, sb, 1, fused=True)
+    got_unfused = oracle.igemm_block_f32(A, Bkn, sa, sb, 1, fused=False)
+    pts = [(int(rng.integers(M)), int(rng.integers(N))) for _ in range(160)]
+    for m, n in pts:
+        acc = Fraction(0)
+        acc_u = Fraction(0)
+        for kb in range(K // QB):
+            d = int(A[m, kb * QB:(kb + 1) * QB].astype(np.int64) @ Bkn[kb * QB:(kb + 1) * QB, n].astype(np.int64))
+            sab = _round_f32(Fraction(float(sa[kb, m // QB])) * Fraction(float(sb[kb, n // QB])))
+            acc = _round_f32(sab * d + acc)
+            acc_u = _round_f32(_round_f32(sab * d) + acc_u)
+        assert Fraction(float(got[m, n])) == acc
+        assert Fraction(float(got_unfused[m, n])) == acc_u
+
+
+@pytest.mark.parametrize("b_layout", [0, 1])
+def test_block_f32_vs_float64_matmul(oracle, b_layout):
+    """A transposed or mis-indexed scale operand shows up as an O(1) error here."""
+    rng = np.random.default_rng(11)
+    M, N, K = 96, 160, 224
+    A = rand_codes(rng, (M, K))
+    Bkn = rand_codes(rng, (K, N))
+    sx = rand_scales(rng, (M // QB, K // QB))     # natural layout, as the reference tests build it
+    sw = rand_scales(rng, (K // QB, N // QB))
+    want = (A * expand_scales(sx).astype(np.float64)) @ (Bkn * expand_scales(sw).astype(np.float64))
+    B = Bkn if b_layout == 1 else np.ascontiguousarray(Bkn.T)
+    got = oracle.igemm_block_f32(A, B, np.ascontiguousarray(sx.T), sw, b_layout)
+    assert np.abs(got - want).max() <= 2e-6 * np.abs(want).max()
+
+
+# ----------------------------------------------------------------------------- requantising epilogues
+def test_requant_det_invariants_and_vectorised_form(oracle):
+    rng = np.random.default_rng(3)
+    acc = (rng.standard_normal((96, 128)) * np.exp2(rng.integers(-6, 6, (96, 128)))).astype(np.float32)
+    acc[32:64, 32:64] = 0.0                       # an all-zero block
+    q, sc = oracle.requant(acc)
+    amax = block_amax(acc)
+    assert np.array_equal(sc, (amax / np.float32(127.0)).astype(np.float32))
+    qb = block_view(q)
+    assert np.abs(q).max() <= 127
+    nz = amax > 0
+    assert np.all(np.abs(qb).max(axis=(2, 3))[nz] == 127)
+    assert np.all(qb[~nz] == 0) and np.all(sc[~nz] == 0)
+    deq = q.astype(np.float64) * expand_scales(sc)
+    assert np.all(np.abs(deq - acc) <= expand_scales(sc) * 0.5 * (1 + 1e-5) + 1e-30)
+    with np.errstate(invalid="ignore", divide="ignore"):
+        t = (np.float32(127.0) * acc) / expand_scales(amax)
+    want = np.where(expand_scales(amax) > 0, np.clip(np.rint(t), -127, 127), 0).astype(np.int8)
+    assert np.array_equal(q, want)
+
+
+def test_requant_bias_and_biasmax(oracle):
+    rng = np.random.default_rng(4)
+    acc = rng.standard_normal((64, 64)).astype(np.float32)
+    bias = (0.1 * rng.standard_normal(64)).astype(np.float32)
+    biasmax = float(np.abs(bias).max())
+    q, sc = oracle.requant(acc, bias=bias, biasmax=biasmax)
+    amax = (block_amax(acc) + np.float32(biasmax)).astype(np.float32)
+    assert np.array_equal(sc, amax / np.float32(127.0))
+    t = (np.float32(127.0) * (acc + bias[None, :])) / expand_scales(amax)
+    assert np.array_equal(q, np.clip(np.rint(t), -127, 127).astype(np.int8))
+
+
+def test_unit_scale_k32_reduces_to_quantising_an_integer_matrix(oracle):
+    rng = np.random.default_rng(5)
+    A = rand_codes(rng, (64, 32))
+    B = rand_codes(rng, (32, 64))
+    one = np.ones((1, 2), np.float32)
+    q, sc = oracle.igemm_block_q(A, B, one, one, 1)
+    d = (A.astype(np.int64) @ B.astype(np.int64)).astype(np.float32)
+    q2, s2 = oracle.requant(d)
+    assert np.array_equal(q, q2) and np.array_equal(sc, s2)
+    assert np.array_equal(oracle.igemm_block_fp(A, B, one, one, 1, "f32"), d)
+
+
+def test_requant_sr_unbiased_and_bounded(oracle):
+    """Mean over R independent draws converges to the un-rounded value like R^-1/2
+    (the check of JetfireGEMMKernel/tests/test_int8igemmoutputIntQuantizeStochastic.py:70-120)."""
+    rng = np.random.default_rng(6)
+    acc = rng.standard_normal((64, 64)).astype(np.float32)
+    amax = expand_scales(block_amax(acc))
+    t = (np.float32(127.0) * acc) / amax
+    errs = []
+    for R in (16, 256):
+        m = np.zeros_like(t, dtype=np.float64)
+        for r in range(R):
+            q, sc = oracle.requant(acc, stochastic=True, seed=99, offset=r * 4096)
+            assert np.all(np.abs(q.astype(np.float64) - t) < 1.0 + 1e-6)
+            m += q
+        errs.append(np.sqrt(np.mean((m / R - t) ** 2)))
+    # rms error of a mean of R Bernoulli roundings: <= 0.5/sqrt(R), ~0.41/sqrt(R) on average
+    assert errs[0] < 0.5 / 4 and errs[1] < 0.5 / 16
+    assert 2.5 < errs[0] / errs[1] < 6.5
+    q0, _ = oracle.requant(acc, stochastic=True, seed=99, offset=0)
+    q1, _ = oracle.requant(acc, stochastic=True, seed=99, offset=0)
+    q2, _ = oracle.requant(acc, stochastic=True, seed=100, offset=0)
+    assert np.array_equal(q0, q1) and not np.array_equal(q0, q2)
+    qd, _ = oracle.requant(acc)
+    assert np.abs(q0.astype(int) - qd.astype(int)).max() <= 1
+
+
+# ----------------------------------------------------------------------------- quantise / dequantise / transpose
+def test_quantize_matches_reference_test_formula(oracle):
+    """(x / s).round() with s = amax/127 -- JetfireGEMMKernel/tests/…Deterministic.py:26-30."""
+    import torch
+    rng = np.random.default_rng(8)
+    x = (rng.standard_normal((96, 160)) * np.exp2(rng.integers(-8, 4, (96, 160)))).astype(np.float32)
+    q, s = oracle.quantize(x)
+    xt = torch.from_numpy(x)
+    bv = xt.reshape(3, 32, 5, 32).permute(0, 2, 1, 3)
+    st = bv.abs().amax(dim=(2, 3)) / 127
+    qt = (bv / st[:, :, None, None]).round().to(torch.int8).permute(0, 2, 1, 3).reshape(96, 160)
+    assert np.array_equal(s, st.numpy())
+    assert np.array_equal(q, qt.numpy())
+    q16, s16 = oracle.quantize(x, scale_dtype="f16")
+    assert s16.dtype == np.float16 and np.array_equal(q16, q)       # scale is rounded AFTER use
+    assert np.array_equal(s16, st.to(torch.float16).numpy())
+
+
+def test_quantize_properties(oracle):
+    from hypothesis import given, settings, strategies as st
+
+    @settings(max_examples=40, deadline=None)
+    @given(st.integers(0, 2 ** 31), st.integers(-20, 10), st.booleans())
+    def run(seed, e, stochastic):
+        rng = np.random.default_rng(seed)
+        x = (rng.standard_normal((32, 64)) * 2.0 ** e).astype(np.float32)
+        x[:, 32:] *= (rng.random((32, 32)) < 0.1)
+        q, s = oracle.quantize(x, stochastic=stochastic, seed=seed, offset=3)
+        assert np.abs(q).max() <= 127
+        err = np.abs(q * expand_scales(s).astype(np.float64) - x)
+        bound = (1.0 if stochastic else 0.5) * expand_scales(s) * (1 + 1e-5)
+        assert np.all(err <= bound + 1e-37)
+        if not stochastic:
+            assert np.all(np.abs(block_view(q)).max(axis=(2, 3))[block_amax(x) > 0] == 127)
+            # idempotent on already-quantised data
+            x2 = oracle.dequantize(q, s)
+            q2, s2 = oracle.quantize(x2)
+            assert np.array_equal(q2, q)
+
+    run()
+    q, s = oracle.quantize(np.zeros((32, 32), np.float32))
+    assert not q.any() and s[0, 0] == 0.0
+
+
+def test_quantize_sr_unbiased(oracle):
+    rng = np.random.default_rng(9)
+    x = rng.standard_normal((32, 32)).astype(np.float32)
+    s = np.float32(np.abs(x).max()) / np.float32(127.0)
+    y = x / s
+    R = 400
+    m = np.zeros_like(y, dtype=np.float64)
+    for r in range(R):
+        q, _ = oracle.quantize(x, stochastic=True, seed=7, offset=1000 * r)
+        m += q
+    assert np.sqrt(np.mean((m / R - y) ** 2)) < 0.5 / np.sqrt(R)
+    assert abs(np.mean(m / R - y)) < 4 * 0.41 / np.sqrt(R * y.size)
+
+
+def test_quantize_truncate_mode(oracle):
+    """The `.to(int8)` without llrint of Jetfire/Nonlinear/add.py:139 rounds toward zero."""
+    rng = np.random.default_rng(10)
+    x = rng.standard_normal((32, 32)).astype(np.float32)
+    q, s = oracle.quantize(x, truncate=True)
+    assert np.array_equal(q, np.trunc(x / s[0, 0]).astype(np.int8))
+
+
+def test_dequantize_transpose(oracle):
+    rng = np.random.default_rng(12)
+    q = rand_codes(rng, (64, 96))
+    s = rand_scales(rng, (2, 3))
+    assert np.array_equal(oracle.dequantize(q, s), q.astype(np.float32) * expand_scales(s))
+    assert np.array_equal(oracle.transpose_s8(q), q.T)
+
+
+def test_fast_division_model_equals_ieee(oracle):
+    """x*r corrected by two fmas (what the kernels do for a block-constant divisor) == x/s."""
+    L = oracle.lib()
+    L.jfo_model_fast_div_mismatches.argtypes = [C.c_void_p, C.c_void_p, C.c_long]
+    L.jfo_model_fast_div_mismatches.restype = C.c_long
+    rng = np.random.default_rng(13)
+    n = 2_000_000
+    s = (rng.uniform(1, 2, n) * np.exp2(rng.integers(-60, 60, n))).astype(np.float32)
+    for x in (rng.uniform(-127.5, 127.5, n) * s.astype(np.float64),
+              rng.uniform(-1, 1, n) * np.exp2(rng.integers(-30, 8, n)) * s.astype(np.float64)):
+        x = x.astype(np.float32)
+        assert L.jfo_model_fast_div_mismatches(x.ctypes.data, s.ctypes.data, n) == 0
+
+
+# ----------------------------------------------------------------------------- elementary functions
+def test_exp_erfc_cdf_tanh_vs_scipy(oracle):
+    import scipy.special as sp
+    x = np.linspace(-87, 88, 5001).astype(np.float32)
+    ref = np.exp(x.astype(np.float64))
+    assert np.max(np.abs(oracle.expf(x) - ref) / ref) < 2e-7
+    z = np.linspace(0, 9, 4001).astype(np.float32)
+    ref = sp.erfc(z.astype(np.float64))
+    assert np.max(np.abs(oracle.erfc_pos(z) - ref) / ref) < 1e-5
+    x = np.linspace(-8, 8, 4001).astype(np.float32)
+    ref = sp.ndtr(x.astype(np.float64))
+    assert np.max(np.abs(oracle.norm_cdf(x) - ref) / ref) < 1e-5
+    u = np.linspace(-20, 20, 4001).astype(np.float32)
+    assert np.max(np.abs(oracle.tanhf(u) - np.tanh(u.astype(np.float64)))) < 3e-7
+
+
+@pytest.mark.parametrize("approx,name", [(0, "none"), (1, "tanh")])
+def test_gelu_and_derivative_vs_torch(oracle, approx, name):
+    import torch
+    x = np.concatenate([np.linspace(-9, 9, 3001), [0.0, -0.0, 1e-6, -1e-6]]).astype(np.float32)
+    xt = torch.tensor(x, dtype=torch.float64, requires_grad=True)
+    yt = torch.nn.functional.gelu(xt, approximate=name)
+    yt.sum().backward()
+    assert np.max(np.abs(oracle.gelu(x, approx) - yt.detach().numpy())) < 1.5e-6
+    assert np.max(np.abs(oracle.dgelu(x, approx) - xt.grad.numpy())) < 2e-6
+
+
+# ----------------------------------------------------------------------------- fused nonlinear ops
+def _rand_block_tensor(rng, R, Cc, scale=1.0):
+    x = (rng.standard_normal((R, Cc)) * scale).astype(np.float32)
+    from oracle import oracle as O
+    q, s = O.quantize(x, scale_dtype="f16")
+    return q, s.astype(np.float32)
+
+
+def _check_block_quant_of(oracle, y, q, s, amax_eps=0.0, stochastic=False):
+    """(q, s) must be the block quantisation of the float64 matrix y, up to fp32 noise in y."""
+    amax = block_amax(y) + amax_eps
+    assert np.allclose(s, amax / 127.0, rtol=2e-5, atol=1e-30)
+    t = y / expand_scales(np.maximum(s, 1e-30))
+    lim = 1.0 if stochastic else 0.5
+    assert np.all(np.abs(q - t) <= lim + 2e-3)
+
+
+@pytest.mark.parametrize("approx,name,eps", [(0, "none", 5e-5), (1, "tanh", 0.0)])
+def test_gelu_fwd_bwd_block_ops_vs_torch(oracle, approx, name, eps):
+    import torch
+    rng = np.random.default_rng(20 + approx)
+    qx, sx = _rand_block_tensor(rng, 64, 96, 1.5)
+    qg, sg = _rand_block_tensor(rng, 64, 96, 1e-3)
+    x = torch.tensor(qx * expand_scales(sx).astype(np.float64), requires_grad=True)
+    g = torch.tensor(qg * expand_scales(sg).astype(np.float64))
+    y = torch.nn.functional.gelu(x, approximate=name)
+    y.backward(g)
+    qy, sy = oracle.gelu_fwd(qx, sx, approx=approx, amax_eps=eps)
+    _check_block_quant_of(oracle, y.detach().numpy(), qy, sy, amax_eps=eps)
+    qd, sd = oracle.gelu_bwd(qx, sx, qg, sg, approx=approx)
+    _check_block_quant_of(oracle, x.grad.numpy(), qd, sd)
+    qs, ss = oracle.gelu_bwd(qx, sx, qg, sg, approx=approx, stochastic=True, seed=5, offset=0)
+    assert np.array_equal(ss, sd)
+    _check_block_quant_of(oracle, x.grad.numpy(), qs, ss, stochastic=True)
+    assert not np.array_equal(qs, qd)
+
+
+def test_rowstats_vs_numpy(oracle):
+    rng = np.random.default_rng(30)
+    q, s = _rand_block_tensor(rng, 64, 160, 2.0)
+    x = q * expand_scales(s).astype(np.float64)
+    mean, rstd = oracle.rowstats(q, s, eps=1e-5)
+    assert np.allclose(mean, x.mean(axis=1), rtol=1e-5, atol=1e-6)
+    assert np.allclose(rstd, 1 / np.sqrt(x.var(axis=1) + 1e-5), rtol=2e-5)
+
+
+def test_layernorm_fwd_bwd_vs_torch(oracle):
+    """torch.nn.functional.layer_norm + autograd on the dequantised input is the library routine
+    (it is also what Jetfire/Nonlinear/layernorm.py:649,661-662 compares with)."""
+    import torch
+    rng = np.random.default_rng(31)
+    R, Cc = 64, 160
+    qx, sx = _rand_block_tensor(rng, R, Cc, 1.0)
+    qg, sg = _rand_block_tensor(rng, R, Cc, 1e-3)
+    gamma = (1 + 0.1 * rng.standard_normal(Cc)).astype(np.float32)
+    beta = (0.1 * rng.standard_normal(Cc)).astype(np.float32)
+    eps = 1e-5
+    mean, rstd = oracle.rowstats(qx, sx, eps=eps)
+    x = torch.tensor(qx * expand_scales(sx).astype(np.float64), requires_grad=True)
+    gt = torch.tensor(gamma.astype(np.float64), requires_grad=True)
+    bt = torch.tensor(beta.astype(np.float64), requires_grad=True)
+    y = torch.nn.functional.layer_norm(x, (Cc,), gt, bt, eps)
+    g = torch.tensor(qg * expand_scales(sg).astype(np.float64))
+    y.backward(g)
+    qy, sy = oracle.layernorm_fwd(qx, sx, gamma, beta, mean, rstd)
+    _check_block_quant_of(oracle, y.detach().numpy(), qy, sy)
+    qy0, sy0 = oracle.layernorm_fwd(qx, sx, gamma, None, mean, rstd)
+    y0 = torch.nn.functional.layer_norm(x, (Cc,), gt, None, eps)
+    _check_block_quant_of(oracle, y0.detach().numpy(), qy0, sy0)
+    qd, sd, dgamma, dbeta = oracle.layernorm_bwd(qx, sx, qg, sg, gamma, mean, rstd)
+    _check_block_quant_of(oracle, x.grad.numpy(), qd, sd)
+    assert np.allclose(dgamma, gt.grad.numpy(), rtol=1e-4, atol=1e-7)
+    assert np.allclose(dbeta, bt.grad.numpy(), rtol=1e-4, atol=1e-7)
+    qs, ss, _, _ = oracle.layernorm_bwd(qx, sx, qg, sg, gamma, mean, rstd, stochastic=True, seed=1)
+    _check_block_quant_of(oracle, x.grad.numpy(), qs, ss, stochastic=True)
+
+
+def test_add_closed_form(oracle):
+    rng = np.random.default_rng(32)
+    R, Cc = 64, 96
+    x1 = rng.standard_normal((R, Cc)).astype(np.float32)
+    q2, s2 = _rand_block_tensor(rng, R, Cc, 0.5)
+    want = x1 + q2.astype(np.float32) * expand_scales(s2)
+    y1, q, s, rs, rq = oracle.add(x1, q2, s2, truncate=True, with_stats=True)
+    assert np.array_equal(y1, want)
+    sw = block_amax(want) / np.float32(127.0)
+    assert np.array_equal(s, sw)
+    assert np.array_equal(q, np.trunc(want / expand_scales(sw)).astype(np.int8))
+    _, qn, _ = oracle.add(x1, q2, s2, truncate=False)
+    assert np.array_equal(qn, np.rint(want / expand_scales(sw)).astype(np.int8))
+    w64 = want.astype(np.float64)
+    assert np.allclose(rs.sum(axis=1), w64.sum(axis=1), rtol=1e-5, atol=1e-4)
+    assert np.allclose(rq.sum(axis=1), (w64 ** 2).sum(axis=1), rtol=1e-5)
+    mean = rs.sum(axis=1) / Cc
+    var = rq.sum(axis=1) / Cc - mean ** 2
+    assert np.allclose(var, w64.var(axis=1), rtol=1e-4)
