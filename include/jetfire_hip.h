@@ -1,0 +1,153 @@
+/*
+ * jetfire_hip.h -- C ABI of libjetfire_hip.so: the gfx950 (MI355X) implementation of the
+ * Jetfire per-block INT8 data-flow path.
+ *
+ * Conventions
+ *   - every pointer is a DEVICE pointer owned by the caller; nothing here allocates, frees,
+ *     synchronises or copies to the host.  Work is enqueued on `stream` (a hipStream_t passed
+ *     as void*; NULL = the default stream).
+ *   - return value: 0 on success, a negative JF_ERR_* for a rejected argument, a positive
+ *     hipError_t if the launch failed.  jf_error_string() names either.
+ *   - a "block tensor" is (q: int8 [R,C] row-major, s: scale [R/32, C/32] row-major), x ~= q*s.
+ *     All of R, C, M, N, K must be positive multiples of 32.  Data pointers must be 16-byte aligned.
+ *   - `scale_dtype` selects the element type of EVERY scale pointer of the call
+ *     (JF_SCALE_F16 = IEEE binary16, what the reference stores; JF_SCALE_F32 = binary32).
+ *   - GEMM scale operands are K-major: sa[kb*(M/32)+mb], sb[kb*(N/32)+nb]; output scales are
+ *     sc[mb*(N/32)+nb]  (reference: …/igemm/igemm_BlockSquare32OutputIntQuantizeBiasRowCol.cu:110-111,
+ *     187-188, 297-304; paths below are relative to JetfireGEMMKernel/BlockQuantize/cpp_extension/).
+ *   - stochastic rounding draws Philox4x32-10 noise keyed by (seed, offset + flat output index / 8),
+ *     16 bits per element, so results do not depend on the launch geometry.
+ */
+#ifndef JETFIRE_HIP_H
+#define JETFIRE_HIP_H
+
+#include <stddef.h>
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+#define JF_OK                 0
+#define JF_ERR_NULL          -1   /* a required pointer is NULL                      */
+#define JF_ERR_SHAPE         -2   /* a dimension is not a positive multiple of 32    */
+#define JF_ERR_ENUM          -3   /* unknown layout / dtype / rounding / approx code */
+#define JF_ERR_ALIGN         -4   /* pointer or leading dimension not 16-byte aligned */
+#define JF_ERR_WORKSPACE     -5   /* workspace missing or smaller than required      */
+#define JF_ERR_DEVICE        -6   /* the current device is not gfx950                */
+
+/* B operand layout of the GEMMs */
+#define JF_B_NK 0                 /* B is [N,K] row-major ("row x col", forward)      */
+#define JF_B_KN 1                 /* B is [K,N] row-major ("row x row", dgrad, wgrad) */
+
+#define JF_SCALE_F16 0
+#define JF_SCALE_F32 1
+
+#define JF_FP_F16  0
+#define JF_FP_F32  1
+#define JF_FP_BF16 2
+
+#define JF_ROUND_NEAREST    0     /* ties-to-even                                    */
+#define JF_ROUND_STOCHASTIC 1
+#define JF_ROUND_TRUNC      2     /* toward zero (the add kernels of the reference)   */
+#define JF_ROUND_STOCHASTIC_TRUNC 3
+
+#define JF_GELU_ERF  0
+#define JF_GELU_TANH 1
+
+typedef void *jf_stream_t;
+
+const char *jf_error_string(int code);
+
+/* Bytes of device scratch the GEMM entry points need for this problem (0 for JF_B_NK; for
+ * JF_B_KN the B operand is re-laid-out K-contiguous first). */
+size_t jf_igemm_workspace_bytes(int M, int N, int K, int b_layout);
+
+/* C_s32[M,N] = A[M,K] * B.   Replaces igemm_basic_int8_gemm (include/igemm.h:3-12,
+ * igemm/igemm_BasicInt8Gemm.cu:113-140). */
+int jf_igemm_s32(const int8_t *A, const int8_t *B, int32_t *C, int M, int N, int K, int b_layout,
+                 void *workspace, size_t workspace_bytes, jf_stream_t stream);
+
+/* acc[kb][M][N] (int32) = A[:, 32kb:32kb+32] * B[32kb:32kb+32, :] for every K block: the per-block
+ * INT32 accumulators (frag_intc at …BiasRowCol.cu:209-211) made observable for parity tests. */
+int jf_igemm_block_acc(const int8_t *A, const int8_t *B, int32_t *acc, int M, int N, int K, int b_layout,
+                       void *workspace, size_t workspace_bytes, jf_stream_t stream);
+
+/* C_fp[M,N] = sum_kb sa*sb*(A_kb*B_kb), fp32 accumulate in ascending kb, stored as out_dtype.
+ * Replaces igemm_output_fp_no_quantize (include/igemm.h:14-25, igemm/igemm_BlockSquare32OutputFp.cu:340-382). */
+int jf_igemm_block_fp(const int8_t *A, const int8_t *B, const void *sa, const void *sb, void *C,
+                      int M, int N, int K, int b_layout, int scale_dtype, int out_dtype,
+                      void *workspace, size_t workspace_bytes, jf_stream_t stream);
+
+/* (C_s8[M,N], sc[M/32,N/32]) = per-32x32-block requantisation of the same accumulation.
+ *   rounding JF_ROUND_NEAREST : q = clamp(rn(127*(acc+bias[n]) / (amax+biasmax)), +-127)
+ *       replaces igemm_output_int_quantize_bias_rowcol / _rowrow / igemm_output_int_quantize
+ *       (include/igemm.h:40-51,53-77; igemm/…BiasRowCol.cu:386-434; …IntQuantize.cu)
+ *   rounding JF_ROUND_STOCHASTIC : q = clamp(rn(127*acc/amax + noise), +-127)
+ *       replaces igemm_output_int_quantize_stochastic (include/igemm.h:79-90; …Stochastic.cu:372-419)
+ * bias ([N] fp32) and biasmax ([1] fp32, device) may be NULL (= zeros). */
+int jf_igemm_block_q(const int8_t *A, const int8_t *B, const void *sa, const void *sb,
+                     const float *bias, const float *biasmax, int8_t *C, void *sc,
+                     int M, int N, int K, int b_layout, int scale_dtype, int rounding,
+                     uint64_t seed, uint64_t offset,
+                     void *workspace, size_t workspace_bytes, jf_stream_t stream);
+
+/* Block quantise x[R,C] (x_dtype: JF_FP_*) -> (q, s); optionally also qT[C,R] = q transposed.
+ * Replaces int8_quantize (Jetfire/Nonlinear/quantize.py:128-164) and, with qT != NULL,
+ * int8_quantize_transpose (Jetfire/Nonlinear/quantize_transpose.py:131-171). */
+int jf_quantize(const void *x, int x_dtype, int R, int C, int8_t *q, void *s, int8_t *qT,
+                int scale_dtype, int rounding, uint64_t seed, uint64_t offset, float amax_eps,
+                jf_stream_t stream);
+
+/* out_f32[R,C] = q*s.  Replaces int8_dequantize (Jetfire/Nonlinear/dequantize.py:86-116). */
+int jf_dequantize(const int8_t *q, const void *s, int R, int C, int scale_dtype, float *out,
+                  jf_stream_t stream);
+
+/* out[C,R] = in[R,C].  Replaces int8_transpose (Jetfire/Nonlinear/transpose.py:69-97). */
+int jf_transpose_s8(const int8_t *in, int R, int C, int8_t *out, jf_stream_t stream);
+
+/* Per-row mean and 1/sqrt(var+eps) of a block tensor (the statistics LayerNorm takes as inputs;
+ * the reference gets them from add_mean_var.py:219-221 or qmodel.py:429-430). */
+int jf_rowstats(const int8_t *q, const void *s, int R, int C, int scale_dtype, float eps,
+                float *mean, float *rstd, jf_stream_t stream);
+
+/* dequant -> (x-mean)*rstd*gamma + beta -> requant.  beta may be NULL.
+ * Replaces int8_layernorm_forward (Jetfire/Nonlinear/layernorm.py:430-465). */
+int jf_layernorm_fwd(const int8_t *q, const void *s, const float *gamma, const float *beta,
+                     const float *mean, const float *rstd, int R, int C, int scale_dtype,
+                     int8_t *qy, void *sy, jf_stream_t stream);
+
+/* Bytes of scratch for jf_layernorm_bwd. */
+size_t jf_layernorm_bwd_workspace_bytes(int R, int C);
+
+/* LayerNorm backward over full rows: (qdx, sdx) requantised dx, dgamma[C], dbeta[C] (either may be NULL).
+ * Replaces int8_layernorm_backward (Jetfire/Nonlinear/layernorm.py:467-526). */
+int jf_layernorm_bwd(const int8_t *qx, const void *sx, const int8_t *qg, const void *sg,
+                     const float *gamma, const float *mean, const float *rstd, int R, int C,
+                     int scale_dtype, int rounding, uint64_t seed, uint64_t offset,
+                     int8_t *qdx, void *sdx, float *dgamma, float *dbeta,
+                     void *workspace, size_t workspace_bytes, jf_stream_t stream);
+
+/* dequant -> GELU -> requant (amax_eps is added to the block amax: 5e-5 in the reference).
+ * Replaces int8_gelu_forward (Jetfire/Nonlinear/gelu_fwd.py:128-162). */
+int jf_gelu_fwd(const int8_t *q, const void *s, int R, int C, int scale_dtype, int approx,
+                float amax_eps, int8_t *qy, void *sy, jf_stream_t stream);
+
+/* dequant(x), dequant(g) -> gelu'(x)*g -> requant.
+ * Replaces int8_gelu_backward (Jetfire/Nonlinear/gelu_bwd.py:173-215). */
+int jf_gelu_bwd(const int8_t *qx, const void *sx, const int8_t *qg, const void *sg, int R, int C,
+                int scale_dtype, int approx, int rounding, uint64_t seed, uint64_t offset,
+                int8_t *qy, void *sy, jf_stream_t stream);
+
+/* y1_f32 = x1 + q2*s2, (q, s) = block quantisation of y1; optional per-row, per-32-column partial
+ * sums of y1 and y1^2 (rowsum, rowsq: [R, C/32] fp32, may be NULL).
+ * Replaces int8_add_Ifp_Ig16_Ofp_Og (Jetfire/Nonlinear/add.py:164-211) and
+ * int8_add_Ifp_Ig16_Ofp_Og_MeanVar (Jetfire/Nonlinear/add_mean_var.py:179-230). */
+int jf_add(const void *x1, int x1_dtype, const int8_t *q2, const void *s2, int R, int C,
+           int scale_dtype, int rounding, uint64_t seed, uint64_t offset,
+           float *y1, int8_t *q, void *s, float *rowsum, float *rowsq, jf_stream_t stream);
+
+#ifdef __cplusplus
+}
+#endif
+#endif /* JETFIRE_HIP_H */

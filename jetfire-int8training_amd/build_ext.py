@@ -1,0 +1,79 @@
+"""Builds the native parts in-tree (no JIT cache, so the artefacts travel with the source tree):
+
+  libjetfire_hip.so        hipcc, gfx950 only: the HIP kernels behind the C ABI of include/jetfire_hip.h
+  BlockQuantizeCUDA*.so    host C++ (g++): the PyTorch extension with the reference's module name and
+                           function signatures (JetfireGEMMKernel/setup.py:13, bindings.cpp:6-35); it is
+                           compiled as plain C++ (no device code, nothing for hipify to rewrite) and
+                           calls the HIP side only through the C ABI.
+
+Usage:  python build_ext.py [hip] [torch]      (default: both)
+"""
+import os
+import subprocess
+import sys
+import sysconfig
+
+HERE = os.path.dirname(os.path.abspath(__file__))
+CSRC = os.path.join(HERE, "csrc")
+HIP_LIB = os.path.join(HERE, "libjetfire_hip.so")
+ROCM = os.environ.get("ROCM_PATH", "/opt/rocm")
+
+HIP_SOURCES = ["jf_gemm.hip", "jf_blockops.hip"]
+HIP_FLAGS = [
+    "--offload-arch=gfx950", "-O3", "-std=c++17", "-fPIC", "-shared",
+    "-ffp-contract=off",                                         # roundings are exactly the ones written
+    "-Xclang", "-target-feature", "-Xclang", "-packed-fp32-ops",  # no packed-fp32 VALU forms
+    "-Wall", "-Wno-unused-function",
+]
+
+
+def torch_ext_path():
+    suffix = sysconfig.get_config_var("EXT_SUFFIX") or ".so"
+    return os.path.join(HERE, "BlockQuantizeCUDA" + suffix)
+
+
+def _run(cmd):
+    print("+", " ".join(cmd), flush=True)
+    subprocess.check_call(cmd)
+
+
+def build_hip():
+    srcs = [os.path.join(CSRC, s) for s in HIP_SOURCES]
+    _run([os.path.join(ROCM, "bin", "hipcc")] + HIP_FLAGS + ["-o", HIP_LIB] + srcs)
+    return HIP_LIB
+
+
+def build_torch():
+    import torch
+    from torch.utils import cpp_extension as ce
+
+    out = torch_ext_path()
+    inc = []
+    for p in ce.include_paths():
+        inc += ["-isystem", p]
+    inc += ["-isystem", os.path.join(ROCM, "include"), "-I", sysconfig.get_paths()["include"]]
+    torch_lib = os.path.join(os.path.dirname(torch.__file__), "lib")
+    cmd = [
+        "g++", "-O2", "-std=c++17", "-fPIC", "-shared", "-Wall", "-Wno-unused-variable",
+        "-D__HIP_PLATFORM_AMD__=1", "-DUSE_ROCM=1", "-DTORCH_EXTENSION_NAME=BlockQuantizeCUDA",
+        "-DTORCH_API_INCLUDE_EXTENSION_H", f"-D_GLIBCXX_USE_CXX11_ABI={int(torch._C._GLIBCXX_USE_CXX11_ABI)}",
+    ] + inc + [
+        os.path.join(CSRC, "bqc_ext.cpp"), "-o", out,
+        "-L" + torch_lib, "-L" + HERE, "-L" + os.path.join(ROCM, "lib"),
+        "-ltorch", "-ltorch_cpu", "-lc10", "-ltorch_hip", "-lc10_hip", "-ltorch_python", "-ljetfire_hip", "-lamdhip64",
+        "-Wl,-rpath,$ORIGIN", "-Wl,-rpath," + torch_lib, "-Wl,-rpath," + os.path.join(ROCM, "lib"),
+    ]
+    _run(cmd)
+    return out
+
+
+def main(argv):
+    what = argv or ["hip", "torch"]
+    if "hip" in what:
+        build_hip()
+    if "torch" in what:
+        build_torch()
+
+
+if __name__ == "__main__":
+    main(sys.argv[1:])

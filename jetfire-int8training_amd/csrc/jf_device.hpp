@@ -1,0 +1,247 @@
+// Device-side building blocks shared by the gfx950 kernels: wave reductions, Philox noise,
+// the exact block-constant division, packing of INT8 codes, and the elementary functions.
+//
+// Everything that feeds an INT8 code is written with IEEE +,*,/ and explicit fmaf only
+// (the translation unit is compiled with -ffp-contract=off), so a host evaluation of the same
+// sequence gives the same bits.
+#pragma once
+
+#include <hip/hip_runtime.h>
+#include <stdint.h>
+
+#include "../../include/jetfire_hip.h"
+
+namespace jf {
+
+constexpr int QB = 32;        // quantisation block edge
+constexpr int WAVE = 64;
+
+typedef int v4i __attribute__((ext_vector_type(4)));
+typedef int v16i __attribute__((ext_vector_type(16)));
+typedef float v4f __attribute__((ext_vector_type(4)));
+typedef _Float16 half_t;
+
+// ---------------------------------------------------------------------------------------------
+// scale element access: binary16 or binary32 behind one template parameter
+template <typename ST> __device__ __forceinline__ float load_scale(const ST *p, int i) { return (float)p[i]; }
+template <typename ST> __device__ __forceinline__ void store_scale(ST *p, int i, float v) { p[i] = (ST)v; }
+
+// ---------------------------------------------------------------------------------------------
+// 64-lane max reduction; every lane returns the maximum.
+__device__ __forceinline__ float wave_max(float v)
+{
+#pragma unroll
+    for (int m = 32; m >= 1; m >>= 1) v = fmaxf(v, __shfl_xor(v, m, WAVE));
+    return v;
+}
+
+// ---------------------------------------------------------------------------------------------
+// Philox4x32-10.  (Salmon et al., SC'11.)
+__device__ __forceinline__ void philox4x32_10(uint32_t c0, uint32_t c1, uint32_t c2, uint32_t c3,
+                                              uint32_t k0, uint32_t k1, uint32_t out[4])
+{
+#pragma unroll
+    for (int r = 0; r < 10; ++r) {
+        uint64_t p0 = (uint64_t)0xD2511F53u * c0;
+        uint64_t p1 = (uint64_t)0xCD9E8D57u * c2;
+        uint32_t n0 = (uint32_t)(p1 >> 32) ^ c1 ^ k0;
+        uint32_t n1 = (uint32_t)p1;
+        uint32_t n2 = (uint32_t)(p0 >> 32) ^ c3 ^ k1;
+        uint32_t n3 = (uint32_t)p0;
+        c0 = n0; c1 = n1; c2 = n2; c3 = n3;
+        k0 += 0x9E3779B9u;
+        k1 += 0xBB67AE85u;
+    }
+    out[0] = c0; out[1] = c1; out[2] = c2; out[3] = c3;
+}
+
+// Rounding noise for the 16 consecutive output elements e0 .. e0+15 (e0 a multiple of 16):
+// two Philox calls at counters offset + e0/8 and +1, 16 bits per element, low half first;
+// noise = (h + 0.5) * 2^-16 - 0.5 in (-0.5, 0.5).
+__device__ __forceinline__ void sr_noise16(uint64_t seed, uint64_t offset, uint64_t e0, float n[16])
+{
+    uint64_t c = offset + (e0 >> 3);
+#pragma unroll
+    for (int call = 0; call < 2; ++call) {
+        uint32_t o[4];
+        uint64_t cc = c + (uint64_t)call;
+        philox4x32_10((uint32_t)cc, (uint32_t)(cc >> 32), 0u, 0u, (uint32_t)seed, (uint32_t)(seed >> 32), o);
+#pragma unroll
+        for (int w = 0; w < 4; ++w) {
+            n[call * 8 + 2 * w]     = ((float)(o[w] & 0xFFFFu) + 0.5f) * 1.52587890625e-05f - 0.5f;
+            n[call * 8 + 2 * w + 1] = ((float)(o[w] >> 16) + 0.5f) * 1.52587890625e-05f - 0.5f;
+        }
+    }
+}
+
+// ---------------------------------------------------------------------------------------------
+// x / s for a divisor shared by many elements.  With r = 1/s (IEEE), q0 = x*r, e = x - q0*s (exact
+// in one fma), q0 + e*r is the correctly rounded quotient as long as nothing under/overflows; the
+// caller takes this path only for s in [2^-60, 2^60] and falls back to the IEEE division otherwise.
+struct BlockDivisor {
+    float s, r;
+    bool fast;
+    __device__ __forceinline__ explicit BlockDivisor(float s_) : s(s_)
+    {
+        fast = (s_ > 8.67361738e-19f) && (s_ < 1.15292150e+18f);
+        r = 1.0f / s_;
+    }
+    __device__ __forceinline__ float div(float x) const
+    {
+        if (fast) {
+            float q0 = x * r;
+            float e = __builtin_fmaf(-q0, s, x);
+            return __builtin_fmaf(e, r, q0);
+        }
+        return x / s;
+    }
+};
+
+__device__ __forceinline__ int clamp127(float y_rounded)
+{
+    float c = fminf(fmaxf(y_rounded, -127.0f), 127.0f);
+    return (int)c;
+}
+
+__device__ __forceinline__ uint32_t pack4(int a, int b, int c, int d)
+{
+    return (uint32_t)(a & 0xFF) | ((uint32_t)(b & 0xFF) << 8) | ((uint32_t)(c & 0xFF) << 16) | ((uint32_t)d << 24);
+}
+
+// ---------------------------------------------------------------------------------------------
+// Block quantisation of 16 values per lane, one wave = one 32x32 block (lane l: row l/2,
+// columns 16*(l%2) .. +15).  Returns the packed codes; *scale_out = amax/127 (all lanes).
+//   y = v / s;  nearest: rn(y);  stochastic: rn(copysign(min(|y|+noise, 127), y));
+//   trunc variants: trunc instead of rn.  All-zero block: s = 0, codes = 0.
+__device__ __forceinline__ v4i quantize16(const float v[16], float amax_eps, int rounding,
+                                          uint64_t seed, uint64_t offset, uint64_t e0, float *scale_out)
+{
+    float m = 0.0f;
+#pragma unroll
+    for (int i = 0; i < 16; ++i) m = fmaxf(m, fabsf(v[i]));
+    float amax = wave_max(m) + amax_eps;
+    v4i out = {0, 0, 0, 0};
+    if (!(amax > 0.0f)) { *scale_out = 0.0f; return out; }
+    float s = amax / 127.0f;
+    *scale_out = s;
+    BlockDivisor d(s);
+    float y[16];
+#pragma unroll
+    for (int i = 0; i < 16; ++i) y[i] = d.div(v[i]);
+    if (rounding == JF_ROUND_STOCHASTIC || rounding == JF_ROUND_STOCHASTIC_TRUNC) {
+        float n[16];
+        sr_noise16(seed, offset, e0, n);
+#pragma unroll
+        for (int i = 0; i < 16; ++i) {
+            float a = fminf(fabsf(y[i]) + n[i], 127.0f);
+            y[i] = __builtin_copysignf(a, y[i]);
+        }
+    }
+    int c[16];
+    if (rounding == JF_ROUND_TRUNC || rounding == JF_ROUND_STOCHASTIC_TRUNC) {
+#pragma unroll
+        for (int i = 0; i < 16; ++i) c[i] = clamp127(__builtin_truncf(y[i]));
+    } else {
+#pragma unroll
+        for (int i = 0; i < 16; ++i) c[i] = clamp127(__builtin_rintf(y[i]));
+    }
+    out.x = (int)pack4(c[0], c[1], c[2], c[3]);
+    out.y = (int)pack4(c[4], c[5], c[6], c[7]);
+    out.z = (int)pack4(c[8], c[9], c[10], c[11]);
+    out.w = (int)pack4(c[12], c[13], c[14], c[15]);
+    return out;
+}
+
+__device__ __forceinline__ void unpack16(v4i p, float scale, float x[16])
+{
+    const int w[4] = {p.x, p.y, p.z, p.w};
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+        x[4 * i + 0] = (float)((w[i] << 24) >> 24) * scale;
+        x[4 * i + 1] = (float)((w[i] << 16) >> 24) * scale;
+        x[4 * i + 2] = (float)((w[i] << 8) >> 24) * scale;
+        x[4 * i + 3] = (float)(w[i] >> 24) * scale;
+    }
+}
+
+// ---------------------------------------------------------------------------------------------
+// Elementary functions (same sequences as the host checker uses).
+__device__ __forceinline__ float expf_det(float x)
+{
+    if (x < -87.0f) return 0.0f;
+    x = fminf(x, 88.0f);
+    float n = __builtin_rintf(x * 1.44269504f);
+    float r = __builtin_fmaf(n, -0.693145752f, x);
+    r = __builtin_fmaf(n, -1.42860677e-06f, r);
+    float p = 1.98412698e-04f;
+    p = __builtin_fmaf(p, r, 1.38888889e-03f);
+    p = __builtin_fmaf(p, r, 8.33333333e-03f);
+    p = __builtin_fmaf(p, r, 4.16666667e-02f);
+    p = __builtin_fmaf(p, r, 1.66666667e-01f);
+    p = __builtin_fmaf(p, r, 0.5f);
+    p = __builtin_fmaf(p, r, 1.0f);
+    p = __builtin_fmaf(p, r, 1.0f);
+    return __int_as_float(__float_as_int(p) + (((int)n) << 23));
+}
+
+// erfc(z), z >= 0: t*exp(-z^2 + P(t)), t = 1/(1+z/2) (Chebyshev fit of Numerical Recipes' erfcc).
+__device__ __forceinline__ float erfc_pos(float z)
+{
+    float t = 1.0f / __builtin_fmaf(0.5f, z, 1.0f);
+    float p = 0.17087277f;
+    p = __builtin_fmaf(p, t, -0.82215223f);
+    p = __builtin_fmaf(p, t, 1.48851587f);
+    p = __builtin_fmaf(p, t, -1.13520398f);
+    p = __builtin_fmaf(p, t, 0.27886807f);
+    p = __builtin_fmaf(p, t, -0.18628806f);
+    p = __builtin_fmaf(p, t, 0.09678418f);
+    p = __builtin_fmaf(p, t, 0.37409196f);
+    p = __builtin_fmaf(p, t, 1.00002368f);
+    p = __builtin_fmaf(p, t, -1.26551223f);
+    float e = __builtin_fmaf(-z, z, p);
+    return t * expf_det(e);
+}
+
+__device__ __forceinline__ float norm_cdf(float x)
+{
+    float z = fabsf(x) * 0.707106781f;
+    float h = 0.5f * erfc_pos(z);
+    return x > 0.0f ? 1.0f - h : h;
+}
+
+__device__ __forceinline__ float tanhf_det(float u)
+{
+    float a = fminf(fabsf(u), 15.0f);
+    float e = expf_det(a + a);
+    float t = 1.0f - 2.0f / (e + 1.0f);
+    return __builtin_copysignf(t, u);
+}
+
+template <int APPROX> __device__ __forceinline__ float gelu(float x)
+{
+    if (APPROX == JF_GELU_ERF) return x * norm_cdf(x);
+    float x2 = x * x;
+    float inner = 0.797884561f * (x * __builtin_fmaf(0.044715f, x2, 1.0f));
+    return (0.5f * x) * (1.0f + tanhf_det(inner));
+}
+
+template <int APPROX> __device__ __forceinline__ float dgelu(float x)
+{
+    if (APPROX == JF_GELU_ERF) {
+        float pdf = 0.398942280f * expf_det(-0.5f * (x * x));
+        return __builtin_fmaf(x, pdf, norm_cdf(x));
+    }
+    float x2 = x * x;
+    float inner = 0.797884561f * (x * __builtin_fmaf(0.044715f, x2, 1.0f));
+    float t = tanhf_det(inner);
+    float dinner = 0.797884561f * __builtin_fmaf(0.134145f, x2, 1.0f);
+    float sech2 = __builtin_fmaf(-t, t, 1.0f);
+    return __builtin_fmaf((0.5f * x) * sech2, dinner, 0.5f * (1.0f + t));
+}
+
+// ---------------------------------------------------------------------------------------------
+// host-side argument checks shared by the entry points
+static inline bool mult32(int v) { return v > 0 && (v % QB) == 0; }
+static inline bool aligned16(const void *p) { return (reinterpret_cast<uintptr_t>(p) & 15u) == 0; }
+
+}  // namespace jf

@@ -1,0 +1,340 @@
+"""Host-side binding of libjetfire_hip.so (ctypes over the C ABI of include/jetfire_hip.h) for torch
+tensors.  PyTorch is used for device memory and the current stream only; every computation below is a
+hand-written gfx950 kernel.  There is no fallback: a missing library or a CPU tensor raises.
+
+Each wrapper allocates its outputs (like the reference's launchers do with torch.empty, e.g.
+JetfireGEMMKernel/BlockQuantize/cpp_extension/igemm/igemm_BlockSquare32OutputIntQuantizeBiasRowCol.cu:404-408,
+Jetfire/Nonlinear/quantize.py:140-141) and takes/returns 2-D tensors; 3-D handling lives in the
+Linear / Nonlinear packages.
+"""
+import ctypes as C
+import os
+
+import torch
+
+_HERE = os.path.dirname(os.path.abspath(__file__))
+LIB_PATH = os.path.join(_HERE, "libjetfire_hip.so")
+QB = 32
+
+B_NK, B_KN = 0, 1
+SCALE_F16, SCALE_F32 = 0, 1
+FP_F16, FP_F32, FP_BF16 = 0, 1, 2
+ROUND_NEAREST, ROUND_STOCHASTIC, ROUND_TRUNC, ROUND_STOCHASTIC_TRUNC = 0, 1, 2, 3
+GELU_ERF, GELU_TANH = 0, 1
+
+EXPORTS = [
+    "jf_error_string", "jf_igemm_workspace_bytes", "jf_igemm_s32", "jf_igemm_block_acc", "jf_igemm_block_fp",
+    "jf_igemm_block_q", "jf_quantize", "jf_dequantize", "jf_transpose_s8", "jf_rowstats", "jf_layernorm_fwd",
+    "jf_layernorm_bwd_workspace_bytes", "jf_layernorm_bwd", "jf_gelu_fwd", "jf_gelu_bwd", "jf_add",
+]
+
+_lib = None
+_p, _i, _u64, _f, _sz = C.c_void_p, C.c_int, C.c_uint64, C.c_float, C.c_size_t
+
+
+def lib():
+    """The loaded library; raises if it has not been built."""
+    global _lib
+    if _lib is None:
+        if not os.path.exists(LIB_PATH):
+            raise RuntimeError(f"{LIB_PATH} is missing: build it with `python {os.path.join(_HERE, 'build_ext.py')} hip`")
+        L = C.CDLL(LIB_PATH)
+        L.jf_error_string.argtypes = [_i]
+        L.jf_error_string.restype = C.c_char_p
+        L.jf_igemm_workspace_bytes.argtypes = [_i, _i, _i, _i]
+        L.jf_igemm_workspace_bytes.restype = _sz
+        L.jf_igemm_s32.argtypes = [_p, _p, _p, _i, _i, _i, _i, _p, _sz, _p]
+        L.jf_igemm_block_acc.argtypes = [_p, _p, _p, _i, _i, _i, _i, _p, _sz, _p]
+        L.jf_igemm_block_fp.argtypes = [_p, _p, _p, _p, _p, _i, _i, _i, _i, _i, _i, _p, _sz, _p]
+        L.jf_igemm_block_q.argtypes = [_p, _p, _p, _p, _p, _p, _p, _p, _i, _i, _i, _i, _i, _i, _u64, _u64, _p, _sz, _p]
+        L.jf_quantize.argtypes = [_p, _i, _i, _i, _p, _p, _p, _i, _i, _u64, _u64, _f, _p]
+        L.jf_dequantize.argtypes = [_p, _p, _i, _i, _i, _p, _p]
+        L.jf_transpose_s8.argtypes = [_p, _i, _i, _p, _p]
+        L.jf_rowstats.argtypes = [_p, _p, _i, _i, _i, _f, _p, _p, _p]
+        L.jf_layernorm_fwd.argtypes = [_p, _p, _p, _p, _p, _p, _i, _i, _i, _p, _p, _p]
+        L.jf_layernorm_bwd_workspace_bytes.argtypes = [_i, _i]
+        L.jf_layernorm_bwd_workspace_bytes.restype = _sz
+        L.jf_layernorm_bwd.argtypes = [_p, _p, _p, _p, _p, _p, _p, _i, _i, _i, _i, _u64, _u64, _p, _p, _p, _p, _p, _sz, _p]
+        L.jf_gelu_fwd.argtypes = [_p, _p, _i, _i, _i, _i, _f, _p, _p, _p]
+        L.jf_gelu_bwd.argtypes = [_p, _p, _p, _p, _i, _i, _i, _i, _i, _u64, _u64, _p, _p, _p]
+        L.jf_add.argtypes = [_p, _i, _p, _p, _i, _i, _i, _i, _u64, _u64, _p, _p, _p, _p, _p, _p]
+        missing = [name for name in EXPORTS if not hasattr(L, name)]
+        if missing:
+            raise RuntimeError(f"{LIB_PATH} does not export {missing}")
+        _lib = L
+    return _lib
+
+
+def check(rc):
+    if rc != 0:
+        raise RuntimeError(lib().jf_error_string(rc).decode())
+
+
+def _ptr(t):
+    return None if t is None else C.c_void_p(t.data_ptr())
+
+
+def _stream():
+    return C.c_void_p(torch.cuda.current_stream().cuda_stream)
+
+
+def _need(t, dtype, name, ndim=2):
+    if not isinstance(t, torch.Tensor) or not t.is_cuda:
+        raise RuntimeError(f"{name}: expected a GPU tensor")
+    if dtype is not None and t.dtype != dtype:
+        raise RuntimeError(f"{name}: expected dtype {dtype}, got {t.dtype}")
+    if ndim is not None and t.dim() != ndim:
+        raise RuntimeError(f"{name}: expected {ndim} dimensions, got {t.dim()}")
+    if not t.is_contiguous():
+        raise RuntimeError(f"{name}: expected a contiguous tensor")
+    return t
+
+
+def _scale_code(s, name):
+    if s.dtype == torch.float16:
+        return SCALE_F16
+    if s.dtype == torch.float32:
+        return SCALE_F32
+    raise RuntimeError(f"{name}: scales must be float16 or float32, got {s.dtype}")
+
+
+_SCALE_TORCH = {SCALE_F16: torch.float16, SCALE_F32: torch.float32}
+_FP_CODE = {torch.float16: FP_F16, torch.float32: FP_F32, torch.bfloat16: FP_BF16}
+
+
+def _mult32(*dims):
+    for d in dims:
+        if d <= 0 or d % QB:
+            raise RuntimeError(f"dimension {d} is not a positive multiple of {QB}")
+
+
+# ------------------------------------------------------------------------------------------------ RNG
+class _Philox:
+    """(seed, offset) for the stochastic-rounding kernels.  The seed follows torch.manual_seed; the
+    offset advances by the number of Philox calls an op may consume, so a program is reproducible."""
+
+    def __init__(self):
+        self.seed = None
+        self.offset = 0
+
+    def next(self, numel):
+        s = torch.initial_seed() & 0xFFFFFFFFFFFFFFFF
+        if s != self.seed:
+            self.seed, self.offset = s, 0
+        off = self.offset
+        self.offset += (numel + 7) // 8
+        return self.seed, off
+
+
+philox = _Philox()
+
+
+def _rng(rounding, numel, seed, offset):
+    if rounding in (ROUND_STOCHASTIC, ROUND_STOCHASTIC_TRUNC) and seed is None:
+        return philox.next(numel)
+    return (seed or 0), (offset or 0)
+
+
+# ------------------------------------------------------------------------------------------------ GEMMs
+def _gemm_operands(A, B, b_layout):
+    _need(A, torch.int8, "A")
+    _need(B, torch.int8, "B")
+    M, K = A.shape
+    if b_layout == B_NK:
+        N, K2 = B.shape
+    elif b_layout == B_KN:
+        K2, N = B.shape
+    else:
+        raise RuntimeError("b_layout must be B_NK or B_KN")
+    if K2 != K:
+        raise RuntimeError(f"inner dimensions differ: A is {tuple(A.shape)}, B is {tuple(B.shape)}")
+    if B.device != A.device:
+        raise RuntimeError("A and B are on different devices")
+    _mult32(M, N, K)
+    nbytes = lib().jf_igemm_workspace_bytes(M, N, K, b_layout)
+    ws = torch.empty(nbytes, dtype=torch.int8, device=A.device) if nbytes else None
+    return M, N, K, ws, nbytes
+
+
+def _gemm_scales(sa, sb, M, N, K):
+    code = _scale_code(sa, "sa")
+    _need(sa, None, "sa")
+    _need(sb, sa.dtype, "sb")
+    if tuple(sa.shape) != (K // QB, M // QB) or tuple(sb.shape) != (K // QB, N // QB):
+        raise RuntimeError(f"scale shapes must be [K/32,M/32]={K // QB, M // QB} and [K/32,N/32]={K // QB, N // QB}, "
+                           f"got {tuple(sa.shape)} and {tuple(sb.shape)}")
+    return code
+
+
+def igemm_s32(A, B, b_layout=B_KN):
+    M, N, K, ws, nb = _gemm_operands(A, B, b_layout)
+    out = torch.empty((M, N), dtype=torch.int32, device=A.device)
+    check(lib().jf_igemm_s32(_ptr(A), _ptr(B), _ptr(out), M, N, K, b_layout, _ptr(ws), nb, _stream()))
+    return out
+
+
+def igemm_block_acc(A, B, b_layout=B_KN):
+    M, N, K, ws, nb = _gemm_operands(A, B, b_layout)
+    out = torch.empty((K // QB, M, N), dtype=torch.int32, device=A.device)
+    check(lib().jf_igemm_block_acc(_ptr(A), _ptr(B), _ptr(out), M, N, K, b_layout, _ptr(ws), nb, _stream()))
+    return out
+
+
+def igemm_block_fp(A, B, sa, sb, b_layout=B_KN, out_dtype=torch.float16):
+    M, N, K, ws, nb = _gemm_operands(A, B, b_layout)
+    code = _gemm_scales(sa, sb, M, N, K)
+    out = torch.empty((M, N), dtype=out_dtype, device=A.device)
+    check(lib().jf_igemm_block_fp(_ptr(A), _ptr(B), _ptr(sa), _ptr(sb), _ptr(out), M, N, K, b_layout, code,
+                                  _FP_CODE[out_dtype], _ptr(ws), nb, _stream()))
+    return out
+
+
+def igemm_block_q(A, B, sa, sb, b_layout=B_KN, bias=None, biasmax=None, rounding=ROUND_NEAREST, seed=None, offset=None):
+    M, N, K, ws, nb = _gemm_operands(A, B, b_layout)
+    code = _gemm_scales(sa, sb, M, N, K)
+    if bias is not None:
+        _need(bias, torch.float32, "bias", 1)
+        if bias.numel() != N:
+            raise RuntimeError("bias must have N elements")
+    if biasmax is not None:
+        _need(biasmax, torch.float32, "biasmax", None)
+    if rounding not in (ROUND_NEAREST, ROUND_STOCHASTIC):
+        raise RuntimeError("rounding must be ROUND_NEAREST or ROUND_STOCHASTIC")
+    seed, offset = _rng(rounding, M * N, seed, offset)
+    out = torch.empty((M, N), dtype=torch.int8, device=A.device)
+    sc = torch.empty((M // QB, N // QB), dtype=sa.dtype, device=A.device)
+    check(lib().jf_igemm_block_q(_ptr(A), _ptr(B), _ptr(sa), _ptr(sb), _ptr(bias), _ptr(biasmax), _ptr(out), _ptr(sc),
+                                 M, N, K, b_layout, code, rounding, seed, offset, _ptr(ws), nb, _stream()))
+    return out, sc
+
+
+# ------------------------------------------------------------------------------------------------ block ops
+def quantize(x, rounding=ROUND_NEAREST, scale_dtype=torch.float16, transpose=False, amax_eps=0.0, seed=None, offset=None):
+    _need(x, None, "x")
+    if x.dtype not in _FP_CODE:
+        raise RuntimeError(f"x: unsupported dtype {x.dtype}")
+    R, Cc = x.shape
+    _mult32(R, Cc)
+    seed, offset = _rng(rounding, R * Cc, seed, offset)
+    q = torch.empty((R, Cc), dtype=torch.int8, device=x.device)
+    s = torch.empty((R // QB, Cc // QB), dtype=scale_dtype, device=x.device)
+    qT = torch.empty((Cc, R), dtype=torch.int8, device=x.device) if transpose else None
+    check(lib().jf_quantize(_ptr(x), _FP_CODE[x.dtype], R, Cc, _ptr(q), _ptr(s), _ptr(qT), _scale_code(s, "s"),
+                            rounding, seed, offset, amax_eps, _stream()))
+    return (q, s, qT) if transpose else (q, s)
+
+
+def _block_tensor(q, s, name):
+    _need(q, torch.int8, name)
+    _need(s, None, name + " scale")
+    R, Cc = q.shape
+    _mult32(R, Cc)
+    if tuple(s.shape) != (R // QB, Cc // QB):
+        raise RuntimeError(f"{name}: scale shape {tuple(s.shape)} does not match codes {tuple(q.shape)}")
+    if s.device != q.device:
+        raise RuntimeError(f"{name}: codes and scales are on different devices")
+    return R, Cc, _scale_code(s, name)
+
+
+def dequantize(q, s):
+    R, Cc, code = _block_tensor(q, s, "x")
+    out = torch.empty((R, Cc), dtype=torch.float32, device=q.device)
+    check(lib().jf_dequantize(_ptr(q), _ptr(s), R, Cc, code, _ptr(out), _stream()))
+    return out
+
+
+def transpose_s8(q):
+    _need(q, torch.int8, "x")
+    R, Cc = q.shape
+    if R % 16 or Cc % 16:
+        raise RuntimeError("transpose: dimensions must be multiples of 16")
+    out = torch.empty((Cc, R), dtype=torch.int8, device=q.device)
+    check(lib().jf_transpose_s8(_ptr(q), R, Cc, _ptr(out), _stream()))
+    return out
+
+
+def rowstats(q, s, eps=1e-5):
+    R, Cc, code = _block_tensor(q, s, "x")
+    mean = torch.empty(R, dtype=torch.float32, device=q.device)
+    rstd = torch.empty(R, dtype=torch.float32, device=q.device)
+    check(lib().jf_rowstats(_ptr(q), _ptr(s), R, Cc, code, eps, _ptr(mean), _ptr(rstd), _stream()))
+    return mean, rstd
+
+
+def _vec(t, n, name):
+    _need(t, torch.float32, name, 1)
+    if t.numel() != n:
+        raise RuntimeError(f"{name}: expected {n} elements, got {t.numel()}")
+    return t
+
+
+def layernorm_fwd(q, s, gamma, beta, mean, rstd):
+    R, Cc, code = _block_tensor(q, s, "x")
+    _vec(gamma, Cc, "gamma")
+    if beta is not None:
+        _vec(beta, Cc, "beta")
+    _vec(mean, R, "mean")
+    _vec(rstd, R, "rstd")
+    qy = torch.empty_like(q)
+    sy = torch.empty_like(s)
+    check(lib().jf_layernorm_fwd(_ptr(q), _ptr(s), _ptr(gamma), _ptr(beta), _ptr(mean), _ptr(rstd), R, Cc, code,
+                                 _ptr(qy), _ptr(sy), _stream()))
+    return qy, sy
+
+
+def layernorm_bwd(qx, sx, qg, sg, gamma, mean, rstd, rounding=ROUND_NEAREST, want_dbeta=True, seed=None, offset=None):
+    R, Cc, code = _block_tensor(qx, sx, "x")
+    R2, C2, code2 = _block_tensor(qg, sg, "g")
+    if (R2, C2, code2) != (R, Cc, code):
+        raise RuntimeError("x and g must have the same shape and scale dtype")
+    _vec(gamma, Cc, "gamma")
+    _vec(mean, R, "mean")
+    _vec(rstd, R, "rstd")
+    seed, offset = _rng(rounding, R * Cc, seed, offset)
+    nbytes = lib().jf_layernorm_bwd_workspace_bytes(R, Cc)
+    ws = torch.empty(nbytes, dtype=torch.int8, device=qx.device)
+    qdx = torch.empty_like(qx)
+    sdx = torch.empty_like(sx)
+    dgamma = torch.empty(Cc, dtype=torch.float32, device=qx.device)
+    dbeta = torch.empty(Cc, dtype=torch.float32, device=qx.device) if want_dbeta else None
+    check(lib().jf_layernorm_bwd(_ptr(qx), _ptr(sx), _ptr(qg), _ptr(sg), _ptr(gamma), _ptr(mean), _ptr(rstd), R, Cc, code,
+                                 rounding, seed, offset, _ptr(qdx), _ptr(sdx), _ptr(dgamma), _ptr(dbeta), _ptr(ws), nbytes,
+                                 _stream()))
+    return qdx, sdx, dgamma, dbeta
+
+
+def gelu_fwd(q, s, approx=GELU_ERF, amax_eps=5e-5):
+    R, Cc, code = _block_tensor(q, s, "x")
+    qy = torch.empty_like(q)
+    sy = torch.empty_like(s)
+    check(lib().jf_gelu_fwd(_ptr(q), _ptr(s), R, Cc, code, approx, amax_eps, _ptr(qy), _ptr(sy), _stream()))
+    return qy, sy
+
+
+def gelu_bwd(qx, sx, qg, sg, approx=GELU_ERF, rounding=ROUND_NEAREST, seed=None, offset=None):
+    R, Cc, code = _block_tensor(qx, sx, "x")
+    R2, C2, code2 = _block_tensor(qg, sg, "g")
+    if (R2, C2, code2) != (R, Cc, code):
+        raise RuntimeError("x and g must have the same shape and scale dtype")
+    seed, offset = _rng(rounding, R * Cc, seed, offset)
+    qy = torch.empty_like(qx)
+    sy = torch.empty_like(sx)
+    check(lib().jf_gelu_bwd(_ptr(qx), _ptr(sx), _ptr(qg), _ptr(sg), R, Cc, code, approx, rounding, seed, offset,
+                            _ptr(qy), _ptr(sy), _stream()))
+    return qy, sy
+
+
+def add(x1, q2, s2, rounding=ROUND_TRUNC, with_stats=False, seed=None, offset=None):
+    R, Cc, code = _block_tensor(q2, s2, "x2")
+    _need(x1, None, "x1")
+    if x1.dtype not in _FP_CODE or tuple(x1.shape) != (R, Cc):
+        raise RuntimeError("x1 must be a float tensor of the same shape as x2")
+    seed, offset = _rng(rounding, R * Cc, seed, offset)
+    y1 = torch.empty((R, Cc), dtype=torch.float32, device=x1.device)
+    q = torch.empty_like(q2)
+    s = torch.empty_like(s2)
+    rs = torch.empty((R, Cc // QB), dtype=torch.float32, device=x1.device) if with_stats else None
+    rq = torch.empty((R, Cc // QB), dtype=torch.float32, device=x1.device) if with_stats else None
+    check(lib().jf_add(_ptr(x1), _FP_CODE[x1.dtype], _ptr(q2), _ptr(s2), R, Cc, code, rounding, seed, offset,
+                       _ptr(y1), _ptr(q), _ptr(s), _ptr(rs), _ptr(rq), _stream()))
+    return (y1, q, s, rs, rq) if with_stats else (y1, q, s)

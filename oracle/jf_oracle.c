@@ -571,7 +571,7 @@ void jfo_layernorm_bwd(const int8_t *qx, const float *sx, const int8_t *qg, cons
 /*
  * Residual add: y1 = x1 + q2*s2 (fp32 out) and its block quantisation.
  * add.py:29-162 (stochastic allowed) / add_mean_var.py:28-177 (+ per-row partial
- * sums of y1 and y1^2 per 32-column block, ascending add / fmaf chains).
+ * sums of y1 and y1^2 per 32-column block: two 16-column add / fmaf chains, added).
  * truncate=1 reproduces the reference's `.to(int8)` without llrint (add.py:139).
  */
 void jfo_add(const float *x1, const int8_t *q2, const float *s2, int R, int C,
@@ -584,15 +584,15 @@ void jfo_add(const float *x1, const int8_t *q2, const float *s2, int R, int C,
         size_t o = (size_t)rb * QB * C + (size_t)cb * QB;
         float sc = s2[rb * SC + cb];
         for (int i = 0; i < QB; ++i) {
-            float a = 0.0f, b = 0.0f;
+            float a[2] = {0.0f, 0.0f}, b[2] = {0.0f, 0.0f};   /* two 16-column chains, then added */
             for (int j = 0; j < QB; ++j) {
                 float v = x1[o + (size_t)i * C + j] + (float)q2[o + (size_t)i * C + j] * sc;
                 tmp[i * QB + j] = v;
                 y1[o + (size_t)i * C + j] = v;
-                a = a + v; b = fmaf(v, v, b);
+                a[j / 16] = a[j / 16] + v; b[j / 16] = fmaf(v, v, b[j / 16]);
             }
-            if (rowsum) rowsum[(size_t)(rb * QB + i) * SC + cb] = a;
-            if (rowsq) rowsq[(size_t)(rb * QB + i) * SC + cb] = b;
+            if (rowsum) rowsum[(size_t)(rb * QB + i) * SC + cb] = a[0] + a[1];
+            if (rowsq) rowsq[(size_t)(rb * QB + i) * SC + cb] = b[0] + b[1];
         }
         quantize_block(tmp, QB, q + o, C, &s[rb * SC + cb], stochastic, seed, offset, (uint64_t)o, (uint64_t)C, 0.0f, truncate);
     }

@@ -17,3 +17,16 @@ def oracle():
     from oracle import oracle as O
     O.lib()
     return O
+
+PKG = os.path.join(ROOT, "jetfire-int8training_amd")
+for p in (PKG, os.path.join(PKG, "Jetfire")):
+    if p not in sys.path:
+        sys.path.insert(0, p)
+
+
+@pytest.fixture(scope="session")
+def jf():
+    """ctypes binding of the HIP library; a GPU test without the built library is an error, not a skip."""
+    import jetfire_hip
+    jetfire_hip.lib()
+    return jetfire_hip

@@ -1,0 +1,42 @@
+"""The C-ABI library loads and exports every entry point include/jetfire_hip.h declares (no GPU needed)."""
+import ctypes
+import os
+import re
+
+ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+
+
+def _declared():
+    text = open(os.path.join(ROOT, "include", "jetfire_hip.h")).read()
+    text = re.sub(r"/\*.*?\*/", "", text, flags=re.S)
+    return sorted(set(re.findall(r"\b(jf_[a-z0-9_]+)\s*\(", text)))
+
+
+def test_header_symbols_are_exported():
+    names = _declared()
+    assert len(names) >= 16
+    lib = ctypes.CDLL(os.path.join(ROOT, "jetfire-int8training_amd", "libjetfire_hip.so"))
+    for n in names:
+        assert hasattr(lib, n), n
+
+
+def test_binding_lists_every_symbol(jf):
+    assert sorted(jf.EXPORTS) == _declared()
+
+
+def test_argument_errors_without_gpu(jf):
+    L = jf.lib()
+    assert L.jf_igemm_s32(None, None, None, 32, 32, 32, 0, None, 0, None) == -1
+    assert b"NULL" in L.jf_error_string(-1)
+    assert b"multiple of 32" in L.jf_error_string(-2)
+    assert L.jf_igemm_workspace_bytes(64, 96, 128, 1) == 96 * 128
+    assert L.jf_igemm_workspace_bytes(64, 96, 128, 0) == 0
+    buf = (ctypes.c_char * 4096)()
+    p = ctypes.addressof(buf)
+    p = (p + 15) & ~15
+    assert L.jf_igemm_s32(p, p, p, 48, 32, 32, 0, None, 0, None) == -2          # 48 is not a multiple of 32
+    assert L.jf_igemm_s32(p, p, p, 32, 32, 32, 7, None, 0, None) == -3          # unknown layout
+    assert L.jf_igemm_s32(p + 1, p, p, 32, 32, 32, 0, None, 0, None) == -4      # misaligned
+    assert L.jf_igemm_s32(p, p, p, 32, 32, 32, 1, None, 0, None) == -5          # [K,N] layout needs a workspace
+    assert L.jf_quantize(p, 9, 32, 32, p, p, None, 0, 0, 0, 0, 0.0, None) == -3
+    assert L.jf_gelu_fwd(p, p, 32, 32, 0, 5, 0.0, p, p, None) == -3

@@ -1,0 +1,210 @@
+"""GPU parity of the memory-bound kernels (quantise, transpose, dequantise, LayerNorm, GELU, add)
+against the CPU oracle, through the C ABI.  INT8 codes and scales: bit-exact.  fp32 outputs of
+elementwise kernels: bit-exact; reductions that end in fp outputs (dgamma, dbeta): 1e-5 relative.
+"""
+import numpy as np
+import pytest
+import torch
+
+from helpers import QB, expand_scales, rand_codes, rand_scales
+from test_gpu_gemm import dev, same
+
+pytestmark = pytest.mark.gpu
+
+SHAPES = [(32, 32), (64, 96), (96, 160), (256, 1600)]
+ROUND = {"nearest": 0, "stochastic": 1, "trunc": 2, "stochastic_trunc": 3}
+
+
+def rand_x(rng, R, C):
+    x = (rng.standard_normal((R, C)) * np.exp2(rng.integers(-6, 3, (R, C)))).astype(np.float32)
+    if R >= 64:
+        x[32:64, :32] = 0.0        # an all-zero block
+    return x
+
+
+def block_tensor(oracle, rng, R, C, scale=1.0, f16=True):
+    q, s = oracle.quantize((rng.standard_normal((R, C)) * scale).astype(np.float32), scale_dtype="f16" if f16 else "f32")
+    return q, s
+
+
+@pytest.mark.parametrize("f16", [True, False])
+@pytest.mark.parametrize("mode", ["nearest", "stochastic", "trunc", "stochastic_trunc"])
+@pytest.mark.parametrize("R,C", SHAPES)
+def test_quantize(jf, oracle, R, C, mode, f16):
+    print(f"case quantize {R}x{C} {mode} f16={f16}", flush=True)
+    rng = np.random.default_rng(R + C)
+    x = rand_x(rng, R, C)
+    sd = torch.float16 if f16 else torch.float32
+    q, s = jf.quantize(dev(x), rounding=ROUND[mode], scale_dtype=sd, seed=42, offset=17)
+    wq, ws = oracle.quantize(x, stochastic="stochastic" in mode, seed=42, offset=17, truncate="trunc" in mode,
+                             scale_dtype="f16" if f16 else "f32")
+    same(q, wq, "codes")
+    same(s, ws, "scales")
+
+
+@pytest.mark.parametrize("dtype", [torch.float16, torch.bfloat16])
+def test_quantize_half_inputs_and_transpose(jf, oracle, dtype):
+    rng = np.random.default_rng(3)
+    x = torch.from_numpy(rand_x(rng, 96, 160)).to(dtype)
+    q, s, qT = jf.quantize(x.cuda(), rounding=jf.ROUND_STOCHASTIC, transpose=True, seed=5, offset=0)
+    wq, ws = oracle.quantize(x.float().numpy(), stochastic=True, seed=5, offset=0, scale_dtype="f16")
+    same(q, wq, "codes")
+    same(s, ws, "scales")
+    same(qT, np.ascontiguousarray(wq.T), "transposed codes")
+
+
+def test_quantize_amax_eps_and_tiny_scales(jf, oracle):
+    rng = np.random.default_rng(4)
+    x = (rng.standard_normal((64, 64)) * 1e-25).astype(np.float32)     # scale below the fast-division range
+    x[:32, :32] *= 1e-10
+    q, s = jf.quantize(dev(x), scale_dtype=torch.float32)
+    wq, ws = oracle.quantize(x)
+    same(q, wq, "codes")
+    same(s, ws, "scales")
+    q, s = jf.quantize(dev(x), scale_dtype=torch.float32, amax_eps=5e-5)
+    wq, ws = oracle.quantize(x, amax_eps=5e-5)
+    same(q, wq, "codes eps")
+    same(s, ws, "scales eps")
+
+
+@pytest.mark.parametrize("R,C", [(32, 32), (96, 160), (16, 48), (1600, 8192)])
+def test_transpose(jf, R, C):
+    rng = np.random.default_rng(R)
+    q = rand_codes(rng, (R, C))
+    same(jf.transpose_s8(dev(q)), np.ascontiguousarray(q.T), "transpose")
+
+
+@pytest.mark.parametrize("f16", [True, False])
+def test_dequantize(jf, oracle, f16):
+    rng = np.random.default_rng(6)
+    q = rand_codes(rng, (96, 160))
+    s = rand_scales(rng, (3, 5), f16=f16)
+    got = jf.dequantize(dev(q), dev(s.astype(np.float16 if f16 else np.float32)))
+    same(got, oracle.dequantize(q, s), "dequantize")
+
+
+@pytest.mark.parametrize("f16", [True, False])
+@pytest.mark.parametrize("approx,eps", [(0, 5e-5), (1, 0.0)])
+@pytest.mark.parametrize("R,C", SHAPES)
+def test_gelu_fwd_bwd(jf, oracle, R, C, approx, eps, f16):
+    print(f"case gelu {R}x{C} approx={approx} f16={f16}", flush=True)
+    rng = np.random.default_rng(R * 3 + C + approx)
+    st = np.float16 if f16 else np.float32
+    sdt = "f16" if f16 else "f32"
+    qx, sx = block_tensor(oracle, rng, R, C, 2.0, f16)
+    qg, sg = block_tensor(oracle, rng, R, C, 1e-3, f16)
+    qy, sy = jf.gelu_fwd(dev(qx), dev(sx), approx, eps)
+    wq, ws = oracle.gelu_fwd(qx, sx.astype(np.float32), approx, eps, scale_dtype=sdt)
+    same(qy, wq, "fwd codes")
+    same(sy, ws, "fwd scales")
+    for rounding, stochastic in ((0, False), (1, True)):
+        qd, sd = jf.gelu_bwd(dev(qx), dev(sx), dev(qg), dev(sg), approx, rounding, seed=8, offset=3)
+        wq, ws = oracle.gelu_bwd(qx, sx.astype(np.float32), qg, sg.astype(np.float32), approx, stochastic, 8, 3,
+                                 scale_dtype=sdt)
+        same(qd, wq, f"bwd codes stochastic={stochastic}")
+        same(sd, ws, "bwd scales")
+
+
+def test_gelu_fwd_close_to_torch(jf, oracle):
+    """1e-3 relative on dequantised outputs vs torch's erf GELU of the dequantised input."""
+    rng = np.random.default_rng(12)
+    qx, sx = block_tensor(oracle, rng, 256, 512, 1.5)
+    qy, sy = jf.gelu_fwd(dev(qx), dev(sx))
+    y = jf.dequantize(qy, sy).cpu().numpy()
+    x = torch.from_numpy(qx * expand_scales(sx.astype(np.float32)).astype(np.float64))
+    ref = torch.nn.functional.gelu(x).numpy()
+    step = expand_scales(sy.cpu().numpy().astype(np.float32))
+    assert np.all(np.abs(y - ref) <= 0.5 * step * (1 + 1e-3) + 1e-3 * np.abs(ref))
+
+
+@pytest.mark.parametrize("f16", [True, False])
+@pytest.mark.parametrize("R,C", SHAPES)
+def test_rowstats_layernorm(jf, oracle, R, C, f16):
+    print(f"case layernorm {R}x{C} f16={f16}", flush=True)
+    rng = np.random.default_rng(R + 7 * C)
+    sdt = "f16" if f16 else "f32"
+    qx, sx = block_tensor(oracle, rng, R, C, 1.0, f16)
+    qg, sg = block_tensor(oracle, rng, R, C, 1e-3, f16)
+    gamma = (1 + 0.1 * rng.standard_normal(C)).astype(np.float32)
+    beta = (0.1 * rng.standard_normal(C)).astype(np.float32)
+    mean, rstd = jf.rowstats(dev(qx), dev(sx), 1e-5)
+    wm, wr = oracle.rowstats(qx, sx.astype(np.float32), 1e-5)
+    same(mean, wm, "mean")
+    same(rstd, wr, "rstd")
+    for b in (beta, None):
+        qy, sy = jf.layernorm_fwd(dev(qx), dev(sx), dev(gamma), None if b is None else dev(b), mean, rstd)
+        wq, ws = oracle.layernorm_fwd(qx, sx.astype(np.float32), gamma, b, wm, wr, scale_dtype=sdt)
+        same(qy, wq, "fwd codes")
+        same(sy, ws, "fwd scales")
+    for rounding, stochastic in ((0, False), (1, True)):
+        qd, sd, dg, db = jf.layernorm_bwd(dev(qx), dev(sx), dev(qg), dev(sg), dev(gamma), mean, rstd, rounding,
+                                          seed=77, offset=1)
+        wq, ws, wdg, wdb = oracle.layernorm_bwd(qx, sx.astype(np.float32), qg, sg.astype(np.float32), gamma, wm, wr,
+                                                stochastic, 77, 1, scale_dtype=sdt)
+        same(qd, wq, f"bwd codes stochastic={stochastic}")
+        same(sd, ws, "bwd scales")
+        assert np.allclose(dg.cpu().numpy(), wdg, rtol=1e-5, atol=1e-5 * np.abs(wdg).max())
+        assert np.allclose(db.cpu().numpy(), wdb, rtol=1e-5, atol=1e-5 * np.abs(wdb).max())
+
+
+def test_layernorm_vs_torch(jf, oracle):
+    """Against torch.nn.functional.layer_norm + autograd on the dequantised operands."""
+    rng = np.random.default_rng(21)
+    R, C = 128, 1600
+    qx, sx = block_tensor(oracle, rng, R, C, 1.0)
+    qg, sg = block_tensor(oracle, rng, R, C, 1e-3)
+    gamma = (1 + 0.1 * rng.standard_normal(C)).astype(np.float32)
+    beta = (0.1 * rng.standard_normal(C)).astype(np.float32)
+    mean, rstd = jf.rowstats(dev(qx), dev(sx), 1e-5)
+    qy, sy = jf.layernorm_fwd(dev(qx), dev(sx), dev(gamma), dev(beta), mean, rstd)
+    qd, sd, dg, db = jf.layernorm_bwd(dev(qx), dev(sx), dev(qg), dev(sg), dev(gamma), mean, rstd)
+    x = torch.tensor(qx * expand_scales(sx.astype(np.float32)).astype(np.float64), requires_grad=True)
+    gt = torch.tensor(gamma.astype(np.float64), requires_grad=True)
+    bt = torch.tensor(beta.astype(np.float64), requires_grad=True)
+    y = torch.nn.functional.layer_norm(x, (C,), gt, bt, 1e-5)
+    y.backward(torch.tensor(qg * expand_scales(sg.astype(np.float32)).astype(np.float64)))
+    for (q, s, ref) in ((qy, sy, y.detach().numpy()), (qd, sd, x.grad.numpy())):
+        got = jf.dequantize(q, s).cpu().numpy()
+        step = expand_scales(s.cpu().numpy().astype(np.float32))
+        assert np.all(np.abs(got - ref) <= 0.5 * step * (1 + 2e-3) + 1e-3 * np.abs(ref))
+    assert np.allclose(dg.cpu().numpy(), gt.grad.numpy(), rtol=1e-3, atol=1e-6)
+    assert np.allclose(db.cpu().numpy(), bt.grad.numpy(), rtol=1e-3, atol=1e-6)
+
+
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16, torch.float16])
+@pytest.mark.parametrize("mode", ["trunc", "nearest", "stochastic_trunc", "stochastic"])
+def test_add(jf, oracle, dtype, mode):
+    rng = np.random.default_rng(31)
+    R, C = 96, 160
+    x1 = torch.from_numpy(rng.standard_normal((R, C)).astype(np.float32)).to(dtype)
+    q2, s2 = block_tensor(oracle, rng, R, C, 0.5)
+    y1, q, s, rs, rq = jf.add(x1.cuda(), dev(q2), dev(s2), ROUND[mode], with_stats=True, seed=9, offset=2)
+    wy, wq, ws, wrs, wrq = oracle.add(x1.float().numpy(), q2, s2.astype(np.float32), "stochastic" in mode, 9, 2,
+                                      "trunc" in mode, True, "f16")
+    same(y1, wy, "fp sum")
+    same(q, wq, "codes")
+    same(s, ws, "scales")
+    same(rs, wrs, "row sums")
+    same(rq, wrq, "row square sums")
+
+
+def test_full_size_nonlinear_properties(jf, oracle):
+    """BASELINE config 4 sizes.  Checked bit-exactly against the oracle on row slabs (the kernels are
+    block-local, so a slab of the input is a complete problem), and by size-independent properties."""
+    g = torch.Generator().manual_seed(0)
+    x = torch.randn(8192, 6400, generator=g)
+    qx, sx = jf.quantize(x.cuda(), scale_dtype=torch.float32)
+    qy, sy = jf.gelu_fwd(qx, sx, jf.GELU_TANH, 0.0)
+    assert int(qy.abs().max()) == 127
+    blocks = qy.reshape(256, 32, 200, 32).abs().amax(dim=(1, 3))
+    assert bool((blocks == 127).all())                      # every non-zero block uses the full code range
+    for r0 in (0, 4096, 8160):
+        wq, ws = oracle.gelu_fwd(qx[r0:r0 + 32].cpu().numpy(), sx[r0 // 32:r0 // 32 + 1].cpu().numpy(), 1, 0.0)
+        same(qy[r0:r0 + 32], wq, f"gelu codes rows {r0}")
+        same(sy[r0 // 32:r0 // 32 + 1], ws, f"gelu scales rows {r0}")
+    # quantise(dequantise(q, s)) == (q, s): idempotence at full size
+    back = jf.dequantize(qy, sy)
+    q2, s2 = jf.quantize(back, scale_dtype=torch.float32)
+    assert torch.equal(q2, qy)
+    # transpose twice is the identity
+    assert torch.equal(jf.transpose_s8(jf.transpose_s8(qy)), qy)
