@@ -108,7 +108,7 @@ def test_gelu_fwd_bwd(jf, oracle, R, C, approx, eps, f16):
 def test_gelu_fwd_close_to_torch(jf, oracle):
     """1e-3 relative on dequantised outputs vs torch's erf GELU of the dequantised input."""
     rng = np.random.default_rng(12)
-    qx, sx = block_tensor(oracle, rng, 256, 512, 1.5)
+    qx, sx = block_tensor(oracle, rng, 256, 512, 1.5, f16=False)   # fp32 scales: the stored scale is the one used
     qy, sy = jf.gelu_fwd(dev(qx), dev(sx))
     y = jf.dequantize(qy, sy).cpu().numpy()
     x = torch.from_numpy(qx * expand_scales(sx.astype(np.float32)).astype(np.float64))
@@ -151,8 +151,8 @@ def test_layernorm_vs_torch(jf, oracle):
     """Against torch.nn.functional.layer_norm + autograd on the dequantised operands."""
     rng = np.random.default_rng(21)
     R, C = 128, 1600
-    qx, sx = block_tensor(oracle, rng, R, C, 1.0)
-    qg, sg = block_tensor(oracle, rng, R, C, 1e-3)
+    qx, sx = block_tensor(oracle, rng, R, C, 1.0, f16=False)       # fp32 scales: the stored scale is the one used
+    qg, sg = block_tensor(oracle, rng, R, C, 1e-3, f16=False)
     gamma = (1 + 0.1 * rng.standard_normal(C)).astype(np.float32)
     beta = (0.1 * rng.standard_normal(C)).astype(np.float32)
     mean, rstd = jf.rowstats(dev(qx), dev(sx), 1e-5)
