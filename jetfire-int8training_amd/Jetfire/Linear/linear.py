@@ -1,0 +1,73 @@
+"""int8_linear_forward / int8_linear_backward on top of the BlockQuantizeCUDA extension.
+
+Data format everywhere: codes int8 [..., R, C] with one scale per 32x32 tile, scales [..., R/32, C/32]
+(float16 as in the reference, float32 accepted).  The GEMM entry points want both scale operands K-major
+([K/32, rows/32]), hence the small transposes below (reference: linear_fwd.py:17-18, linear_bwd.py:11).
+"""
+import os
+import sys
+
+import torch
+
+_PKG = os.path.dirname(os.path.dirname(os.path.dirname(os.path.abspath(__file__))))
+if _PKG not in sys.path:
+    sys.path.insert(0, _PKG)
+
+import BlockQuantizeCUDA as BQC  # noqa: E402
+import jetfire_hip as _jf  # noqa: E402
+
+
+def _flat2(t):
+    """[..., C] -> [prod(...), C] without copying when possible."""
+    return t.reshape(-1, t.shape[-1])
+
+
+def _k_major(s2d):
+    return s2d.t().contiguous()
+
+
+def _check_block(B):
+    if B != 32:
+        raise RuntimeError(f"the INT8 GEMM kernels use 32x32 quantisation blocks, got B={B}")
+
+
+def _dequant_like(q2d, s2d, lead_shape):
+    out = _jf.dequantize(q2d, s2d).to(s2d.dtype)
+    return out.reshape(*lead_shape, q2d.shape[-1])
+
+
+def int8_linear_forward(X8_3D, SX16_3D, W8, SW16, output_quantized, B):
+    """Y = X W^T.  X8 [BS,T,K] (or [M,K]), SX [BS,T/32,K/32]; W8 [N,K], SW [N/32,K/32].
+    Returns (O8 [BS,T,N], SO [BS,T/32,N/32]) or, with output_quantized=False, the dequantised
+    output in the scale dtype (reference: linear_fwd.py:4-32)."""
+    _check_block(B)
+    lead = tuple(X8_3D.shape[:-1])
+    s_lead = tuple(SX16_3D.shape[:-1])
+    x2 = _flat2(X8_3D)
+    sx2 = _flat2(SX16_3D)
+    n_out = W8.shape[0]
+    m, k = x2.shape
+    zero_bias = torch.zeros(n_out, dtype=torch.float32, device=W8.device)
+    zero_biasmax = torch.zeros(1, dtype=torch.float32, device=W8.device)
+    o8, so = BQC.igemm_output_int_quantize_bias_rowcol(x2.contiguous(), W8.t(), zero_bias, zero_biasmax,
+                                                       _k_major(sx2), _k_major(SW16), m, n_out, k)
+    if not output_quantized:
+        return _dequant_like(o8, so, lead)
+    return o8.reshape(*lead, n_out), so.reshape(*s_lead, SW16.shape[0])
+
+
+def int8_linear_backward(X8_3D, SX16_3D, G8_3D, SG16_3D, G8T, W8, SW16, B, stochastic=True, dgrad_quantize=True):
+    """dX = dY W (requantised with stochastic rounding) and dW = dY^T X (fp16).
+    G8 [BS,T,N] with SG [BS,T/32,N/32]; G8T = G8 transposed to [N, BS*T]; W8 [N,K], SW [N/32,K/32].
+    Returns (GX8, GSX, GW) or (GX_fp, GW) when dgrad_quantize=False (reference: linear_bwd.py:4-29; like
+    there, the activation gradient is always rounded stochastically)."""
+    _check_block(B)
+    g2, sg2 = _flat2(G8_3D).contiguous(), _flat2(SG16_3D).contiguous()
+    x2, sx2 = _flat2(X8_3D).contiguous(), _flat2(SX16_3D).contiguous()
+    tokens, c_out = g2.shape
+    c_in = W8.shape[1]
+    gx8, gsx = BQC.igemm_output_int_quantize_stochastic(g2, W8, _k_major(sg2), SW16, tokens, c_in, c_out)
+    gw = BQC.igemm_output_fp_no_quantize(G8T, x2, sg2, sx2, G8T.shape[0], c_in, G8T.shape[1])
+    if not dgrad_quantize:
+        return _dequant_like(gx8, gsx, tuple(G8_3D.shape[:-1])), gw
+    return (gx8.reshape(*G8_3D.shape[:-1], c_in), gsx.reshape(*SG16_3D.shape[:-1], SW16.shape[1]), gw)

@@ -1,0 +1,239 @@
+"""The drop-in boundary: module BlockQuantizeCUDA and packages Linear / Nonlinear, imported the way
+INT8_GPT2/qmodel.py:18-22 imports them, with the reference's names, argument order and return shapes."""
+import inspect
+
+import numpy as np
+import pytest
+import torch
+
+from helpers import QB, rand_codes, rand_scales
+
+
+# ------------------------------------------------------------------------------------------- CPU side
+def test_imports_and_names():
+    import BlockQuantizeCUDA as BQC
+    from Linear import int8_linear_backward, int8_linear_forward  # noqa: F401
+    from Nonlinear import (int8_add_Ifp_Ig16_Ofp_Og, int8_add_Ifp_Ig16_Ofp_Og_MeanVar, int8_gelu_backward,  # noqa: F401
+                           int8_gelu_forward, int8_layernorm_backward, int8_layernorm_forward, int8_quantize,
+                           int8_quantize_transpose, int8_transpose)
+    for name in ("igemm_output_int_quantize_stochastic", "igemm_output_int_quantize_bias_rowcol",
+                 "igemm_output_int_quantize_bias_rowrow", "igemm_output_int_quantize",
+                 "igemm_output_int_quantize_fused", "igemm_output_fp_no_quantize", "igemm_basic_int8_gemm", "hgemm_v1"):
+        assert callable(getattr(BQC, name)), name
+
+
+# positional parameters of the reference launchers (Jetfire/Linear/*.py, Jetfire/Nonlinear/*.py)
+SIGNATURES = {
+    "Linear.int8_linear_forward": ["X8_3D", "SX16_3D", "W8", "SW16", "output_quantized", "B"],
+    "Linear.int8_linear_backward": ["X8_3D", "SX16_3D", "G8_3D", "SG16_3D", "G8T", "W8", "SW16", "B", "stochastic",
+                                    "dgrad_quantize"],
+    "Nonlinear.int8_quantize": ["x", "QB", "stochastic"],
+    "Nonlinear.int8_quantize_transpose": ["x", "QB", "stochastic", "transpose_output_2d"],
+    "Nonlinear.int8_transpose": ["x", "transpose_output_2d"],
+    "Nonlinear.int8_dequantize": ["x", "s_x", "QB"],
+    "Nonlinear.int8_layernorm_forward": ["x", "sx", "weight", "mean", "rstd", "QB", "eps"],
+    "Nonlinear.int8_layernorm_backward": ["x", "sx", "g", "sg", "w", "QB", "m", "v", "stochastic", "eps"],
+    "Nonlinear.int8_gelu_forward": ["x", "s_x", "QB"],
+    "Nonlinear.int8_gelu_backward": ["x", "s_x", "g", "s_g", "QB", "stochastic"],
+    "Nonlinear.int8_add_Ifp_Ig16_Ofp_Og": ["x1", "x2", "s_x2", "QB", "stochastic"],
+    "Nonlinear.int8_add_Ifp_Ig16_Ofp_Og_MeanVar": ["x1", "x2", "s_x2", "QB"],
+}
+
+
+@pytest.mark.parametrize("qual,params", SIGNATURES.items())
+def test_signatures(qual, params):
+    import importlib
+    mod, fn = qual.split(".")
+    f = getattr(importlib.import_module(mod), fn)
+    got = list(inspect.signature(f).parameters)
+    assert got[:len(params)] == params
+    for extra in got[len(params):]:                 # anything we add must be optional
+        assert inspect.signature(f).parameters[extra].default is not inspect.Parameter.empty
+
+
+def test_cpu_tensors_are_rejected_not_computed():
+    """No CPU fallback: host tensors raise."""
+    import BlockQuantizeCUDA as BQC
+    from Nonlinear import int8_gelu_forward, int8_quantize
+    x = torch.randn(32, 32)
+    with pytest.raises(RuntimeError, match="GPU"):
+        int8_quantize(x, 32)
+    with pytest.raises(RuntimeError, match="GPU"):
+        int8_gelu_forward(torch.zeros(32, 32, dtype=torch.int8), torch.ones(1, 1, dtype=torch.float16), 32)
+    with pytest.raises(RuntimeError, match="32"):
+        int8_quantize(x, 16)
+    a = torch.zeros(32, 32, dtype=torch.int8)
+    s = torch.ones(1, 1, dtype=torch.float16)
+    with pytest.raises(RuntimeError, match="GPU"):
+        BQC.igemm_output_int_quantize(a, a, s, s, 32, 32, 32)
+    with pytest.raises(RuntimeError, match="multiples of 32"):
+        BQC.igemm_basic_int8_gemm(a, a, 32, 48, 32)
+    with pytest.raises(RuntimeError, match="not implemented"):
+        BQC.igemm_output_int_quantize_fused(a, a, s, s, 32, 32, 32)
+
+
+# ------------------------------------------------------------------------------------------- GPU side
+def dev(a):
+    return torch.from_numpy(np.ascontiguousarray(a)).cuda()
+
+
+def eq(got, want):
+    got = got.cpu().numpy()
+    if got.dtype == np.float16:
+        return np.array_equal(got.view(np.uint16), np.asarray(want, np.float16).view(np.uint16))
+    return np.array_equal(got, want)
+
+
+@pytest.mark.gpu
+def test_bqc_functions_match_oracle(oracle):
+    """Layouts as the reference's test scripts build them: sx [m/b,k/b] passed as sx.t().contiguous(),
+    sw [k/b,n/b] passed as is (JetfireGEMMKernel/tests/test_int8igemmoutputIntQuantizeStochastic.py:24-41)."""
+    import BlockQuantizeCUDA as BQC
+    rng = np.random.default_rng(0)
+    m, n, k = 128, 256, 96
+    qx, qw = rand_codes(rng, (m, k)), rand_codes(rng, (k, n))
+    sx, sw = rand_scales(rng, (m // QB, k // QB)), rand_scales(rng, (k // QB, n // QB))
+    sxT = np.ascontiguousarray(sx.T)
+    dqx, dqw = dev(qx), dev(qw)
+    dsxT, dsw = dev(sxT.astype(np.float16)), dev(sw.astype(np.float16))
+
+    assert eq(BQC.igemm_basic_int8_gemm(dqx, dqw, m, n, k), oracle.igemm_s32(qx, qw, 1))
+    out = BQC.igemm_output_fp_no_quantize(dqx, dqw, dsxT, dsw, m, n, k)
+    assert out.dtype == torch.float16 and eq(out, oracle.igemm_block_fp(qx, qw, sxT, sw, 1, "f16"))
+    o, so = BQC.igemm_output_int_quantize(dqx, dqw, dsxT, dsw, m, n, k)
+    wq, ws = oracle.igemm_block_q(qx, qw, sxT, sw, 1, scale_dtype="f16")
+    assert o.dtype == torch.int8 and so.dtype == torch.float16 and tuple(so.shape) == (m // QB, n // QB)
+    assert eq(o, wq) and eq(so, ws)
+
+    torch.manual_seed(1234)
+    BQC.philox_set_offset(0, 40)
+    seed, offset = BQC.philox_peek(0)
+    assert (seed, offset) == (1234, 40)
+    o, so = BQC.igemm_output_int_quantize_stochastic(dqx, dqw, dsxT, dsw, m, n, k)
+    wq, ws = oracle.igemm_block_q(qx, qw, sxT, sw, 1, stochastic=True, seed=seed, offset=offset, scale_dtype="f16")
+    assert eq(o, wq) and eq(so, ws)
+    assert BQC.philox_peek(0) == (1234, 40 + m * n // 8)
+    o2, _ = BQC.igemm_output_int_quantize_stochastic(dqx, dqw, dsxT, dsw, m, n, k)
+    assert not torch.equal(o, o2)                    # fresh noise on every call
+
+    bias = (0.05 * rng.standard_normal(n)).astype(np.float32)
+    biasmax = np.array([np.abs(bias).max()], np.float32)
+    wq, ws = oracle.igemm_block_q(qx, qw, sxT, sw, 1, bias=bias, biasmax=float(biasmax[0]), scale_dtype="f16")
+    o, so = BQC.igemm_output_int_quantize_bias_rowrow(dqx, dqw, dev(bias), dev(biasmax), dsxT, dsw, m, n, k)
+    assert eq(o, wq) and eq(so, ws)
+    # row x col: W stored [n,k], passed as its .t() view (JetfireGEMMKernel/tests/…BiasRowCol.py:38-40)
+    w_nk = dev(np.ascontiguousarray(qw.T))
+    view = w_nk.t()
+    assert not view.is_contiguous()
+    o, so = BQC.igemm_output_int_quantize_bias_rowcol(dqx, view, dev(bias), dev(biasmax), dsxT, dsw, m, n, k)
+    assert eq(o, wq) and eq(so, ws)
+    h = BQC.hgemm_v1(dqx.half(), dqw.half(), m, n, k)
+    assert h.dtype == torch.float16 and tuple(h.shape) == (m, n)
+
+
+@pytest.mark.gpu
+def test_bqc_error_paths():
+    import BlockQuantizeCUDA as BQC
+    a = torch.zeros(64, 64, dtype=torch.int8, device="cuda")
+    s = torch.ones(2, 2, dtype=torch.float16, device="cuda")
+    with pytest.raises(RuntimeError, match="int8"):
+        BQC.igemm_output_int_quantize(a.float(), a, s, s, 64, 64, 64)
+    with pytest.raises(RuntimeError, match="SX must be"):
+        BQC.igemm_output_int_quantize(a, a, s[:1], s, 64, 64, 64)
+    with pytest.raises(RuntimeError, match="same dtype"):
+        BQC.igemm_output_int_quantize(a, a, s, s.float(), 64, 64, 64)
+    with pytest.raises(RuntimeError, match="contiguous"):
+        BQC.igemm_output_int_quantize(a, a.t(), s, s, 64, 64, 64)
+    with pytest.raises(RuntimeError, match="same GPU"):
+        BQC.igemm_output_int_quantize(a, a.cpu(), s, s, 64, 64, 64)
+    with pytest.raises(RuntimeError, match=r"\[M,K\]"):
+        BQC.igemm_output_int_quantize(a, a, s, s, 32, 64, 64)
+
+
+@pytest.mark.gpu
+def test_linear_package_3d_shapes_and_values(oracle):
+    from Linear import int8_linear_backward, int8_linear_forward
+    from Nonlinear import int8_dequantize, int8_quantize, int8_quantize_transpose, int8_transpose
+    import BlockQuantizeCUDA as BQC
+    torch.manual_seed(7)
+    BS, T, Cin, Cout = 2, 64, 96, 160
+    x = torch.randn(BS, T, Cin, device="cuda")
+    w = torch.randn(Cout, Cin, device="cuda") * 0.02
+    g = torch.randn(BS, T, Cout, device="cuda", dtype=torch.float16) * 1e-3
+    qx, sx = int8_quantize(x, 32)
+    qw, sw = int8_quantize(w, 32)
+    assert tuple(qx.shape) == (BS, T, Cin) and tuple(sx.shape) == (BS, T // 32, Cin // 32) and sx.dtype == torch.float16
+    o8, so = int8_linear_forward(qx, sx, qw, sw, True, 32)
+    assert tuple(o8.shape) == (BS, T, Cout) and tuple(so.shape) == (BS, T // 32, Cout // 32)
+    sx2 = sx.reshape(-1, Cin // 32)
+    wq, ws = oracle.igemm_block_q(qx.reshape(-1, Cin).cpu().numpy(), qw.cpu().numpy(),
+                                  np.ascontiguousarray(sx2.float().cpu().numpy().T),
+                                  np.ascontiguousarray(sw.float().cpu().numpy().T), 0, scale_dtype="f16")
+    assert eq(o8.reshape(-1, Cout), wq) and eq(so.reshape(-1, Cout // 32), ws)
+    ofp = int8_linear_forward(qx, sx, qw, sw, False, 32)
+    assert ofp.dtype == torch.float16 and tuple(ofp.shape) == (BS, T, Cout)
+    assert torch.equal(ofp, int8_dequantize(o8, so, 32).half())
+    ref = x.reshape(-1, Cin) @ w.t()
+    assert torch.nn.functional.cosine_similarity(ofp.reshape(-1).float(), ref.reshape(-1), dim=0) > 0.999
+
+    qg, sg, qgt = int8_quantize_transpose(g, 32, stochastic=True, transpose_output_2d=True)
+    assert tuple(qgt.shape) == (Cout, BS * T)
+    assert torch.equal(qgt, int8_transpose(qg, transpose_output_2d=True))
+    seed, off = BQC.philox_peek(0)
+    gx8, gsx, gw = int8_linear_backward(qx, sx, qg, sg, qgt, qw, sw, 32, stochastic=True)
+    assert tuple(gx8.shape) == (BS, T, Cin) and tuple(gsx.shape) == (BS, T // 32, Cin // 32)
+    assert tuple(gw.shape) == (Cout, Cin) and gw.dtype == torch.float16
+    sg2 = sg.reshape(-1, Cout // 32).float().cpu().numpy()
+    wq, ws = oracle.igemm_block_q(qg.reshape(-1, Cout).cpu().numpy(), qw.cpu().numpy(), np.ascontiguousarray(sg2.T),
+                                  sw.float().cpu().numpy(), 1, stochastic=True, seed=seed, offset=off, scale_dtype="f16")
+    assert eq(gx8.reshape(-1, Cin), wq) and eq(gsx.reshape(-1, Cin // 32), ws)
+    wgw = oracle.igemm_block_fp(qgt.cpu().numpy(), qx.reshape(-1, Cin).cpu().numpy(), sg2, sx2.float().cpu().numpy(), 1, "f16")
+    assert eq(gw, wgw)
+    gx, gw2 = int8_linear_backward(qx, sx, qg, sg, qgt, qw, sw, 32, stochastic=True, dgrad_quantize=False)
+    assert gx.dtype == torch.float16 and tuple(gx.shape) == (BS, T, Cin) and torch.equal(gw2, gw)
+    ref_gx = g.reshape(-1, Cout).float() @ w
+    assert torch.nn.functional.cosine_similarity(gx.reshape(-1).float(), ref_gx.reshape(-1), dim=0) > 0.99
+    ref_gw = g.reshape(-1, Cout).float().t() @ x.reshape(-1, Cin)
+    assert torch.nn.functional.cosine_similarity(gw.reshape(-1).float(), ref_gw.reshape(-1), dim=0) > 0.999
+
+
+@pytest.mark.gpu
+def test_nonlinear_package_3d(oracle):
+    from Nonlinear import (int8_add_Ifp_Ig16_Ofp_Og, int8_add_Ifp_Ig16_Ofp_Og_MeanVar, int8_dequantize,
+                           int8_gelu_backward, int8_gelu_forward, int8_layernorm_backward, int8_layernorm_forward,
+                           int8_quantize, int8_rowstats, int8_transpose)
+    torch.manual_seed(3)
+    BS, T, C = 2, 64, 160
+    x = torch.randn(BS, T, C, device="cuda")
+    res = torch.randn(BS, T, C, device="cuda").bfloat16()
+    w = (1 + 0.1 * torch.randn(C, device="cuda"))
+    qx, sx = int8_quantize(x, 32)
+    fp, q2, s2, mean, rstd = int8_add_Ifp_Ig16_Ofp_Og_MeanVar(res, qx, sx, 32)
+    assert fp.dtype == torch.float32 and tuple(fp.shape) == (BS, T, C) and tuple(mean.shape) == (BS, T)
+    want = res.float() + int8_dequantize(qx, sx, 32)
+    assert torch.equal(fp, want)
+    assert torch.allclose(mean, want.mean(-1), atol=1e-5) and torch.allclose(rstd, want.var(-1, unbiased=False).rsqrt(), rtol=1e-4)
+    qy, sy, (m_, r_) = int8_layernorm_forward(q2, s2, w, mean, rstd, 32)
+    assert tuple(qy.shape) == (BS, T, C) and tuple(sy.shape) == (BS, T // 32, C // 32) and m_ is mean
+    y_ref = torch.nn.functional.layer_norm(int8_dequantize(q2, s2, 32), (C,), w, None, 0.0)
+    assert torch.nn.functional.cosine_similarity(int8_dequantize(qy, sy, 32).reshape(-1), y_ref.reshape(-1), dim=0) > 0.999
+    qy2, sy2, (m2, r2) = int8_layernorm_forward(q2, s2, w, None, None, 32, eps=1e-5)     # statistics computed here
+    assert tuple(m2.shape) == (BS, T)
+    ms, rs = int8_rowstats(q2, s2, 32, 1e-5)
+    assert torch.equal(ms, m2)
+    g = torch.randn(BS, T, C, device="cuda") * 1e-3
+    qg, sg = int8_quantize(g, 32, stochastic=True)
+    qd, sd, dw = int8_layernorm_backward(q2, s2, qg, sg, w, 32, mean, rstd, stochastic=True)
+    assert tuple(qd.shape) == (BS, T, C) and tuple(dw.shape) == (C,) and dw.dtype == w.dtype
+    qh, sh = int8_gelu_forward(qx, sx, 32)
+    assert tuple(qh.shape) == (BS, T, C)
+    ref = torch.nn.functional.gelu(int8_dequantize(qx, sx, 32))
+    assert torch.nn.functional.cosine_similarity(int8_dequantize(qh, sh, 32).reshape(-1), ref.reshape(-1), dim=0) > 0.999
+    qb, sb = int8_gelu_backward(qx, sx, qg, sg, 32, stochastic=True)
+    assert tuple(qb.shape) == (BS, T, C) and sb.dtype == torch.float16
+    fpg, qa, sa = int8_add_Ifp_Ig16_Ofp_Og(g, qb, sb, 32, stochastic=True)
+    assert fpg.dtype == torch.float32 and tuple(qa.shape) == (BS, T, C)
+    t2 = int8_transpose(qx, transpose_output_2d=True)
+    assert tuple(t2.shape) == (C, BS * T)
+    t3 = int8_transpose(qx)
+    assert t3.dim() == 3 and t3.shape[0] == BS and t3.shape[-1] == BS * T     # 3-D when not asked for 2-D
