@@ -8,24 +8,22 @@
 // v_cvt_f32_i32 + one v_fma_f32 per value.  (Reference kernels: igemm_BlockSquare32OutputIntQuantize
 // BiasRowCol.cu:134-225 and its siblings under JetfireGEMMKernel/BlockQuantize/cpp_extension/igemm/.)
 //
-// Work decomposition: workgroup = 256 threads = 4 waves (2x2), tile 128x128, each wave owns a
-// 64x64 sub-tile = 2x2 quantisation blocks (64 fp32 accumulators per lane).  K is consumed in
-// stages of KB_STAGE blocks, double-buffered in LDS.  The LDS image of a 32x32 int8 block is stored
-// in MFMA operand order ([k-half][row][16 bytes]) so that every operand fetch is one linear
-// ds_read_b128 (lane l reads bytes 16*l .. 16*l+15).  Both operands are K-contiguous ("NT"); a
-// [K,N] B operand is transposed into a caller-provided workspace first.
+// Work decomposition: workgroup = 512 threads = 8 waves, tile 256x128 (or 128x256), each wave owns a
+// 64x64 sub-tile = 2x2 quantisation blocks (64 fp32 accumulators per lane).  K is consumed in stages
+// of 4 blocks (128 bytes per row) through a 3-deep LDS ring filled by LDS-direct loads
+// (global_load_lds_dwordx4: no register staging, two stages in flight while one is computed).  LDS rows
+// are 128 bytes with an XOR chunk swizzle, so the 16-byte MFMA operand reads are conflict-free.  Both
+// operands are K-contiguous ("NT"); a [K,N] B operand is transposed into a caller-provided workspace
+// first.  Scales are wave-uniform and come in through scalar loads.
 #include "jf_device.hpp"
+
+#include <type_traits>
 
 namespace jf {
 
-constexpr int BM = 128, BN = 128;
-constexpr int KB_STAGE = 4;                         // 32-deep K blocks per LDS stage (BK = 128 bytes)
-constexpr int NTHREADS = 256;
-constexpr int TILE_BYTES = (BM / QB) * KB_STAGE * 1024;          // one operand, one stage
-constexpr int STAGE_BYTES = 2 * TILE_BYTES + 2 * KB_STAGE * 4 * (int)sizeof(float);
+constexpr int KB_STAGE = 4;                         // 32-deep K blocks per LDS stage (128 bytes of K per row)
+constexpr int ROW_BYTES = KB_STAGE * QB;            // 128: one LDS row = one 128-byte global segment
 constexpr int EPI_LD = 36;                          // floats per staged row (32 + pad, keeps 16B alignment)
-constexpr int EPI_BYTES = 4 * QB * EPI_LD * (int)sizeof(float);
-constexpr int SMEM_BYTES = (2 * STAGE_BYTES > EPI_BYTES) ? 2 * STAGE_BYTES : EPI_BYTES;
 
 enum Epilogue { EPI_S32 = 0, EPI_FP = 1, EPI_Q = 2 };
 
@@ -64,15 +62,39 @@ __device__ __forceinline__ void tile_of_workgroup(int tiles_m, int tiles_n, int 
     tn = in_group / gm;
 }
 
-template <int EPI, typename ST>
-__global__ __launch_bounds__(NTHREADS, 2) void igemm_nt_kernel(GemmArgs p)
+template <int I, int N, typename F> __device__ __forceinline__ void static_for(F &&f)
 {
+    if constexpr (I < N) {
+        f(std::integral_constant<int, I>{});
+        static_for<I + 1, N>(f);
+    }
+}
+
+// vmcnt(n), no wait on the other counters (gfx9 encoding: vmcnt = bits 3:0 and 15:14)
+#define JF_WAIT_VMCNT(n) __builtin_amdgcn_s_waitcnt(((n) & 0xF) | (((n) >> 4) << 14) | 0x0F70)
+
+// WGM x WGN waves, each owning WBM x WBN quantisation blocks (64x32 elements).
+constexpr int WBM = 2, WBN = 1;
+// NSTAGE = depth of the LDS ring (one stage being computed, NSTAGE-1 in flight); WGPC = workgroups per CU.
+template <int EPI, typename ST, int WGM, int WGN, int NSTAGE, int WGPC>
+__global__ __launch_bounds__(64 * WGM * WGN, WGPC) void igemm_nt_kernel(GemmArgs p)
+{
+    constexpr int NW = WGM * WGN;
+    constexpr int BM = QB * WBM * WGM, BN = QB * WBN * WGN;
+    constexpr int A_BYTES = BM * ROW_BYTES;                  // one stage of A
+    constexpr int STAGE_BYTES = (BM + BN) * ROW_BYTES;
+    constexpr int GROUPS = (BM + BN) / 8;                    // 8-row groups (1 KiB each) per stage
+    constexpr int LPW = GROUPS / NW;                         // LDS-direct loads per wave per stage
+    static_assert(GROUPS % NW == 0, "stage must split evenly over the waves");
+    static_assert(NSTAGE >= 2 && NSTAGE <= 5, "ring depth");
+    static_assert((BM + BN) / QB <= 16, "scale patch holds 16 blocks per K block");
+
     extern __shared__ __attribute__((aligned(16))) unsigned char smem[];
 
     const int tid = threadIdx.x;
     const int lane = tid & 63;
     const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
-    const int wm = wave & 1, wn = wave >> 1;
+    const int wm = wave % WGM, wn = wave / WGM;
 
     int tile_m, tile_n;
     tile_of_workgroup(p.tiles_m, p.tiles_n, tile_m, tile_n);
@@ -81,110 +103,218 @@ __global__ __launch_bounds__(NTHREADS, 2) void igemm_nt_kernel(GemmArgs p)
     const int nkb = p.K / QB;
     const int nstages = (nkb + KB_STAGE - 1) / KB_STAGE;
 
-    // ---- global -> register -> LDS staging -------------------------------------------------
-    // One operand stage is 128 rows x 8 chunks of 16 bytes; thread t moves chunks t, t+256, ...
-    // (8 consecutive lanes cover one 128-byte row segment).
-    constexpr int CHUNKS = BM * KB_STAGE * 2 / NTHREADS;      // 4 per operand per thread
-    v4i ra[CHUNKS], rb[CHUNKS];
-    float rs = 0.0f;                                          // this thread's scale of the stage (tid < 32)
+    // ---- global -> LDS, without passing through registers ------------------------------------
+    // A stage in LDS is (BM+BN) rows of 128 bytes (A rows first).  One load instruction of one wave
+    // moves 8 rows: lane l supplies the address of one 16-byte chunk and the hardware writes it to
+    // LDS at (base + 16*l), i.e. row l/8, slot l%8.  To keep the later 16-byte operand reads free of
+    // bank conflicts, slot c' of row r holds global chunk c' ^ ((r>>1)&7); the permutation stays
+    // inside the row's 128-byte segment, so every instruction still reads 8 full 128-byte lines.
+    unsigned goff[LPW];            // byte offset of this lane's chunk from the operand base (stage 0)
+    bool is_a[LPW];
+#pragma unroll
+    for (int j = 0; j < LPW; ++j) {
+        const int grp = wave + j * NW;                        // wave-uniform
+        is_a[j] = grp < BM / 8;
+        const int r = (is_a[j] ? grp : grp - BM / 8) * 8 + (lane >> 3);   // row inside the operand tile
+        const int c = (lane & 7) ^ ((r >> 1) & 7);
+        int gr = (is_a[j] ? m0 : n0) + r;
+        const int lim = is_a[j] ? p.M : p.N;
+        gr = gr < lim ? gr : lim - 1;                         // rows of a partial tile: any valid row
+        goff[j] = (unsigned)gr * (unsigned)(is_a[j] ? p.lda : p.ldb) + c * 16;
+    }
+    // Scales of a stage: every wave fetches, again LDS-direct, the 4 x (BM/32 + BN/32) scales of the stage into a
+    // private 256-byte patch (lane l: K block l/16, tile block l%16; A blocks first), so that scale reads need no
+    // cross-wave synchronisation and every wave has the same number of loads in flight.  binary16 scales are
+    // fetched as the aligned 32-bit word that contains them.
+    constexpr int SCALE_WORDS = 64;
+    unsigned char *const scale_ring = smem + NSTAGE * STAGE_BYTES + wave * (NSTAGE * SCALE_WORDS * 4);
+    const int s_blk = lane & 15;
+    const bool s_is_a = s_blk < BM / QB || s_blk >= (BM + BN) / QB;      // spare lanes repeat A block 0
+    int s_idx = s_is_a ? m0 / QB + (s_blk < BM / QB ? s_blk : 0) : n0 / QB + s_blk - BM / QB;
+    { const int lim = s_is_a ? SM : SN; s_idx = s_idx < lim ? s_idx : lim - 1; }
+    const int s_ld = s_is_a ? SM : SN;
+    const unsigned char *const s_base = reinterpret_cast<const unsigned char *>(s_is_a ? p.sa : p.sb);
 
-    auto load_stage = [&](int stage) {
+    auto issue_stage = [&](int stage) {
+        unsigned char *dst = smem + (stage % NSTAGE) * STAGE_BYTES;
         const int kb0 = stage * KB_STAGE;
-#pragma unroll
-        for (int c = 0; c < CHUNKS; ++c) {
-            const int id = tid + c * NTHREADS;
-            const int row = id >> 3, ch = id & 7;
-            const int kb = kb0 + (ch >> 1);
-            const int kbc = kb < nkb ? kb : nkb - 1;          // clamp: data of a missing block is never used
-            const int koff = kbc * QB + (ch & 1) * 16;
-            int ar = m0 + row; ar = ar < p.M ? ar : p.M - 1;  // clamp rows of partial tiles
-            int br = n0 + row; br = br < p.N ? br : p.N - 1;
-            ra[c] = *reinterpret_cast<const v4i *>(p.A + (size_t)ar * p.lda + koff);
-            rb[c] = *reinterpret_cast<const v4i *>(p.B + (size_t)br * p.ldb + koff);
+        if (EPI != EPI_S32) {
+            int kbg = kb0 + (lane >> 4);
+            kbg = kbg < nkb ? kbg : nkb - 1;
+            const unsigned e = (unsigned)(kbg * s_ld + s_idx);
+            const unsigned char *src = s_base + (sizeof(ST) == 4 ? e * 4u : (e >> 1) * 4u);
+            __builtin_amdgcn_global_load_lds((const __attribute__((address_space(1))) void *)src,
+                                             (__attribute__((address_space(3))) void *)(scale_ring + (stage % NSTAGE) * (SCALE_WORDS * 4)),
+                                             4, 0, 0);
         }
-        if (EPI != EPI_S32 && tid < 2 * KB_STAGE * 4) {
-            // tid = which*16 + kb*4 + blk : scale of K block kb for tile block blk of A (which=0) / B (1)
-            const int which = tid >> 4, kb = (tid >> 2) & 3, blk = tid & 3;
-            int kbg = kb0 + kb; kbg = kbg < nkb ? kbg : nkb - 1;
-            if (which == 0) {
-                int mb = m0 / QB + blk; mb = mb < SM ? mb : SM - 1;
-                rs = load_scale(reinterpret_cast<const ST *>(p.sa), kbg * SM + mb);
-            } else {
-                int nb = n0 / QB + blk; nb = nb < SN ? nb : SN - 1;
-                rs = load_scale(reinterpret_cast<const ST *>(p.sb), kbg * SN + nb);
+        const bool partial = kb0 + KB_STAGE > nkb;            // last stage of a K that is not a multiple of 128
+#pragma unroll
+        for (int j = 0; j < LPW; ++j) {
+            const int grp = wave + j * NW;
+            unsigned off = goff[j] + (unsigned)kb0 * QB;
+            if (partial) {
+                // chunks of missing K blocks: fetch the stage's first block again (never used)
+                const int r = (is_a[j] ? grp : grp - BM / 8) * 8 + (lane >> 3);
+                const int c = (lane & 7) ^ ((r >> 1) & 7);
+                if (kb0 + (c >> 1) >= nkb) off -= (unsigned)(c >> 1) * QB;
             }
+            const int8_t *src = (is_a[j] ? p.A : p.B) + off;
+            __builtin_amdgcn_global_load_lds((const __attribute__((address_space(1))) void *)src,
+                                             (__attribute__((address_space(3))) void *)(dst + grp * 1024), 16, 0, 0);
         }
     };
-    auto store_stage = [&](int buf) {
-        unsigned char *base = smem + buf * STAGE_BYTES;
+
+    // ---- operand fetch addresses ----------------------------------------------------------------
+    // MFMA operand layout: lane l holds row l%32 of the block and K bytes 16*(l/32) .. +15, i.e. chunk
+    // 2*kb + l/32 of the stage row.  Both operands use the same mapping, so one offset per K block.
+    // (Ring slot, block index and the A/B split are compile-time offsets folded into the instruction.)
+    unsigned fa_off[KB_STAGE], fb_off[KB_STAGE];
 #pragma unroll
-        for (int c = 0; c < CHUNKS; ++c) {
-            const int id = tid + c * NTHREADS;
-            const int row = id >> 3, ch = id & 7;
-            const int off = (((row >> 5) * KB_STAGE + (ch >> 1)) * 2 + (ch & 1)) * 512 + (row & 31) * 16;
-            *reinterpret_cast<v4i *>(base + off) = ra[c];
-            *reinterpret_cast<v4i *>(base + TILE_BYTES + off) = rb[c];
-        }
-        if (EPI != EPI_S32 && tid < 2 * KB_STAGE * 4)
-            reinterpret_cast<float *>(base + 2 * TILE_BYTES)[tid] = rs;
-    };
+    for (int kb = 0; kb < KB_STAGE; ++kb) {
+        const unsigned fo = (lane & 31) * ROW_BYTES + (((2 * kb + (lane >> 5)) ^ ((lane >> 1) & 7)) << 4);
+        fa_off[kb] = fo + (wm * WBM * QB) * ROW_BYTES;
+        fb_off[kb] = fo + (wn * WBN * QB) * ROW_BYTES;
+    }
 
     // ---- accumulators ------------------------------------------------------------------------
-    float acc[2][2][16];
-    v16i iacc[2][2];
+    float acc[WBM][WBN][16];
+    v16i iacc[WBM][WBN];
 #pragma unroll
-    for (int i = 0; i < 2; ++i)
+    for (int i = 0; i < WBM; ++i)
 #pragma unroll
-        for (int j = 0; j < 2; ++j) {
+        for (int j = 0; j < WBN; ++j) {
 #pragma unroll
             for (int v = 0; v < 16; ++v) { acc[i][j][v] = 0.0f; iacc[i][j][v] = 0; }
         }
-
-    load_stage(0);
-    store_stage(0);
-    __syncthreads();
-
-    for (int s = 0; s < nstages; ++s) {
-        if (s + 1 < nstages) load_stage(s + 1);
-        const unsigned char *base = smem + (s & 1) * STAGE_BYTES;
-        const float *sc_lds = reinterpret_cast<const float *>(base + 2 * TILE_BYTES);
-        const int kbs = (nkb - s * KB_STAGE) < KB_STAGE ? (nkb - s * KB_STAGE) : KB_STAGE;
-        for (int kb = 0; kb < kbs; ++kb) {
-            v4i a[2], b[2];
+    // 1.5*2^23 as an integer bit pattern in 16 registers: the accumulator INPUT of every product (see below).
+    // Written through asm so that the compiler keeps the registers instead of re-creating the constant.
+    v16i magic;
 #pragma unroll
-            for (int i = 0; i < 2; ++i) {
-                a[i] = *reinterpret_cast<const v4i *>(base + ((wm * 2 + i) * KB_STAGE + kb) * 1024 + lane * 16);
-                b[i] = *reinterpret_cast<const v4i *>(base + TILE_BYTES + ((wn * 2 + i) * KB_STAGE + kb) * 1024 + lane * 16);
-            }
+    for (int v = 0; v < 16; ++v) {
+        int m;
+        asm volatile("v_mov_b32 %0, 0x4b400000" : "=v"(m));
+        magic[v] = m;
+    }
+
+    // block indices of this wave's scales (clamped for partial tiles: those blocks are never stored)
+    int mb[WBM], nb[WBN];
+#pragma unroll
+    for (int i = 0; i < WBM; ++i) { mb[i] = m0 / QB + wm * WBM + i; mb[i] = mb[i] < SM ? mb[i] : SM - 1; }
+#pragma unroll
+    for (int j = 0; j < WBN; ++j) { nb[j] = n0 / QB + wn * WBN + j; nb[j] = nb[j] < SN ? nb[j] : SN - 1; }
+
+    constexpr int AHEAD = NSTAGE - 1;                         // stages in flight beyond the one being computed
+#pragma unroll
+    for (int s = 0; s < AHEAD; ++s)
+        if (s < nstages) issue_stage(s);
+
+    for (int s0 = 0; s0 < nstages; s0 += NSTAGE) static_for<0, NSTAGE>([&](auto slot_c) {
+        constexpr int SLOT = decltype(slot_c)::value;         // ring slot of this stage, a compile-time constant
+        const int s = s0 + SLOT;
+        if (s >= nstages) return;
+        // Loads retire in order, so stage s has landed once only the loads of the younger stages
+        // (s+1 .. s+AHEAD-1, those that exist) are still outstanding.  The barrier then (a) publishes every
+        // wave's part of stage s and (b) guarantees that all waves are done with stage s-1, whose ring slot
+        // the loads issued below overwrite.  (A bare s_barrier: __syncthreads() would drain all loads.)
+        constexpr int LOADS = LPW + (EPI != EPI_S32 ? 1 : 0);    // per wave and stage
+        int younger = nstages - 1 - s;
+        younger = younger < AHEAD - 1 ? younger : AHEAD - 1;
+        if (younger >= 3) JF_WAIT_VMCNT(3 * LOADS);
+        else if (younger == 2) JF_WAIT_VMCNT(2 * LOADS);
+        else if (younger == 1) JF_WAIT_VMCNT(LOADS);
+        else JF_WAIT_VMCNT(0);
+#if !(defined(JF_DBG_MODE) && (JF_DBG_MODE == 6 || JF_DBG_MODE == 7))
+        asm volatile("" ::: "memory");
+        __builtin_amdgcn_s_barrier();
+        asm volatile("" ::: "memory");
+#endif
+#if !(defined(JF_DBG_MODE) && (JF_DBG_MODE == 6))
+        if (s + AHEAD < nstages) issue_stage(s + AHEAD);
+#endif
+
+        const unsigned char *base = smem + SLOT * STAGE_BYTES;
+        const float *sc_lds = reinterpret_cast<const float *>(scale_ring + SLOT * (SCALE_WORDS * 4));
+        const int kbs = (nkb - s * KB_STAGE) < KB_STAGE ? (nkb - s * KB_STAGE) : KB_STAGE;
+        auto compute_kb = [&](int kb) {
+            v4i a[WBM], b[WBN];
+#if defined(JF_DBG_MODE) && (JF_DBG_MODE == 1 || JF_DBG_MODE == 3)
+#pragma unroll
+            for (int i = 0; i < WBM; ++i) a[i] = v4i{lane, kb, i, 1};
+#pragma unroll
+            for (int j = 0; j < WBN; ++j) b[j] = v4i{lane, 2, j, kb};
+#else
+#pragma unroll
+            for (int i = 0; i < WBM; ++i)
+                a[i] = *reinterpret_cast<const v4i *>(base + i * (QB * ROW_BYTES) + fa_off[kb]);
+#pragma unroll
+            for (int j = 0; j < WBN; ++j)
+                b[j] = *reinterpret_cast<const v4i *>(base + A_BYTES + j * (QB * ROW_BYTES) + fb_off[kb]);
+#endif
+#if defined(JF_DBG_MODE) && (JF_DBG_MODE == 1 || JF_DBG_MODE == 2)
             if (EPI == EPI_S32) {
 #pragma unroll
-                for (int i = 0; i < 2; ++i)
+                for (int i = 0; i < WBM; ++i)
 #pragma unroll
-                    for (int j = 0; j < 2; ++j)
+                    for (int j = 0; j < WBN; ++j) { iacc[i][j][0] ^= a[i].x ^ b[j].y; iacc[i][j][1] ^= a[i].z ^ b[j].w; }
+            } else
+#endif
+            if (EPI == EPI_S32) {
+#pragma unroll
+                for (int i = 0; i < WBM; ++i)
+#pragma unroll
+                    for (int j = 0; j < WBN; ++j)
                         iacc[i][j] = __builtin_amdgcn_mfma_i32_32x32x32_i8(a[i], b[j], iacc[i][j], 0, 0, 0);
             } else {
-                float fa[2], fb[2];
+                float fa[WBM], fb[WBN];
+                int kbg = s * KB_STAGE + kb; kbg = kbg < nkb ? kbg : nkb - 1;
+                // binary16 scales arrive as the 32-bit word that holds them: the half to use is the parity of the
+                // scale's element index (wave-uniform)
+                auto scale_at = [&](int word, int elem) -> float {
+                    if (sizeof(ST) == 4) return sc_lds[word];
+                    const uint32_t w = __float_as_uint(sc_lds[word]);
+                    const uint16_t h = (elem & 1) ? (uint16_t)(w >> 16) : (uint16_t)w;
+                    return (float)__builtin_bit_cast(half_t, h);
+                };
 #pragma unroll
-                for (int i = 0; i < 2; ++i) {
-                    fa[i] = sc_lds[kb * 4 + wm * 2 + i];
-                    fb[i] = sc_lds[16 + kb * 4 + wn * 2 + i];
-                }
-                const v16i zero = {0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0};
+                for (int i = 0; i < WBM; ++i) fa[i] = scale_at(kb * 16 + wm * WBM + i, kbg * SM + mb[i]);
 #pragma unroll
-                for (int i = 0; i < 2; ++i)
+                for (int j = 0; j < WBN; ++j) fb[j] = scale_at(kb * 16 + BM / QB + wn * WBN + j, kbg * SN + nb[j]);
+                // The accumulator input is the bit pattern of 1.5*2^23: the INT32 result d + 0x4B400000, read as a
+                // float, IS 12582912.0 + d (|d| <= 32*127^2 < 2^22), so one exact fp32 subtraction replaces the
+                // slower integer-to-float conversion.  All products are issued before the first one is consumed,
+                // so the matrix pipe works while the vector ALU does the scale-accumulate.
+                v16i d[WBM][WBN];
 #pragma unroll
-                    for (int j = 0; j < 2; ++j) {
-                        const v16i d = __builtin_amdgcn_mfma_i32_32x32x32_i8(a[i], b[j], zero, 0, 0, 0);
+                for (int i = 0; i < WBM; ++i)
+#pragma unroll
+                    for (int j = 0; j < WBN; ++j)
+                        d[i][j] = __builtin_amdgcn_mfma_i32_32x32x32_i8(a[i], b[j], magic, 0, 0, 0);
+#pragma unroll
+                for (int i = 0; i < WBM; ++i)
+#pragma unroll
+                    for (int j = 0; j < WBN; ++j) {
                         const float sab = fa[i] * fb[j];
+                        float t[16];
 #pragma unroll
-                        for (int v = 0; v < 16; ++v)
-                            acc[i][j][v] = __builtin_fmaf(sab, (float)d[v], acc[i][j][v]);
+                        for (int v = 0; v < 16; ++v) t[v] = __int_as_float(d[i][j][v]) - 12582912.0f;
+#pragma unroll
+                        for (int v = 0; v < 16; ++v) acc[i][j][v] = __builtin_fmaf(sab, t[v], acc[i][j][v]);
                     }
             }
+        };
+#pragma unroll
+        for (int kb = 0; kb < KB_STAGE; ++kb)
+            if (kb < kbs) compute_kb(kb);                     // uniform; only the last stage can be short
+    });
+    __syncthreads();           // the epilogue reuses the ring as scratch
+#if defined(JF_DBG_MODE) && (JF_DBG_MODE >= 5)
+    {   // timing experiment: main loop only
+        for (int i = 0; i < WBM; ++i) for (int j = 0; j < WBN; ++j) for (int v = 0; v < 16; ++v) {
+            if (EPI == EPI_S32) asm volatile("" :: "v"(iacc[i][j][v])); else asm volatile("" :: "v"(acc[i][j][v]));
         }
-        if (s + 1 < nstages) store_stage((s + 1) & 1);
-        __syncthreads();
+        return;
     }
+#endif
 
     // ---- epilogue: one 32x32 block at a time through a wave-private LDS patch ------------------
     // MFMA result layout: lane l, register v  <->  row 8*(v/4) + 4*(l/32) + v%4, column l%32.
@@ -194,10 +324,10 @@ __global__ __launch_bounds__(NTHREADS, 2) void igemm_nt_kernel(GemmArgs p)
     const float biasmax = (EPI == EPI_Q && p.biasmax) ? p.biasmax[0] : 0.0f;
 
 #pragma unroll
-    for (int i = 0; i < 2; ++i)
+    for (int i = 0; i < WBM; ++i)
 #pragma unroll
-        for (int j = 0; j < 2; ++j) {
-            const int bm = m0 + (wm * 2 + i) * QB, bn = n0 + (wn * 2 + j) * QB;
+        for (int j = 0; j < WBN; ++j) {
+            const int bm = m0 + (wm * WBM + i) * QB, bn = n0 + (wn * WBN + j) * QB;
             const bool valid = bm < p.M && bn < p.N;          // wave-uniform
             float amax = 0.0f;
             if (EPI == EPI_Q) {
@@ -320,18 +450,39 @@ static int launch_transpose(const int8_t *in, int R, int C, int8_t *out, hipStre
     return (int)hipGetLastError();
 }
 
-template <int EPI, typename ST> static int launch_gemm(const GemmArgs &a, hipStream_t st)
+template <int EPI, typename ST, int WGM, int WGN, int NSTAGE, int WGPC>
+static int launch_gemm_cfg(const GemmArgs &a, hipStream_t st)
 {
+    constexpr int BM = QB * WBM * WGM, BN = QB * WBN * WGN, NT = 64 * WGM * WGN;
+    constexpr int RING = NSTAGE * (BM + BN) * ROW_BYTES + WGM * WGN * NSTAGE * 256;   // operand ring + per-wave scale patches
+    constexpr int PATCH = WGM * WGN * QB * EPI_LD * (int)sizeof(float);
+    constexpr int SMEM = RING > PATCH ? RING : PATCH;
     GemmArgs p = a;
     p.tiles_m = (p.M + BM - 1) / BM;
     p.tiles_n = (p.N + BN - 1) / BN;
-    auto kern = igemm_nt_kernel<EPI, ST>;
+    auto kern = igemm_nt_kernel<EPI, ST, WGM, WGN, NSTAGE, WGPC>;
     // more than 64 KiB of dynamic LDS has to be opted into, per function
-    hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void *>(kern), hipFuncAttributeMaxDynamicSharedMemorySize,
-                                       SMEM_BYTES);
+    hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void *>(kern), hipFuncAttributeMaxDynamicSharedMemorySize, SMEM);
     if (e != hipSuccess) return (int)e;
-    hipLaunchKernelGGL(kern, dim3(p.tiles_m * p.tiles_n), dim3(NTHREADS), SMEM_BYTES, st, p);
+    hipLaunchKernelGGL(kern, dim3(p.tiles_m * p.tiles_n), dim3(NT), SMEM, st, p);
     return (int)hipGetLastError();
+}
+
+// Tile configuration.  JF_GEMM_CFG selects it at build time (for experiments); the default is 128x128 tiles,
+// 8 waves, a 2-deep ring and two workgroups per CU (the epilogue of one overlaps the main loop of the other).
+#ifndef JF_GEMM_CFG
+#define JF_GEMM_CFG 0
+#endif
+template <int EPI, typename ST> static int launch_gemm(const GemmArgs &a, hipStream_t st)
+{
+#if JF_GEMM_CFG == 0
+    return launch_gemm_cfg<EPI, ST, 2, 4, 2, 2>(a, st);
+#else
+    // 256x128 or 128x256, whichever pads the problem less (1600 = 12.5 x 128 but 6.25 x 256); 16 waves, 3-deep ring
+    auto padded = [](long d, long t) { return (d + t - 1) / t * t; };
+    const long tall = padded(a.M, 256) * padded(a.N, 128), wide = padded(a.M, 128) * padded(a.N, 256);
+    return tall <= wide ? launch_gemm_cfg<EPI, ST, 4, 4, 3, 1>(a, st) : launch_gemm_cfg<EPI, ST, 2, 8, 3, 1>(a, st);
+#endif
 }
 
 static int check_gemm_common(const void *A, const void *B, const void *C, int M, int N, int K, int b_layout,
