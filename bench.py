@@ -24,6 +24,7 @@ for p in (ROOT, PKG):
         sys.path.insert(0, p)
 
 INT8_PEAK_TOPS = 5000.0      # MI355X dense INT8 MFMA peak, tera-ops/s
+MEASURED_TRAFFIC_BYTES = 152.9e6   # fc forward GEMM: 100.2 MB fetched + 52.8 MB written per launch (counter run)
 TOKENS = 8192
 LAYERS = [("qkv", 1600, 4800), ("proj", 1600, 1600), ("fc", 1600, 6400), ("fc2", 6400, 1600)]
 
@@ -83,7 +84,68 @@ def dominant_kernel_roofline(jf, torch, ops, iters=20):
     achieved = 2.0 * M * N * K / avg_s / 1e12
     return {"bound": "mfma", "kernel": "igemm_nt_kernel<EPI_Q,f32> fc forward 8192x6400x1600",
             "achieved": round(achieved, 2), "peak": INT8_PEAK_TOPS, "unit": "TOP/s",
-            "frac": round(achieved / INT8_PEAK_TOPS, 4), "avg_launch_us": round(avg_s * 1e6, 2), "traffic": None}
+            "frac": round(achieved / INT8_PEAK_TOPS, 4), "avg_launch_us": round(avg_s * 1e6, 2),
+            # HBM-side bytes per launch from rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE (profiles/igemm_fc_forward_pmc.md);
+            # algorithmic minimum is 75.9 MB (A + W + C)
+            "traffic": MEASURED_TRAFFIC_BYTES}
+
+
+def nonlinear_extras(jf, torch):
+    """Achieved GB/s (algorithmic bytes / event time) of the memory-bound kernels at the GPT-2 XL sizes of BASELINE
+    config 4 (LayerNorm on 8192x1600, GELU on 8192x6400), fp32 scales."""
+    def t(fn, n=30):
+        for _ in range(3):
+            fn()
+        e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+        e0.record()
+        for _ in range(n):
+            fn()
+        e1.record()
+        torch.cuda.synchronize()
+        return e0.elapsed_time(e1) * 1e-3 / n
+    g = torch.Generator().manual_seed(0)
+    S = torch.float32
+    out = {}
+    def put(name, secs, nbytes):
+        out[name] = {"GB/s": round(nbytes / secs / 1e9, 1), "us": round(secs * 1e6, 1), "frac_of_8TB/s": round(nbytes / secs / 8e12, 3)}
+    R, C = TOKENS, 1600
+    x = torch.randn(R, C, generator=g).cuda()
+    dy = (torch.randn(R, C, generator=g) * 1e-3).cuda()
+    gamma = (1 + 0.1 * torch.randn(C, generator=g)).cuda()
+    beta = (0.1 * torch.randn(C, generator=g)).cuda()
+    qx, sx = jf.quantize(x, scale_dtype=S)
+    qg, sg = jf.quantize(dy, jf.ROUND_STOCHASTIC, S, seed=0, offset=0)
+    mean, rstd = jf.rowstats(qx, sx)
+    n = R * C
+    put("quantize_f32_8192x1600", t(lambda: jf.quantize(x, scale_dtype=S)), 5 * n)
+    put("quantize_transpose_sr_8192x1600", t(lambda: jf.quantize(x, jf.ROUND_STOCHASTIC, S, transpose=True, seed=1, offset=0)), 6 * n)
+    put("transpose_8192x1600", t(lambda: jf.transpose_s8(qx)), 2 * n)
+    put("layernorm_fwd_8192x1600", t(lambda: jf.layernorm_fwd(qx, sx, gamma, beta, mean, rstd)), 2 * n)
+    put("layernorm_bwd_sr_8192x1600", t(lambda: jf.layernorm_bwd(qx, sx, qg, sg, gamma, mean, rstd, jf.ROUND_STOCHASTIC, seed=1, offset=0)), 3 * n)
+    R, C = TOKENS, 6400
+    x = torch.randn(R, C, generator=g).cuda()
+    dy = (torch.randn(R, C, generator=g) * 1e-3).cuda()
+    qx, sx = jf.quantize(x, scale_dtype=S)
+    qg, sg = jf.quantize(dy, jf.ROUND_STOCHASTIC, S, seed=0, offset=0)
+    n = R * C
+    put("gelu_fwd_tanh_8192x6400", t(lambda: jf.gelu_fwd(qx, sx, jf.GELU_TANH, 0.0)), 2 * n)
+    put("gelu_fwd_erf_8192x6400", t(lambda: jf.gelu_fwd(qx, sx, jf.GELU_ERF, 5e-5)), 2 * n)
+    put("gelu_bwd_tanh_sr_8192x6400", t(lambda: jf.gelu_bwd(qx, sx, qg, sg, jf.GELU_TANH, jf.ROUND_STOCHASTIC, seed=1, offset=0)), 3 * n)
+    put("gelu_bwd_erf_sr_8192x6400", t(lambda: jf.gelu_bwd(qx, sx, qg, sg, jf.GELU_ERF, jf.ROUND_STOCHASTIC, seed=1, offset=0)), 3 * n)
+    return out
+
+
+def pmc_probe(jf, torch, ops):
+    """For counter runs (rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE): one device copy of known size (256 MiB read,
+    256 MiB written: the calibration kernel) followed by three launches of the dominant GEMM, and nothing else."""
+    buf = torch.empty(256 << 20, dtype=torch.uint8, device="cuda")
+    dst = torch.empty_like(buf)
+    torch.cuda.synchronize()
+    dst.copy_(buf)
+    o = ops[2]
+    for _ in range(3):
+        jf.igemm_block_q(o["qx"], o["qw"], o["sxT"], o["swT"], jf.B_NK)
+    torch.cuda.synchronize()
 
 
 def cpu_baseline(ops, rows=512):
@@ -116,6 +178,9 @@ def main():
     ap.add_argument("--warmup", type=int, default=3)
     ap.add_argument("--cpu-rows", type=int, default=8192)
     ap.add_argument("--no-cpu", action="store_true")
+    ap.add_argument("--no-extras", action="store_true")
+    ap.add_argument("--pmc-probe", action="store_true", help="copy kernel + 3 GEMM launches only (for rocprofv3 --pmc)")
+    ap.add_argument("--roofline-only", action="store_true", help="only the dominant-kernel measurement (for rocprofv3 --stats)")
     a = ap.parse_args()
     if a.gpus != 1:
         sys.exit("bench.py: this build measures one GPU only (--gpus 1); nothing here uses a second GPU")
@@ -127,6 +192,12 @@ def main():
         sys.exit("bench.py: no GPU visible")
     torch.cuda.set_device(0)
     ops = make_inputs(jf, torch)
+    if a.pmc_probe:
+        pmc_probe(jf, torch, ops)
+        return
+    if a.roofline_only:
+        print(json.dumps({"roofline": dominant_kernel_roofline(jf, torch, ops)}))
+        return
 
     for i in range(a.warmup):
         step(jf, torch, ops, i)
@@ -155,6 +226,8 @@ def main():
                    "event_ms_per_step": round(e0.elapsed_time(e1) / a.steps, 4)},
         "roofline": roof,
     }
+    if not a.no_extras:
+        out["memory_bound_kernels"] = nonlinear_extras(jf, torch)
     if not a.no_cpu:
         out["cpu_baseline"] = cpu_baseline(ops, a.cpu_rows)
     print(json.dumps(out))

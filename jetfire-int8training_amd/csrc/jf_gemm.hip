@@ -75,9 +75,10 @@ template <int I, int N, typename F> __device__ __forceinline__ void static_for(F
 
 // WGM x WGN waves, each owning WBM x WBN quantisation blocks (64x32 elements).
 constexpr int WBM = 2, WBN = 1;
-// NSTAGE = depth of the LDS ring (one stage being computed, NSTAGE-1 in flight); WGPC = workgroups per CU.
+// NSTAGE = depth of the LDS ring (one stage being computed, NSTAGE-1 in flight); WGPC = workgroups per CU
+// (the second launch bound counts waves per SIMD: WGPC workgroups of WGM*WGN waves over 4 SIMDs).
 template <int EPI, typename ST, int WGM, int WGN, int NSTAGE, int WGPC>
-__global__ __launch_bounds__(64 * WGM * WGN, WGPC) void igemm_nt_kernel(GemmArgs p)
+__global__ __launch_bounds__(64 * WGM * WGN, WGPC * WGM * WGN / 4) void igemm_nt_kernel(GemmArgs p)
 {
     constexpr int NW = WGM * WGN;
     constexpr int BM = QB * WBM * WGM, BN = QB * WBN * WGN;
