@@ -232,27 +232,46 @@ __global__ __launch_bounds__(NT) void rowstats_kernel(const int8_t *q, const ST 
     }
 }
 
-// LayerNorm backward, pass 1.  One workgroup per 32-row strip.  Per row: 16-column partial sums of
-// xhat*wdy (fmaf chain) and wdy (add chain), then all C/16 partials added in ascending order by one
-// lane per row -> c1 = sum/C, c2 = sum/C.  Also the strip's column sums of dy*xhat and dy
-// (partial dgamma / dbeta, reduced over strips by colsum_kernel).
-template <typename ST>
-__global__ __launch_bounds__(NT) void layernorm_bwd_stats_kernel(const int8_t *qx, const ST *sx, const int8_t *qg,
-                                                                 const ST *sg, const float *gamma, const float *mean,
-                                                                 const float *rstd, int R, int C, float *c1, float *c2,
-                                                                 float *pdg, float *pdb)
+// Sum of 32 per-lane values over the 32 lanes that share (lane & 1): a halving butterfly over lane bits 5..1.
+// On return lane l holds the total of value index  ((l>>5)&1)*16 + ((l>>4)&1)*8 + ((l>>3)&1)*4 + ((l>>2)&1)*2 + ((l>>1)&1).
+__device__ __forceinline__ float reduce32_over_rows(float (&v)[32], int lane)
 {
-    extern __shared__ float fsm[];                // part1[32][C/16], part2[32][C/16], patch[4][2][32][33]
+#define JF_BFLY(N, MASK)                                                   \
+    {                                                                      \
+        const bool up = (lane & (MASK)) != 0;                              \
+        _Pragma("unroll") for (int i = 0; i < (N) / 2; ++i) {              \
+            const float send = up ? v[i] : v[(N) / 2 + i];                 \
+            const float keep = up ? v[(N) / 2 + i] : v[i];                 \
+            v[i] = keep + __shfl_xor(send, (MASK), WAVE);                  \
+        }                                                                  \
+    }
+    JF_BFLY(32, 32) JF_BFLY(16, 16) JF_BFLY(8, 8) JF_BFLY(4, 4) JF_BFLY(2, 2)
+#undef JF_BFLY
+    return v[0];
+}
+
+// LayerNorm backward, pass 1.  One workgroup (16 waves) per 32-row strip; the waves take the column blocks
+// round-robin.  Per row: 16-column partial sums of xhat*wdy (fmaf chain) and wdy (add chain) go to LDS, then one
+// lane per row adds all C/16 partials in ascending order -> c1 = sum/C, c2 = sum/C (a defined order, so the
+// requantised dx is bit-reproducible).  Also the strip's column sums of dy*xhat and dy (partial dgamma / dbeta,
+// reduced over strips by colsum_kernel), by a butterfly over the 32 rows of the block.
+constexpr int LNB_THREADS = 1024;
+template <typename ST>
+__global__ __launch_bounds__(LNB_THREADS) void layernorm_bwd_stats_kernel(const int8_t *qx, const ST *sx, const int8_t *qg,
+                                                                          const ST *sg, const float *gamma, const float *mean,
+                                                                          const float *rstd, int R, int C, float *c1, float *c2,
+                                                                          float *pdg, float *pdb)
+{
+    extern __shared__ float fsm[];                // part1[32][C/16], part2[32][C/16]
     const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
     const int SC = C / QB, H = C / 16, rb = blockIdx.x;
     float *part1 = fsm, *part2 = fsm + QB * H;
-    float *patch = fsm + 2 * QB * H + wave * (2 * QB * 33);
     const int r = lane >> 1;
     const float mu = mean[rb * QB + r], rs = rstd[rb * QB + r];
-    for (int cb = wave; cb < SC; cb += WPB) {
+    for (int cb = wave; cb < SC; cb += LNB_THREADS / WAVE) {
         const int col = cb * QB + (lane & 1) * 16;
         const size_t e0 = (size_t)(rb * QB + r) * C + col;
-        float x[16], g[16], w[16];
+        float x[16], g[16], w[16], v[32];
         unpack16(*reinterpret_cast<const v4i *>(qx + e0), load_scale(sx, rb * SC + cb), x);
         unpack16(*reinterpret_cast<const v4i *>(qg + e0), load_scale(sg, rb * SC + cb), g);
         Load16<float>::run(gamma + col, w);
@@ -263,23 +282,17 @@ __global__ __launch_bounds__(NT) void layernorm_bwd_stats_kernel(const int8_t *q
             const float wdy = w[k] * g[k];
             p1 = __builtin_fmaf(xh, wdy, p1);
             p2 = p2 + wdy;
-            patch[r * 33 + (lane & 1) * 16 + k] = g[k] * xh;
-            patch[QB * 33 + r * 33 + (lane & 1) * 16 + k] = g[k];
+            v[k] = g[k] * xh;
+            v[16 + k] = g[k];
         }
         part1[r * H + cb * 2 + (lane & 1)] = p1;
         part2[r * H + cb * 2 + (lane & 1)] = p2;
         if (pdg) {
-            __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
-            __builtin_amdgcn_wave_barrier();
-            __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
-            const float *src = patch + (lane >> 5) * (QB * 33) + (lane & 31);
-            float acc = 0.0f;
-#pragma unroll
-            for (int k = 0; k < QB; ++k) acc += src[k * 33];
-            float *dst = (lane >> 5) ? pdb : pdg;
-            dst[(size_t)rb * C + cb * QB + (lane & 31)] = acc;
-            __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
-            __builtin_amdgcn_wave_barrier();
+            const float total = reduce32_over_rows(v, lane);
+            const int idx = ((lane >> 5) & 1) * 16 + ((lane >> 4) & 1) * 8 + ((lane >> 3) & 1) * 4 + ((lane >> 2) & 1) * 2 +
+                            ((lane >> 1) & 1);
+            float *dst = (idx & 16) ? pdb : pdg;
+            dst[(size_t)rb * C + cb * QB + (lane & 1) * 16 + (idx & 15)] = total;
         }
     }
     __syncthreads();
@@ -321,14 +334,24 @@ __global__ __launch_bounds__(NT) void layernorm_bwd_dx_kernel(const int8_t *qx, 
     }
 }
 
-// out[c] = sum over strips of part[strip][c]   (layernorm.py:405-428)
-__global__ __launch_bounds__(NT) void colsum_kernel(const float *part, int strips, int C, float *out)
+// out[c] = sum over strips of part[strip][c]   (layernorm.py:405-428).  64 columns per workgroup, 16 strip lanes
+// per column (fixed partition and a fixed tree, so the result is reproducible).
+__global__ __launch_bounds__(1024) void colsum_kernel(const float *part, int strips, int C, float *out)
 {
-    const int c = blockIdx.x * NT + threadIdx.x;
-    if (c >= C) return;
+    __shared__ float red[16][65];
+    const int tx = threadIdx.x & 63, ty = threadIdx.x >> 6;
+    const int c = blockIdx.x * 64 + tx;
     float a = 0.0f;
-    for (int i = 0; i < strips; ++i) a += part[(size_t)i * C + c];
-    out[c] = a;
+    if (c < C)
+        for (int i = ty; i < strips; i += 16) a += part[(size_t)i * C + c];
+    red[ty][tx] = a;
+    __syncthreads();
+    if (ty == 0 && c < C) {
+        float t = 0.0f;
+#pragma unroll
+        for (int k = 0; k < 16; ++k) t += red[k][tx];
+        out[c] = t;
+    }
 }
 
 // add.py:29-162 / add_mean_var.py:28-177
@@ -480,8 +503,8 @@ int jf_layernorm_bwd(const int8_t *qx, const void *sx, const int8_t *qg, const v
     if (!aligned16(qdx) || !aligned16(gamma)) return JF_ERR_ALIGN;
     if (!workspace || workspace_bytes < jf_layernorm_bwd_workspace_bytes(R, C)) return JF_ERR_WORKSPACE;
     if (!aligned16(workspace)) return JF_ERR_ALIGN;
-    const size_t smem = ((size_t)2 * QB * (C / 16) + (size_t)WPB * 2 * QB * 33) * sizeof(float);
-    if (smem > 64 * 1024) return JF_ERR_SHAPE;
+    const size_t smem = (size_t)2 * QB * (C / 16) * sizeof(float);
+    if (smem > 64 * 1024) return JF_ERR_SHAPE;                 // rows of up to 4096 columns
     hipStream_t st = (hipStream_t)stream;
     float *c1 = (float *)workspace, *c2 = c1 + R;
     const bool want_dw = dgamma || dbeta;
@@ -489,7 +512,7 @@ int jf_layernorm_bwd(const int8_t *qx, const void *sx, const int8_t *qg, const v
     const int grid = grid_for_blocks(R, C);
 #define JF_LNB(ST)                                                                                                   \
     do {                                                                                                             \
-        hipLaunchKernelGGL(layernorm_bwd_stats_kernel<ST>, dim3(R / QB), dim3(NT), smem, st, qx, (const ST *)sx, qg,   \
+        hipLaunchKernelGGL(layernorm_bwd_stats_kernel<ST>, dim3(R / QB), dim3(LNB_THREADS), smem, st, qx, (const ST *)sx, qg, \
                            (const ST *)sg, gamma, mean, rstd, R, C, c1, c2, pdg, pdb);                               \
         hipLaunchKernelGGL(layernorm_bwd_dx_kernel<ST>, dim3(grid), dim3(NT), 0, st, qx, (const ST *)sx, qg,          \
                            (const ST *)sg, gamma, mean, rstd, c1, c2, R, C, rounding, seed, offset, qdx, (ST *)sdx);  \
@@ -497,8 +520,8 @@ int jf_layernorm_bwd(const int8_t *qx, const void *sx, const int8_t *qg, const v
     if (scale_dtype == JF_SCALE_F16) JF_LNB(half_t);
     else JF_LNB(float);
 #undef JF_LNB
-    if (dgamma) hipLaunchKernelGGL(colsum_kernel, dim3((C + NT - 1) / NT), dim3(NT), 0, st, pdg, R / QB, C, dgamma);
-    if (dbeta) hipLaunchKernelGGL(colsum_kernel, dim3((C + NT - 1) / NT), dim3(NT), 0, st, pdb, R / QB, C, dbeta);
+    if (dgamma) hipLaunchKernelGGL(colsum_kernel, dim3((C + 63) / 64), dim3(1024), 0, st, pdg, R / QB, C, dgamma);
+    if (dbeta) hipLaunchKernelGGL(colsum_kernel, dim3((C + 63) / 64), dim3(1024), 0, st, pdb, R / QB, C, dbeta);
     return (int)hipGetLastError();
 }
 
