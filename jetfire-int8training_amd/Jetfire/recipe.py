@@ -1,0 +1,169 @@
+"""INT8 data-flow transformer block built on the Linear / Nonlinear operators.
+
+Counterpart of the autograd Functions of the reference recipe (INT8_GPT2/qmodel.py:86-171 attention,
+:190-268 MLP, :295-363 model begin/end): between Functions an activation travels as the triple
+(fp residual, INT8 codes, per-block scales [, row mean, row rstd]) and a gradient as (fp residual grad, INT8 codes,
+scales).  Autograd only carries floating tensors, so the INT8 codes cross Function boundaries re-viewed as
+float8_e4m3fn (same bytes), exactly as the reference does (qmodel.py:131,153,230,266).
+
+Linear biases are not part of the data flow (the reference ignores them as well); LayerNorm has a weight only.
+"""
+import torch
+import torch.nn as nn
+import torch.nn.functional as F
+
+from Linear import int8_linear_backward, int8_linear_forward
+from Nonlinear import (int8_add_Ifp_Ig16_Ofp_Og, int8_add_Ifp_Ig16_Ofp_Og_MeanVar, int8_gelu_backward, int8_gelu_forward,
+                       int8_layernorm_backward, int8_layernorm_forward, int8_quantize, int8_quantize_transpose,
+                       int8_transpose)
+
+QB = 32
+_F8 = torch.float8_e4m3fn
+
+
+def _as_f8(q):
+    return q.view(_F8)
+
+
+def _as_s8(q):
+    return q.view(torch.int8)
+
+
+class StreamBegin(torch.autograd.Function):
+    """fp activation -> (fp, codes, scales).  Gradient: the fp gradient passes through (qmodel.py:309-327)."""
+
+    @staticmethod
+    def forward(ctx, x):
+        q, s = int8_quantize(x, QB)
+        return x, _as_f8(q), s
+
+    @staticmethod
+    def backward(ctx, g, _qg, _sg):
+        return g
+
+
+class StreamEnd(torch.autograd.Function):
+    """(fp, codes, scales) -> fp.  Gradient: the fp gradient plus its stochastic block quantisation
+    (qmodel.py:343-362)."""
+
+    @staticmethod
+    def forward(ctx, x, qx, sx):
+        return x
+
+    @staticmethod
+    def backward(ctx, g):
+        qg, sg = int8_quantize(g.contiguous(), QB, stochastic=True)
+        return g, _as_f8(qg), sg
+
+
+class AttentionIn(torch.autograd.Function):
+    """LayerNorm -> QKV projection, fp16 out for the attention kernel (qmodel.py:86-131)."""
+
+    @staticmethod
+    def forward(ctx, residual, qx, sx, w_qkv, ln_w, mean, rstd):
+        qw, sw = int8_quantize(w_qkv, QB)
+        qx = _as_s8(qx)
+        qn, sn, _ = int8_layernorm_forward(qx, sx, ln_w, mean, rstd, QB)
+        qkv = int8_linear_forward(qn, sn, qw, sw, False, QB)
+        ctx.save_for_backward(qx, sx, qn, sn, qw, sw, ln_w, mean, rstd)
+        return residual, qkv
+
+    @staticmethod
+    def backward(ctx, fpg, g):
+        qx, sx, qn, sn, qw, sw, ln_w, mean, rstd = ctx.saved_tensors
+        qg, sg, qgt = int8_quantize_transpose(g.contiguous(), QB, stochastic=True, transpose_output_2d=True)
+        qg, sg, gw = int8_linear_backward(qn, sn, qg, sg, qgt, qw, sw, QB, stochastic=True)
+        qg, sg, g_ln = int8_layernorm_backward(qx, sx, qg, sg, ln_w, QB, mean, rstd, stochastic=True)
+        res_g, qg, sg = int8_add_Ifp_Ig16_Ofp_Og(fpg.contiguous(), qg, sg, QB, stochastic=True)
+        return res_g, _as_f8(qg), sg, gw, g_ln, None, None
+
+
+class AttentionOut(torch.autograd.Function):
+    """Output projection + residual add, producing the statistics of the next LayerNorm (qmodel.py:134-171)."""
+
+    @staticmethod
+    def forward(ctx, residual, y, w_proj):
+        qw, sw = int8_quantize(w_proj, QB)
+        qy, sy = int8_quantize(y.contiguous(), QB)
+        qo, so = int8_linear_forward(qy, sy, qw, sw, True, QB)
+        fp, q, s, mean, rstd = int8_add_Ifp_Ig16_Ofp_Og_MeanVar(residual.contiguous(), qo, so, QB)
+        ctx.save_for_backward(qy, sy, qw, sw)
+        return fp, _as_f8(q), s, mean, rstd
+
+    @staticmethod
+    def backward(ctx, fpg, qg, sg, _m, _r):
+        qy, sy, qw, sw = ctx.saved_tensors
+        qg = _as_s8(qg)
+        qgt = int8_transpose(qg, transpose_output_2d=True)
+        g, gw = int8_linear_backward(qy, sy, qg, sg, qgt, qw, sw, QB, stochastic=True, dgrad_quantize=False)
+        return fpg, g, gw
+
+
+class MLPResidual(torch.autograd.Function):
+    """LayerNorm -> fc -> GELU -> proj -> residual add, all on INT8 block tensors (qmodel.py:190-268)."""
+
+    @staticmethod
+    def forward(ctx, residual, qx, sx, w_fc, w_proj, ln_w, mean, rstd):
+        qx = _as_s8(qx)
+        qw1, sw1 = int8_quantize(w_fc, QB)
+        qw2, sw2 = int8_quantize(w_proj, QB)
+        qn, sn, _ = int8_layernorm_forward(qx, sx, ln_w, mean, rstd, QB)
+        qh, sh = int8_linear_forward(qn, sn, qw1, sw1, True, QB)
+        qa, sa = int8_gelu_forward(qh, sh, QB)
+        qo, so = int8_linear_forward(qa, sa, qw2, sw2, True, QB)
+        fp, q, s, mean2, rstd2 = int8_add_Ifp_Ig16_Ofp_Og_MeanVar(residual.contiguous(), qo, so, QB)
+        ctx.save_for_backward(qx, sx, qn, sn, qh, sh, qa, sa, qw1, sw1, qw2, sw2, ln_w, mean, rstd)
+        return fp, _as_f8(q), s, mean2, rstd2
+
+    @staticmethod
+    def backward(ctx, fpg, qg, sg, _m, _r):
+        qx, sx, qn, sn, qh, sh, qa, sa, qw1, sw1, qw2, sw2, ln_w, mean, rstd = ctx.saved_tensors
+        qg = _as_s8(qg)
+        qgt = int8_transpose(qg, transpose_output_2d=True)
+        qg, sg, gw2 = int8_linear_backward(qa, sa, qg, sg, qgt, qw2, sw2, QB, stochastic=True)
+        qg, sg = int8_gelu_backward(qh, sh, qg, sg, QB, stochastic=True)
+        qgt = int8_transpose(qg, transpose_output_2d=True)
+        qg, sg, gw1 = int8_linear_backward(qn, sn, qg, sg, qgt, qw1, sw1, QB, stochastic=True)
+        qg, sg, g_ln = int8_layernorm_backward(qx, sx, qg, sg, ln_w, QB, mean, rstd, stochastic=True)
+        res_g, qg, sg = int8_add_Ifp_Ig16_Ofp_Og(fpg.contiguous(), qg, sg, QB, stochastic=True)
+        return res_g, _as_f8(qg), sg, gw1, gw2, g_ln, None, None
+
+
+class QBlock(nn.Module):
+    """One pre-LayerNorm transformer block (causal self-attention + MLP) on the INT8 data flow."""
+
+    def __init__(self, n_embd, n_head):
+        super().__init__()
+        assert n_embd % n_head == 0 and n_embd % QB == 0
+        self.n_embd, self.n_head = n_embd, n_head
+        self.ln_1 = nn.Parameter(torch.ones(n_embd))
+        self.ln_2 = nn.Parameter(torch.ones(n_embd))
+        self.w_qkv = nn.Parameter(torch.randn(3 * n_embd, n_embd) * 0.02)
+        self.w_attn_proj = nn.Parameter(torch.randn(n_embd, n_embd) * 0.02)
+        self.w_fc = nn.Parameter(torch.randn(4 * n_embd, n_embd) * 0.02)
+        self.w_mlp_proj = nn.Parameter(torch.randn(n_embd, 4 * n_embd) * 0.02)
+
+    def forward(self, x, qx, sx, mean, rstd):
+        B, T, C = x.shape
+        res, qkv = AttentionIn.apply(x, qx, sx, self.w_qkv, self.ln_1, mean, rstd)
+        q, k, v = (t.view(B, T, self.n_head, C // self.n_head).transpose(1, 2) for t in qkv.split(C, dim=2))
+        y = F.scaled_dot_product_attention(q, k, v, is_causal=True).transpose(1, 2).contiguous().view(B, T, C)
+        x, qx, sx, mean, rstd = AttentionOut.apply(res, y, self.w_attn_proj)
+        return MLPResidual.apply(x, qx, sx, self.w_fc, self.w_mlp_proj, self.ln_2, mean, rstd)
+
+
+class QStack(nn.Module):
+    """A stack of QBlocks between StreamBegin and StreamEnd: fp in, fp out (qmodel.py:418-446 without the
+    embedding and the language-model head)."""
+
+    def __init__(self, n_layer, n_embd, n_head):
+        super().__init__()
+        self.blocks = nn.ModuleList(QBlock(n_embd, n_head) for _ in range(n_layer))
+
+    def forward(self, x):
+        x, qx, sx = StreamBegin.apply(x)
+        mean = x.float().mean(dim=-1)
+        rstd = torch.rsqrt(x.float().var(dim=-1, unbiased=False))
+        for blk in self.blocks:
+            x, qx, sx, mean, rstd = blk(x, qx, sx, mean, rstd)
+        return StreamEnd.apply(x, qx, sx)

@@ -189,6 +189,9 @@ __global__ __launch_bounds__(64 * WGM * WGN, WGPC * WGM * WGN / 4) void igemm_nt
         }
     // 1.5*2^23 as an integer bit pattern in 16 registers: the accumulator INPUT of every product (see below).
     // Written through asm so that the compiler keeps the registers instead of re-creating the constant.
+    // -1.5*2^23 in a scalar register: as a literal it would double the size of every v_add_f32 that uses it
+    float neg_magic;
+    asm volatile("s_mov_b32 %0, 0xcb400000" : "=s"(neg_magic));
     v16i magic;
 #pragma unroll
     for (int v = 0; v < 16; ++v) {
@@ -289,7 +292,11 @@ __global__ __launch_bounds__(64 * WGM * WGN, WGPC * WGM * WGN / 4) void igemm_nt
                 for (int i = 0; i < WBM; ++i)
 #pragma unroll
                     for (int j = 0; j < WBN; ++j)
+#ifdef JF_ZERO_C
+                        { const v16i z = {0,0,0,0,0,0,0,0,0,0,0,0,0,0,0,0}; d[i][j] = __builtin_amdgcn_mfma_i32_32x32x32_i8(a[i], b[j], z, 0, 0, 0); }
+#else
                         d[i][j] = __builtin_amdgcn_mfma_i32_32x32x32_i8(a[i], b[j], magic, 0, 0, 0);
+#endif
 #pragma unroll
                 for (int i = 0; i < WBM; ++i)
 #pragma unroll
@@ -297,7 +304,11 @@ __global__ __launch_bounds__(64 * WGM * WGN, WGPC * WGM * WGN / 4) void igemm_nt
                         const float sab = fa[i] * fb[j];
                         float t[16];
 #pragma unroll
-                        for (int v = 0; v < 16; ++v) t[v] = __int_as_float(d[i][j][v]) - 12582912.0f;
+#ifdef JF_ZERO_C
+                        for (int v = 0; v < 16; ++v) t[v] = (float)d[i][j][v];
+#else
+                        for (int v = 0; v < 16; ++v) t[v] = __int_as_float(d[i][j][v]) + neg_magic;
+#endif
 #pragma unroll
                         for (int v = 0; v < 16; ++v) acc[i][j][v] = __builtin_fmaf(sab, t[v], acc[i][j][v]);
                     }

@@ -1,0 +1,71 @@
+"""End-to-end check of the operator sequence of the INT8 GPT-2 recipe (our counterpart of the autograd
+Functions of INT8_GPT2/qmodel.py) against an fp32 torch transformer block: outputs and gradients agree within
+quantisation noise, and a small stack trains."""
+import pytest
+import torch
+import torch.nn.functional as F
+
+pytestmark = pytest.mark.gpu
+
+
+def ref_block(x, blk):
+    C = x.shape[-1]
+    B, T, _ = x.shape
+    h = F.layer_norm(x, (C,), blk.ln_1, None, 0.0)
+    qkv = h @ blk.w_qkv.t()
+    q, k, v = (t.view(B, T, blk.n_head, C // blk.n_head).transpose(1, 2) for t in qkv.split(C, dim=2))
+    y = F.scaled_dot_product_attention(q, k, v, is_causal=True).transpose(1, 2).contiguous().view(B, T, C)
+    x = x + y @ blk.w_attn_proj.t()
+    h = F.layer_norm(x, (C,), blk.ln_2, None, 0.0)
+    return x + F.gelu(h @ blk.w_fc.t()) @ blk.w_mlp_proj.t()
+
+
+def cos(a, b):
+    return float(F.cosine_similarity(a.detach().reshape(-1).float(), b.detach().reshape(-1).float(), dim=0))
+
+
+def test_one_block_matches_fp32_reference():
+    from recipe import QStack
+    torch.manual_seed(0)
+    B, T, C, H = 2, 64, 128, 4
+    model = QStack(1, C, H).cuda()
+    with torch.no_grad():
+        for p in model.parameters():
+            if p.dim() == 1:
+                p.add_(0.1 * torch.randn_like(p))
+    x = torch.randn(B, T, C, device="cuda", requires_grad=True)
+    w = torch.randn(B, T, C, device="cuda")
+    out = model(x)
+    assert out.shape == x.shape and out.dtype == torch.float32
+    (out * w).sum().backward()
+    got = {n: p.grad.clone() for n, p in model.named_parameters()}
+    gx = x.grad.clone()
+    for p in model.parameters():
+        p.grad = None
+    x2 = x.detach().clone().requires_grad_(True)
+    ref = ref_block(x2, model.blocks[0])
+    (ref * w).sum().backward()
+    assert cos(out, ref) > 0.999
+    assert cos(gx, x2.grad) > 0.99
+    for n, p in model.named_parameters():
+        assert got[n].shape == p.shape and got[n].dtype == p.dtype
+        assert cos(got[n], p.grad) > 0.97, n
+
+
+def test_small_stack_trains():
+    from recipe import QStack
+    torch.manual_seed(1)
+    B, T, C, H = 2, 64, 128, 4
+    model = QStack(2, C, H).cuda()
+    opt = torch.optim.AdamW(model.parameters(), lr=3e-3)
+    x = torch.randn(B, T, C, device="cuda")
+    target = torch.roll(x, 1, dims=1) * 0.5 + 0.1
+    losses = []
+    for _ in range(20):
+        opt.zero_grad(set_to_none=True)
+        loss = F.mse_loss(model(x), target)
+        loss.backward()
+        opt.step()
+        losses.append(float(loss))
+    assert losses[-1] < 0.8 * losses[0], losses
+    assert all(torch.isfinite(p).all() for p in model.parameters())
