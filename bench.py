@@ -135,6 +135,23 @@ def nonlinear_extras(jf, torch):
     return out
 
 
+def calibration(jf, torch):
+    """Register-only loops: what the matrix pipe and the vector ALU deliver alone and together on this part."""
+    simds = torch.cuda.get_device_properties(0).multi_processor_count * 4
+    out = {}
+    t, n = jf.calibrate(1, 0)
+    out["mfma_only_TOPs"] = round(n * 65536 / t / 1e12, 1)
+    out["mfma_only_ns_per_mfma_per_simd"] = round(t * 1e9 * simds / n, 2)
+    t, n = jf.calibrate(0, 32)
+    out["valu_32fmac_ns_per_simd"] = round(t * 1e9 * simds / n, 2)
+    t, n = jf.calibrate(1, 32)
+    out["mfma_plus_32fmac_ns_per_simd"] = round(t * 1e9 * simds / n, 2)
+    out["mfma_plus_32fmac_TOPs"] = round(n * 65536 / t / 1e12, 1)
+    out["note"] = ("per SIMD, 4 waves resident; the scale-accumulate needs 32 VALU instructions per MFMA, and the two "
+                   "pipes add up rather than overlap: the last line is the ceiling of any exact per-block kernel")
+    return out
+
+
 def pmc_probe(jf, torch, ops):
     """For counter runs (rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE): one device copy of known size (256 MiB read,
     256 MiB written: the calibration kernel) followed by three launches of the dominant GEMM, and nothing else."""
@@ -227,6 +244,7 @@ def main():
         "roofline": roof,
     }
     if not a.no_extras:
+        out["calibration"] = calibration(jf, torch)
         out["memory_bound_kernels"] = nonlinear_extras(jf, torch)
     if not a.no_cpu:
         out["cpu_baseline"] = cpu_baseline(ops, a.cpu_rows)

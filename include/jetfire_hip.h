@@ -147,6 +147,12 @@ int jf_add(const void *x1, int x1_dtype, const int8_t *q2, const void *s2, int R
            int scale_dtype, int rounding, uint64_t seed, uint64_t offset,
            float *y1, int8_t *q, void *s, float *rowsum, float *rowsq, jf_stream_t stream);
 
+/* Calibration (no counterpart in the reference; used by bench.py for the roofline discussion): launches
+ * `workgroups` x 256 threads, each wave doing `iters` x 4 x ( [one 32x32x32 INT8 MFMA if with_mfma] + [valu_per_mfma
+ * independent v_fmac_f32] ) from registers.  Supported (with_mfma, valu_per_mfma): (1,0) (0,32) (1,32) (0,16) (1,16).
+ * `scratch` is a device buffer of at least 4 bytes (never written in practice). */
+int jf_calibrate(int with_mfma, int valu_per_mfma, int iters, int workgroups, float *scratch, jf_stream_t stream);
+
 #ifdef __cplusplus
 }
 #endif

@@ -18,7 +18,7 @@ CSRC = os.path.join(HERE, "csrc")
 HIP_LIB = os.path.join(HERE, "libjetfire_hip.so")
 ROCM = os.environ.get("ROCM_PATH", "/opt/rocm")
 
-HIP_SOURCES = ["jf_gemm.hip", "jf_blockops.hip"]
+HIP_SOURCES = ["jf_gemm.hip", "jf_blockops.hip", "jf_calib.hip"]
 HIP_FLAGS = [
     "--offload-arch=gfx950", "-O3", "-std=c++17", "-fPIC", "-shared",
     "-ffp-contract=off",                                         # roundings are exactly the ones written

@@ -25,7 +25,7 @@ GELU_ERF, GELU_TANH = 0, 1
 EXPORTS = [
     "jf_error_string", "jf_igemm_workspace_bytes", "jf_igemm_s32", "jf_igemm_block_acc", "jf_igemm_block_fp",
     "jf_igemm_block_q", "jf_quantize", "jf_dequantize", "jf_transpose_s8", "jf_rowstats", "jf_layernorm_fwd",
-    "jf_layernorm_bwd_workspace_bytes", "jf_layernorm_bwd", "jf_gelu_fwd", "jf_gelu_bwd", "jf_add",
+    "jf_layernorm_bwd_workspace_bytes", "jf_layernorm_bwd", "jf_gelu_fwd", "jf_gelu_bwd", "jf_add", "jf_calibrate",
 ]
 
 _lib = None
@@ -58,6 +58,7 @@ def lib():
         L.jf_gelu_fwd.argtypes = [_p, _p, _i, _i, _i, _i, _f, _p, _p, _p]
         L.jf_gelu_bwd.argtypes = [_p, _p, _p, _p, _i, _i, _i, _i, _i, _u64, _u64, _p, _p, _p]
         L.jf_add.argtypes = [_p, _i, _p, _p, _i, _i, _i, _i, _u64, _u64, _p, _p, _p, _p, _p, _p]
+        L.jf_calibrate.argtypes = [_i, _i, _i, _i, _p, _p]
         missing = [name for name in EXPORTS if not hasattr(L, name)]
         if missing:
             raise RuntimeError(f"{LIB_PATH} does not export {missing}")
@@ -338,3 +339,20 @@ def add(x1, q2, s2, rounding=ROUND_TRUNC, with_stats=False, seed=None, offset=No
     check(lib().jf_add(_ptr(x1), _FP_CODE[x1.dtype], _ptr(q2), _ptr(s2), R, Cc, code, rounding, seed, offset,
                        _ptr(y1), _ptr(q), _ptr(s), _ptr(rs), _ptr(rq), _stream()))
     return (y1, q, s, rs, rq) if with_stats else (y1, q, s)
+
+
+def calibrate(with_mfma, valu_per_mfma, iters=2000, workgroups_per_cu=4):
+    """Seconds per launch of the register-only calibration kernel and the number of MFMA-sized work items it ran
+    (workgroups * 4 waves * iters * 4)."""
+    cus = torch.cuda.get_device_properties(0).multi_processor_count
+    wgs = cus * workgroups_per_cu
+    scratch = torch.zeros(16, dtype=torch.float32, device="cuda")
+    run = lambda: check(lib().jf_calibrate(with_mfma, valu_per_mfma, iters, wgs, _ptr(scratch), _stream()))
+    run()
+    e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+    e0.record()
+    for _ in range(3):
+        run()
+    e1.record()
+    torch.cuda.synchronize()
+    return e0.elapsed_time(e1) * 1e-3 / 3, wgs * 4 * iters * 4
