@@ -19,6 +19,8 @@
 
 #include <type_traits>
 
+#pragma clang diagnostic ignored "-Winline-asm"     // M0 appears in clobber lists on purpose
+
 namespace jf {
 
 constexpr int KB_STAGE = 4;                         // 32-deep K blocks per LDS stage (128 bytes of K per row)
@@ -91,6 +93,7 @@ __global__ __launch_bounds__(64 * WGM * WGN, WGPC * WGM * WGN / 4) void igemm_nt
     static_assert((BM + BN) / QB <= 16, "scale patch holds 16 blocks per K block");
 
     extern __shared__ __attribute__((aligned(16))) unsigned char smem[];
+    typedef __attribute__((address_space(3))) unsigned char lds_u8;
 
     const int tid = threadIdx.x;
     const int lane = tid & 63;
@@ -110,71 +113,100 @@ __global__ __launch_bounds__(64 * WGM * WGN, WGPC * WGM * WGN / 4) void igemm_nt
     // LDS at (base + 16*l), i.e. row l/8, slot l%8.  To keep the later 16-byte operand reads free of
     // bank conflicts, slot c' of row r holds global chunk c' ^ ((r>>1)&7); the permutation stays
     // inside the row's 128-byte segment, so every instruction still reads 8 full 128-byte lines.
-    unsigned goff[LPW];            // byte offset of this lane's chunk from the operand base (stage 0)
+    // Address split: the 8-row group of load j is wave-uniform (scalar base pointer, advanced by 128 bytes per
+    // stage on the scalar ALU); the lane contributes a fixed offset (its row of the group, its swizzled chunk).
+    // The vector ALU is the bottleneck of this kernel, so the loads must not cost vector instructions.
+    static_assert(NW % 2 == 0, "the chunk swizzle of a lane must not depend on the load index");
+    const int lrow = lane >> 3;
+    const int gchunk = (lane & 7) ^ (((wave & 1) * 4 + (lane >> 4)) & 7);     // global chunk this lane fetches
+    const unsigned loff_a = (unsigned)lrow * (unsigned)p.lda + gchunk * 16;
+    const unsigned loff_b = (unsigned)lrow * (unsigned)p.ldb + gchunk * 16;
+    const int8_t *gbase[LPW];      // wave-uniform: first byte of the group's first row
     bool is_a[LPW];
 #pragma unroll
     for (int j = 0; j < LPW; ++j) {
-        const int grp = wave + j * NW;                        // wave-uniform
+        const int grp = wave + j * NW;
         is_a[j] = grp < BM / 8;
-        const int r = (is_a[j] ? grp : grp - BM / 8) * 8 + (lane >> 3);   // row inside the operand tile
-        const int c = (lane & 7) ^ ((r >> 1) & 7);
-        int gr = (is_a[j] ? m0 : n0) + r;
-        const int lim = is_a[j] ? p.M : p.N;
-        gr = gr < lim ? gr : lim - 1;                         // rows of a partial tile: any valid row
-        goff[j] = (unsigned)gr * (unsigned)(is_a[j] ? p.lda : p.ldb) + c * 16;
+        int r0 = (is_a[j] ? m0 : n0) + (is_a[j] ? grp : grp - BM / 8) * 8;
+        if (r0 >= (is_a[j] ? p.M : p.N)) r0 = is_a[j] ? m0 : n0;   // groups of a partial tile: any valid group
+        gbase[j] = (is_a[j] ? p.A : p.B) + (size_t)r0 * (size_t)(is_a[j] ? p.lda : p.ldb);
     }
-    // Scales of a stage: every wave fetches, again LDS-direct, the 4 x (BM/32 + BN/32) scales of the stage into a
-    // private 256-byte patch (lane l: K block l/16, tile block l%16; A blocks first), so that scale reads need no
-    // cross-wave synchronisation and every wave has the same number of loads in flight.  binary16 scales are
-    // fetched as the aligned 32-bit word that contains them.
+    // Scales of a stage: every wave fetches, again LDS-direct, the scales it needs itself into a private 256-byte
+    // patch (lane l: K block l/16; word l%16 = the wave's WBM A-side scales, then its WBN B-side scales, the rest
+    // padding), so that scale reads need no cross-wave synchronisation, every wave has the same number of loads in
+    // flight, and one LDS read per K block fetches all of them.  binary16 scales are fetched as the aligned 32-bit
+    // word that contains them.  The lane keeps a running pointer.
     constexpr int SCALE_WORDS = 64;
+    constexpr int NSC = WBM + WBN;                            // scales per wave and K block
+    static_assert(NSC <= 4, "one 16-byte LDS read per K block");
     unsigned char *const scale_ring = smem + NSTAGE * STAGE_BYTES + wave * (NSTAGE * SCALE_WORDS * 4);
     const int s_blk = lane & 15;
-    const bool s_is_a = s_blk < BM / QB || s_blk >= (BM + BN) / QB;      // spare lanes repeat A block 0
-    int s_idx = s_is_a ? m0 / QB + (s_blk < BM / QB ? s_blk : 0) : n0 / QB + s_blk - BM / QB;
+    const bool s_is_a = !(s_blk >= WBM && s_blk < NSC);       // padding lanes repeat the first A-side scale
+    int s_idx = s_is_a ? m0 / QB + wm * WBM + (s_blk < WBM ? s_blk : 0) : n0 / QB + wn * WBN + s_blk - WBM;
     { const int lim = s_is_a ? SM : SN; s_idx = s_idx < lim ? s_idx : lim - 1; }
     const int s_ld = s_is_a ? SM : SN;
     const unsigned char *const s_base = reinterpret_cast<const unsigned char *>(s_is_a ? p.sa : p.sb);
+    auto scale_addr = [&](int kbg) {
+        const unsigned e = (unsigned)(kbg * s_ld + s_idx);
+        return s_base + (sizeof(ST) == 4 ? e * 4u : (e >> 1) * 4u);
+    };
+    const unsigned char *s_ptr = scale_addr((lane >> 4) < nkb ? (lane >> 4) : nkb - 1);
+    const unsigned s_step = (unsigned)(KB_STAGE * s_ld) * (unsigned)sizeof(ST);   // KB_STAGE*s_ld is even: exact for binary16
 
-    auto issue_stage = [&](int stage) {
-        unsigned char *dst = smem + (stage % NSTAGE) * STAGE_BYTES;
+    constexpr int A_LOADS = (BM / 8) / NW;                    // loads 0 .. A_LOADS-1 of a wave fetch A rows, the rest B rows
+    static_assert((BM / 8) % NW == 0, "a load instruction fetches rows of one operand");
+    // FULL: the stage has all KB_STAGE K blocks (every stage but a short last one)
+    auto issue_stage_as = [&](int stage, auto full_c) {
+        constexpr bool FULL = decltype(full_c)::value;
+        const unsigned slot_lds = (unsigned)(uintptr_t)(lds_u8 *)smem + (unsigned)(stage % NSTAGE) * STAGE_BYTES;
+        const unsigned scale_lds = (unsigned)(uintptr_t)(lds_u8 *)scale_ring + (unsigned)(stage % NSTAGE) * (SCALE_WORDS * 4);
         const int kb0 = stage * KB_STAGE;
+        // asm: scalar base + 32-bit lane offset is the addressing mode that costs no vector instruction, and the
+        // compiler does not choose it by itself here.  M0 holds the LDS destination of an LDS-direct load.
         if (EPI != EPI_S32) {
-            int kbg = kb0 + (lane >> 4);
-            kbg = kbg < nkb ? kbg : nkb - 1;
-            const unsigned e = (unsigned)(kbg * s_ld + s_idx);
-            const unsigned char *src = s_base + (sizeof(ST) == 4 ? e * 4u : (e >> 1) * 4u);
-            __builtin_amdgcn_global_load_lds((const __attribute__((address_space(1))) void *)src,
-                                             (__attribute__((address_space(3))) void *)(scale_ring + (stage % NSTAGE) * (SCALE_WORDS * 4)),
-                                             4, 0, 0);
+            const unsigned char *src = s_ptr;
+            if (!FULL) {                                      // missing K blocks: fetch the last one again (never used)
+                int kbg = kb0 + (lane >> 4);
+                src = scale_addr(kbg < nkb ? kbg : nkb - 1);
+            }
+            asm volatile("s_mov_b32 m0, %1\n\ts_nop 0\n\tglobal_load_lds_dword %0, off" ::"v"(src), "s"(scale_lds) : "memory", "m0");
+            s_ptr += s_step;
         }
-        const bool partial = kb0 + KB_STAGE > nkb;            // last stage of a K that is not a multiple of 128
+        unsigned la = loff_a, lb = loff_b;
+        if (!FULL && kb0 + (gchunk >> 1) >= nkb) {            // chunks of missing K blocks: the stage's first block again
+            la -= (unsigned)(gchunk >> 1) * QB;
+            lb -= (unsigned)(gchunk >> 1) * QB;
+        }
 #pragma unroll
         for (int j = 0; j < LPW; ++j) {
             const int grp = wave + j * NW;
-            unsigned off = goff[j] + (unsigned)kb0 * QB;
-            if (partial) {
-                // chunks of missing K blocks: fetch the stage's first block again (never used)
-                const int r = (is_a[j] ? grp : grp - BM / 8) * 8 + (lane >> 3);
-                const int c = (lane & 7) ^ ((r >> 1) & 7);
-                if (kb0 + (c >> 1) >= nkb) off -= (unsigned)(c >> 1) * QB;
-            }
-            const int8_t *src = (is_a[j] ? p.A : p.B) + off;
-            __builtin_amdgcn_global_load_lds((const __attribute__((address_space(1))) void *)src,
-                                             (__attribute__((address_space(3))) void *)(dst + grp * 1024), 16, 0, 0);
+            const int8_t *base = gbase[j] + (size_t)kb0 * QB;  // wave-uniform
+            asm volatile("s_mov_b32 m0, %2\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %0, %1"
+                         ::"v"(j < A_LOADS ? la : lb), "s"(base), "s"(slot_lds + (unsigned)grp * 1024u) : "memory", "m0");
         }
+    };
+    auto issue_stage = [&](int stage) {                       // stage < nstages
+        if (stage < nkb / KB_STAGE) issue_stage_as(stage, std::true_type{});
+        else issue_stage_as(stage, std::false_type{});
     };
 
     // ---- operand fetch addresses ----------------------------------------------------------------
     // MFMA operand layout: lane l holds row l%32 of the block and K bytes 16*(l/32) .. +15, i.e. chunk
     // 2*kb + l/32 of the stage row.  Both operands use the same mapping, so one offset per K block.
     // (Ring slot, block index and the A/B split are compile-time offsets folded into the instruction.)
-    unsigned fa_off[KB_STAGE], fb_off[KB_STAGE];
+    lds_u8 *const lds = (lds_u8 *)smem;
+    unsigned fa_u[KB_STAGE], fb_u[KB_STAGE];          // per-lane LDS addresses (ring slot 0), fixed for the whole kernel
 #pragma unroll
     for (int kb = 0; kb < KB_STAGE; ++kb) {
         const unsigned fo = (lane & 31) * ROW_BYTES + (((2 * kb + (lane >> 5)) ^ ((lane >> 1) & 7)) << 4);
-        fa_off[kb] = fo + (wm * WBM * QB) * ROW_BYTES;
-        fb_off[kb] = fo + (wn * WBN * QB) * ROW_BYTES;
+        fa_u[kb] = (unsigned)(uintptr_t)lds + fo + (wm * WBM * QB) * ROW_BYTES;
+        fb_u[kb] = (unsigned)(uintptr_t)lds + A_BYTES + fo + (wn * WBN * QB) * ROW_BYTES;
+    }
+    // scale patch of this wave: a uniform address, parked in a vector register once (LDS reads take a VGPR address)
+    unsigned sc_v;
+    {
+        const unsigned sc_u = (unsigned)(uintptr_t)(lds_u8 *)scale_ring;
+        asm volatile("v_mov_b32 %0, %1" : "=v"(sc_v) : "s"(sc_u));
     }
 
     // ---- accumulators ------------------------------------------------------------------------
@@ -187,19 +219,6 @@ __global__ __launch_bounds__(64 * WGM * WGN, WGPC * WGM * WGN / 4) void igemm_nt
 #pragma unroll
             for (int v = 0; v < 16; ++v) { acc[i][j][v] = 0.0f; iacc[i][j][v] = 0; }
         }
-    // 1.5*2^23 as an integer bit pattern in 16 registers: the accumulator INPUT of every product (see below).
-    // Written through asm so that the compiler keeps the registers instead of re-creating the constant.
-    // -1.5*2^23 in a scalar register: as a literal it would double the size of every v_add_f32 that uses it
-    float neg_magic;
-    asm volatile("s_mov_b32 %0, 0xcb400000" : "=s"(neg_magic));
-    v16i magic;
-#pragma unroll
-    for (int v = 0; v < 16; ++v) {
-        int m;
-        asm volatile("v_mov_b32 %0, 0x4b400000" : "=v"(m));
-        magic[v] = m;
-    }
-
     // block indices of this wave's scales (clamped for partial tiles: those blocks are never stored)
     int mb[WBM], nb[WBN];
 #pragma unroll
@@ -207,133 +226,197 @@ __global__ __launch_bounds__(64 * WGM * WGN, WGPC * WGM * WGN / 4) void igemm_nt
 #pragma unroll
     for (int j = 0; j < WBN; ++j) { nb[j] = n0 / QB + wn * WBN + j; nb[j] = nb[j] < SN ? nb[j] : SN - 1; }
 
-    constexpr int AHEAD = NSTAGE - 1;                         // stages in flight beyond the one being computed
+    // ---- main loop ----------------------------------------------------------------------------
+    // The whole ring is filled up front; afterwards the loads of stage s+NSTAGE are issued when the last K block
+    // of stage s has been read.  Operand fragments and scales of K block k+1 are read from LDS into a second set
+    // of registers BEFORE the products of K block k are issued, so the LDS pipe works while the wave multiplies
+    // and accumulates; without this all waves of a SIMD queue at the LDS together and then compute together.
+    constexpr int AHEAD = NSTAGE - 1;                         // stages in flight beyond the one being consumed
+    constexpr int LOADS = LPW + (EPI != EPI_S32 ? 1 : 0);     // LDS-direct loads per wave and stage
+    const int nfull = nkb / KB_STAGE;                         // stages with all KB_STAGE blocks
+    const int ktail = nkb - nfull * KB_STAGE;                 // K blocks of the short last stage (0: none)
 #pragma unroll
-    for (int s = 0; s < AHEAD; ++s)
+    for (int s = 0; s < NSTAGE; ++s)
         if (s < nstages) issue_stage(s);
 
-    for (int s0 = 0; s0 < nstages; s0 += NSTAGE) static_for<0, NSTAGE>([&](auto slot_c) {
-        constexpr int SLOT = decltype(slot_c)::value;         // ring slot of this stage, a compile-time constant
-        const int s = s0 + SLOT;
-        if (s >= nstages) return;
-        // Loads retire in order, so stage s has landed once only the loads of the younger stages
-        // (s+1 .. s+AHEAD-1, those that exist) are still outstanding.  The barrier then (a) publishes every
-        // wave's part of stage s and (b) guarantees that all waves are done with stage s-1, whose ring slot
-        // the loads issued below overwrite.  (A bare s_barrier: __syncthreads() would drain all loads.)
-        constexpr int LOADS = LPW + (EPI != EPI_S32 ? 1 : 0);    // per wave and stage
-        int younger = nstages - 1 - s;
-        younger = younger < AHEAD - 1 ? younger : AHEAD - 1;
-        if (younger >= 3) JF_WAIT_VMCNT(3 * LOADS);
+    // The fragment reads are written as asm so that they stay where they are and so that the wait for them can
+    // name a count: the compiler, tracking them itself, waits for ALL outstanding LDS reads (the prefetch included)
+    // on every other K block.  LDS reads of a wave return in order, so "at most FETCH_OPS outstanding" after issuing
+    // the next K block's reads means that the current K block's have arrived.
+    typedef float scale_vec __attribute__((ext_vector_type(NSC == 3 ? 3 : NSC <= 2 ? 2 : 4)));
+    v4i fa_reg[2][WBM], fb_reg[2][WBN];
+    scale_vec sc_raw[2];
+    constexpr int FETCH_OPS = WBM + WBN + (EPI != EPI_S32 ? 1 : 0);
+    static_assert(2 * FETCH_OPS <= 15, "lgkmcnt is a 4-bit counter");
+    // pa/pb: this lane's fragment addresses for the K block (ring slot 0); psc: the wave's scale patch;
+    // slot_bytes / slot_words: compile-time offset of the ring slot in the tile ring and of the K block in the patch
+    auto fetch = [&](const unsigned pa, const unsigned pb, const unsigned psc, auto slot_bytes_c, auto slot_words_c, auto buf_c) {
+        constexpr int BUF = decltype(buf_c)::value;
+        constexpr int SB = decltype(slot_bytes_c)::value, SW = decltype(slot_words_c)::value;
+#pragma unroll
+        for (int i = 0; i < WBM; ++i)
+            asm volatile("ds_read_b128 %0, %1 offset:%2" : "=v"(fa_reg[BUF][i]) : "v"(pa), "n"(SB + i * (QB * ROW_BYTES)));
+#pragma unroll
+        for (int j = 0; j < WBN; ++j)
+            asm volatile("ds_read_b128 %0, %1 offset:%2" : "=v"(fb_reg[BUF][j]) : "v"(pb), "n"(SB + j * (QB * ROW_BYTES)));
+        if (EPI != EPI_S32) {
+            scale_vec &dst = sc_raw[BUF];
+            if (NSC == 3) asm volatile("ds_read_b96 %0, %1 offset:%2" : "=v"(dst) : "v"(psc), "n"(SW * 4));
+            else if (NSC <= 2) asm volatile("ds_read_b64 %0, %1 offset:%2" : "=v"(dst) : "v"(psc), "n"(SW * 4));
+            else asm volatile("ds_read_b128 %0, %1 offset:%2" : "=v"(dst) : "v"(psc), "n"(SW * 4));
+        }
+    };
+    // wait until at most `n` LDS reads are outstanding, and tie register set BUF to that point in program order
+    auto fetched = [&](auto n_c, auto buf_c) {
+        constexpr int BUF = decltype(buf_c)::value, N = decltype(n_c)::value;
+        __builtin_amdgcn_s_waitcnt(0xC07F | (N << 8));        // lgkmcnt(N) only
+#pragma unroll
+        for (int i = 0; i < WBM; ++i) asm volatile("" : "+v"(fa_reg[BUF][i]));
+#pragma unroll
+        for (int j = 0; j < WBN; ++j) asm volatile("" : "+v"(fb_reg[BUF][j]));
+        if (EPI != EPI_S32) { scale_vec &r = sc_raw[BUF]; asm volatile("" : "+v"(r)); }
+    };
+    // Products and scale-accumulate of one K block (global index kbg) from register set CUR.
+    // The matrix pipe and the vector ALU do not run concurrently on this part, and a product needs about 40 cycles
+    // before the vector ALU can read it.  So the accumulation lags the products by one: product n is issued, THEN
+    // product n-1 (long finished) is converted and accumulated.  (d_pend, sab_pend) carry the lagging product across
+    // K blocks and stages; the first accumulation adds 0*0 and the last product is accumulated after the loop.
+    constexpr int NBLK = WBM * WBN;
+    v16i d_pend = {0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0};
+    float sab_pend = 0.0f;
+    auto accumulate = [&](auto blk_c) {
+        constexpr int i = decltype(blk_c)::value / WBN, j = decltype(blk_c)::value % WBN;
+        float t[16];
+#pragma unroll
+        for (int v = 0; v < 16; ++v) t[v] = (float)d_pend[v];          // exact: |d| <= 32*127^2
+#pragma unroll
+        for (int v = 0; v < 16; ++v) acc[i][j][v] = __builtin_fmaf(sab_pend, t[v], acc[i][j][v]);
+        // pin the accumulation here: the optimiser would otherwise postpone it past the next K blocks and keep their
+        // products alive in registers it does not have
+#pragma unroll
+        for (int v = 0; v < 16; ++v) asm volatile("" : "+v"(acc[i][j][v]));
+    };
+    auto compute = [&](auto cur_c, const int kbg) {
+        constexpr int CUR = decltype(cur_c)::value;
+        if (EPI == EPI_S32) {
+#pragma unroll
+            for (int i = 0; i < WBM; ++i)
+#pragma unroll
+                for (int j = 0; j < WBN; ++j)
+                    iacc[i][j] = __builtin_amdgcn_mfma_i32_32x32x32_i8(fa_reg[CUR][i], fb_reg[CUR][j], iacc[i][j], 0, 0, 0);
+        } else {
+            float fa[WBM], fb[WBN];
+            // binary16 scales arrive as the 32-bit word that holds them: the half to use is the parity of the
+            // scale's element index (wave-uniform)
+            auto scale_of = [&](float raw, int elem) -> float {
+                if (sizeof(ST) == 4) return raw;
+                const uint32_t w = __float_as_uint(raw);
+                const uint16_t h = (elem & 1) ? (uint16_t)(w >> 16) : (uint16_t)w;
+                return (float)__builtin_bit_cast(half_t, h);
+            };
+#pragma unroll
+            for (int i = 0; i < WBM; ++i) fa[i] = scale_of(sc_raw[CUR][i], kbg * SM + mb[i]);
+#pragma unroll
+            for (int j = 0; j < WBN; ++j) fb[j] = scale_of(sc_raw[CUR][WBM + j], kbg * SN + nb[j]);
+            static_for<0, NBLK>([&](auto n_c) {
+                constexpr int n = decltype(n_c)::value, i = n / WBN, j = n % WBN;
+                const v16i z = {0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0};
+                const v16i d_new = __builtin_amdgcn_mfma_i32_32x32x32_i8(fa_reg[CUR][i], fb_reg[CUR][j], z, 0, 0, 0);
+                const float sab_new = fa[i] * fb[j];
+                __builtin_amdgcn_sched_barrier(0);
+                accumulate(std::integral_constant<int, (n + NBLK - 1) % NBLK>{});
+                __builtin_amdgcn_sched_barrier(0);
+                d_pend = d_new;
+                sab_pend = sab_new;
+            });
+        }
+    };
+    // Loads retire in order: stage t has landed once only the loads of the stages issued after it are outstanding.
+    auto wait_stage = [&](int t, int last_issued) {
+        int younger = (last_issued < nstages - 1 ? last_issued : nstages - 1) - t;
+        if (younger >= 4) JF_WAIT_VMCNT(4 * LOADS);
+        else if (younger == 3) JF_WAIT_VMCNT(3 * LOADS);
         else if (younger == 2) JF_WAIT_VMCNT(2 * LOADS);
         else if (younger == 1) JF_WAIT_VMCNT(LOADS);
         else JF_WAIT_VMCNT(0);
-#if !(defined(JF_DBG_MODE) && (JF_DBG_MODE == 6 || JF_DBG_MODE == 7))
-        asm volatile("" ::: "memory");
-        __builtin_amdgcn_s_barrier();
-        asm volatile("" ::: "memory");
-#endif
-#if !(defined(JF_DBG_MODE) && (JF_DBG_MODE == 6))
-        if (s + AHEAD < nstages) issue_stage(s + AHEAD);
-#endif
+    };
+    using c0 = std::integral_constant<int, 0>;
+    using c1 = std::integral_constant<int, 1>;
+    wait_stage(0, NSTAGE - 1);
+    asm volatile("" ::: "memory");
+    __builtin_amdgcn_s_barrier();                              // bare: __syncthreads() would drain every load
+    asm volatile("" ::: "memory");
+    fetch(fa_u[0], fb_u[0], sc_v, c0{}, c0{}, c0{});
 
-        const unsigned char *base = smem + SLOT * STAGE_BYTES;
-        const float *sc_lds = reinterpret_cast<const float *>(scale_ring + SLOT * (SCALE_WORDS * 4));
-        const int kbs = (nkb - s * KB_STAGE) < KB_STAGE ? (nkb - s * KB_STAGE) : KB_STAGE;
-        auto compute_kb = [&](int kb) {
-            v4i a[WBM], b[WBN];
-#if defined(JF_DBG_MODE) && (JF_DBG_MODE == 1 || JF_DBG_MODE == 3)
-#pragma unroll
-            for (int i = 0; i < WBM; ++i) a[i] = v4i{lane, kb, i, 1};
-#pragma unroll
-            for (int j = 0; j < WBN; ++j) b[j] = v4i{lane, 2, j, kb};
-#else
-#pragma unroll
-            for (int i = 0; i < WBM; ++i)
-                a[i] = *reinterpret_cast<const v4i *>(base + i * (QB * ROW_BYTES) + fa_off[kb]);
-#pragma unroll
-            for (int j = 0; j < WBN; ++j)
-                b[j] = *reinterpret_cast<const v4i *>(base + A_BYTES + j * (QB * ROW_BYTES) + fb_off[kb]);
-#endif
-#if defined(JF_DBG_MODE) && (JF_DBG_MODE == 1 || JF_DBG_MODE == 2)
-            if (EPI == EPI_S32) {
-#pragma unroll
-                for (int i = 0; i < WBM; ++i)
-#pragma unroll
-                    for (int j = 0; j < WBN; ++j) { iacc[i][j][0] ^= a[i].x ^ b[j].y; iacc[i][j][1] ^= a[i].z ^ b[j].w; }
-            } else
-#endif
-            if (EPI == EPI_S32) {
-#pragma unroll
-                for (int i = 0; i < WBM; ++i)
-#pragma unroll
-                    for (int j = 0; j < WBN; ++j)
-                        iacc[i][j] = __builtin_amdgcn_mfma_i32_32x32x32_i8(a[i], b[j], iacc[i][j], 0, 0, 0);
+    for (int s0 = 0; s0 < nfull; s0 += NSTAGE) static_for<0, NSTAGE>([&](auto slot_c) {
+        constexpr int SLOT = decltype(slot_c)::value;         // ring slot of this stage, a compile-time constant
+        constexpr int NEXT_SLOT = (SLOT + 1) % NSTAGE;
+        const int s = s0 + SLOT;
+        if (s >= nfull) return;
+        static_for<0, KB_STAGE>([&](auto kb_c) {
+            constexpr int kb = decltype(kb_c)::value;
+            constexpr int CUR = kb & 1, NXT = CUR ^ 1;
+            if constexpr (kb == KB_STAGE - 1) {
+                if (s + 1 < nstages) {
+                    // Stage hand-over.  This wave's LDS reads of stage s are complete (lgkmcnt 0) and stage s+1 has
+                    // landed; after the barrier that holds for every wave, so (a) stage s+1 may be read and (b) the
+                    // ring slot of stage s may be overwritten by the loads of stage s+NSTAGE.
+                    __builtin_amdgcn_s_waitcnt(0xC07F);       // lgkmcnt(0) only
+                    wait_stage(s + 1, s + NSTAGE - 1);
+                    asm volatile("" ::: "memory");
+                    __builtin_amdgcn_s_barrier();
+                    asm volatile("" ::: "memory");
+                    if (s + NSTAGE < nstages) issue_stage(s + NSTAGE);
+                }
+                // unconditional: past the last stage it reads bytes of the ring that nobody uses
+                fetch(fa_u[0], fb_u[0], sc_v, std::integral_constant<int, NEXT_SLOT * STAGE_BYTES>{},
+                      std::integral_constant<int, NEXT_SLOT * 64>{}, std::integral_constant<int, NXT>{});
             } else {
-                float fa[WBM], fb[WBN];
-                int kbg = s * KB_STAGE + kb; kbg = kbg < nkb ? kbg : nkb - 1;
-                // binary16 scales arrive as the 32-bit word that holds them: the half to use is the parity of the
-                // scale's element index (wave-uniform)
-                auto scale_at = [&](int word, int elem) -> float {
-                    if (sizeof(ST) == 4) return sc_lds[word];
-                    const uint32_t w = __float_as_uint(sc_lds[word]);
-                    const uint16_t h = (elem & 1) ? (uint16_t)(w >> 16) : (uint16_t)w;
-                    return (float)__builtin_bit_cast(half_t, h);
-                };
-#pragma unroll
-                for (int i = 0; i < WBM; ++i) fa[i] = scale_at(kb * 16 + wm * WBM + i, kbg * SM + mb[i]);
-#pragma unroll
-                for (int j = 0; j < WBN; ++j) fb[j] = scale_at(kb * 16 + BM / QB + wn * WBN + j, kbg * SN + nb[j]);
-                // The accumulator input is the bit pattern of 1.5*2^23: the INT32 result d + 0x4B400000, read as a
-                // float, IS 12582912.0 + d (|d| <= 32*127^2 < 2^22), so one exact fp32 subtraction replaces the
-                // slower integer-to-float conversion.  All products are issued before the first one is consumed,
-                // so the matrix pipe works while the vector ALU does the scale-accumulate.
-                v16i d[WBM][WBN];
-#pragma unroll
-                for (int i = 0; i < WBM; ++i)
-#pragma unroll
-                    for (int j = 0; j < WBN; ++j)
-#ifdef JF_ZERO_C
-                        { const v16i z = {0,0,0,0,0,0,0,0,0,0,0,0,0,0,0,0}; d[i][j] = __builtin_amdgcn_mfma_i32_32x32x32_i8(a[i], b[j], z, 0, 0, 0); }
-#else
-                        d[i][j] = __builtin_amdgcn_mfma_i32_32x32x32_i8(a[i], b[j], magic, 0, 0, 0);
-#endif
-#pragma unroll
-                for (int i = 0; i < WBM; ++i)
-#pragma unroll
-                    for (int j = 0; j < WBN; ++j) {
-                        const float sab = fa[i] * fb[j];
-                        float t[16];
-#pragma unroll
-#ifdef JF_ZERO_C
-                        for (int v = 0; v < 16; ++v) t[v] = (float)d[i][j][v];
-#else
-                        for (int v = 0; v < 16; ++v) t[v] = __int_as_float(d[i][j][v]) + neg_magic;
-#endif
-#pragma unroll
-                        for (int v = 0; v < 16; ++v) acc[i][j][v] = __builtin_fmaf(sab, t[v], acc[i][j][v]);
-                    }
+                fetch(fa_u[kb + 1], fb_u[kb + 1], sc_v, std::integral_constant<int, SLOT * STAGE_BYTES>{},
+                      std::integral_constant<int, SLOT * 64 + (kb + 1) * 16>{}, std::integral_constant<int, NXT>{});
             }
-        };
-#pragma unroll
-        for (int kb = 0; kb < KB_STAGE; ++kb)
-            if (kb < kbs) compute_kb(kb);                     // uniform; only the last stage can be short
+            fetched(std::integral_constant<int, FETCH_OPS>{}, std::integral_constant<int, CUR>{});
+            __builtin_amdgcn_sched_barrier(0);                // the reads above stay above the products below,
+            compute(std::integral_constant<int, CUR>{}, s * KB_STAGE + kb);
+            __builtin_amdgcn_sched_barrier(0);                // and K blocks are scheduled one by one (register pressure)
+        });
     });
-    __syncthreads();           // the epilogue reuses the ring as scratch
-#if defined(JF_DBG_MODE) && (JF_DBG_MODE >= 5)
-    {   // timing experiment: main loop only
-        for (int i = 0; i < WBM; ++i) for (int j = 0; j < WBN; ++j) for (int v = 0; v < 16; ++v) {
-            if (EPI == EPI_S32) asm volatile("" :: "v"(iacc[i][j][v])); else asm volatile("" :: "v"(acc[i][j][v]));
-        }
-        return;
+    if (ktail) {
+        // short last stage (K not a multiple of 128): its first K block is already on its way to register set 0
+        const unsigned slot = (unsigned)(nfull % NSTAGE);
+        static_for<0, KB_STAGE - 1>([&](auto kb_c) {
+            constexpr int kb = decltype(kb_c)::value;
+            constexpr int CUR = kb & 1;
+            if (kb < ktail) {
+                if (kb > 0)
+                    fetch(fa_u[kb] + slot * STAGE_BYTES, fb_u[kb] + slot * STAGE_BYTES, sc_v + slot * 256,
+                          c0{}, std::integral_constant<int, kb * 16>{}, std::integral_constant<int, CUR>{});
+                fetched(c0{}, std::integral_constant<int, CUR>{});
+                compute(std::integral_constant<int, CUR>{}, nfull * KB_STAGE + kb);
+            }
+        });
     }
-#endif
+    __builtin_amdgcn_s_waitcnt(0xC07F);                        // the last, unused prefetch must land before its registers are reused
+    if (EPI != EPI_S32) accumulate(std::integral_constant<int, NBLK - 1>{});
+    __syncthreads();           // the epilogue reuses the ring as scratch
 
-    // ---- epilogue: one 32x32 block at a time through a wave-private LDS patch ------------------
-    // MFMA result layout: lane l, register v  <->  row 8*(v/4) + 4*(l/32) + v%4, column l%32.
-    // Read-back layout: lane l  <->  row l/2, columns 16*(l%2) .. +15 (row-contiguous stores).
+    // ---- epilogue ------------------------------------------------------------------------------------------
+    // One 32x32 block at a time goes through a wave-private LDS patch that turns the MFMA result layout
+    //   (lane l, register v  <->  row 8*(v/4) + 4*(l/32) + v%4, column l%32)
+    // into a row layout (lane l <-> row l/2, columns 16*(l%2) .. +15): 16 consecutive columns per lane are what the
+    // Philox noise (8 elements per call) and 16-byte packing want.  One- and two-byte outputs are then collected in
+    // a workgroup-wide LDS image of the tile and written out in full 128-byte (or 256-byte) rows; four-byte outputs
+    // (INT32, fp32) are stored straight from the row layout (64 contiguous bytes per lane).
+    auto wave_sync = [] {
+        __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
+        __builtin_amdgcn_wave_barrier();
+        __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
+    };
     float *patch = reinterpret_cast<float *>(smem) + wave * (QB * EPI_LD);
+    unsigned char *tile = smem + NW * (QB * EPI_LD) * sizeof(float);       // [BM][BN * out_bytes]
     const int rrow = lane >> 1, rcol = (lane & 1) * 16;
     const float biasmax = (EPI == EPI_Q && p.biasmax) ? p.biasmax[0] : 0.0f;
+    const int out_bytes = EPI == EPI_Q ? 1 : (EPI == EPI_FP && p.out_dtype != JF_FP_F32 ? 2 : 4);   // uniform
 
 #pragma unroll
     for (int i = 0; i < WBM; ++i)
@@ -341,6 +424,7 @@ __global__ __launch_bounds__(64 * WGM * WGN, WGPC * WGM * WGN / 4) void igemm_nt
         for (int j = 0; j < WBN; ++j) {
             const int bm = m0 + (wm * WBM + i) * QB, bn = n0 + (wn * WBN + j) * QB;
             const bool valid = bm < p.M && bn < p.N;          // wave-uniform
+            if (!valid) continue;
             float amax = 0.0f;
             if (EPI == EPI_Q) {
                 float m = 0.0f;
@@ -354,16 +438,17 @@ __global__ __launch_bounds__(64 * WGM * WGN, WGPC * WGM * WGN / 4) void igemm_nt
                 if (EPI == EPI_S32) patch[r * EPI_LD + (lane & 31)] = __int_as_float(iacc[i][j][v]);
                 else patch[r * EPI_LD + (lane & 31)] = acc[i][j][v];
             }
-            __syncthreads();
+            wave_sync();
             float x[16];
 #pragma unroll
             for (int k = 0; k < 4; ++k) {
                 const v4f t = *reinterpret_cast<const v4f *>(patch + rrow * EPI_LD + rcol + 4 * k);
                 x[4 * k] = t.x; x[4 * k + 1] = t.y; x[4 * k + 2] = t.z; x[4 * k + 3] = t.w;
             }
-            __syncthreads();
-            if (!valid) continue;
+            wave_sync();
             const size_t e0 = (size_t)(bm + rrow) * p.N + bn + rcol;
+            // position of the lane's 16 values inside the workgroup's tile image
+            const int trow = (wm * WBM + i) * QB + rrow, tcol = (wn * WBN + j) * QB + rcol;
             if (EPI == EPI_S32) {
                 v4i *dst = reinterpret_cast<v4i *>(reinterpret_cast<int32_t *>(p.C) + e0);
 #pragma unroll
@@ -380,20 +465,21 @@ __global__ __launch_bounds__(64 * WGM * WGN, WGPC * WGM * WGN / 4) void igemm_nt
                         v4f t = {x[4 * k], x[4 * k + 1], x[4 * k + 2], x[4 * k + 3]};
                         dst[k] = t;
                     }
-                } else if (p.out_dtype == JF_FP_F16) {
-                    half_t h[16];
-#pragma unroll
-                    for (int k = 0; k < 16; ++k) h[k] = (half_t)x[k];
-                    v4i *dst = reinterpret_cast<v4i *>(reinterpret_cast<half_t *>(p.C) + e0);
-                    dst[0] = *reinterpret_cast<v4i *>(&h[0]);
-                    dst[1] = *reinterpret_cast<v4i *>(&h[8]);
                 } else {
-                    __bf16 h[16];
+                    v4i lo, hi;
+                    if (p.out_dtype == JF_FP_F16) {
+                        half_t h[16];
 #pragma unroll
-                    for (int k = 0; k < 16; ++k) h[k] = (__bf16)x[k];
-                    v4i *dst = reinterpret_cast<v4i *>(reinterpret_cast<__bf16 *>(p.C) + e0);
-                    dst[0] = *reinterpret_cast<v4i *>(&h[0]);
-                    dst[1] = *reinterpret_cast<v4i *>(&h[8]);
+                        for (int k = 0; k < 16; ++k) h[k] = (half_t)x[k];
+                        lo = *reinterpret_cast<v4i *>(&h[0]); hi = *reinterpret_cast<v4i *>(&h[8]);
+                    } else {
+                        __bf16 h[16];
+#pragma unroll
+                        for (int k = 0; k < 16; ++k) h[k] = (__bf16)x[k];
+                        lo = *reinterpret_cast<v4i *>(&h[0]); hi = *reinterpret_cast<v4i *>(&h[8]);
+                    }
+                    v4i *dst = reinterpret_cast<v4i *>(tile + (size_t)trow * (BN * 2) + tcol * 2);
+                    dst[0] = lo; dst[1] = hi;
                 }
             } else {
                 v4i codes = {0, 0, 0, 0};
@@ -422,10 +508,24 @@ __global__ __launch_bounds__(64 * WGM * WGN, WGPC * WGM * WGN / 4) void igemm_nt
                     codes.z = (int)pack4(c[8], c[9], c[10], c[11]);
                     codes.w = (int)pack4(c[12], c[13], c[14], c[15]);
                 }
-                *reinterpret_cast<v4i *>(reinterpret_cast<int8_t *>(p.C) + e0) = codes;
+                *reinterpret_cast<v4i *>(tile + (size_t)trow * BN + tcol) = codes;
                 if (lane == 0) store_scale(reinterpret_cast<ST *>(p.sc), (bm / QB) * SN + bn / QB, scale);
             }
         }
+
+    if (out_bytes < 4) {
+        __syncthreads();
+        // the tile image leaves in whole rows: consecutive lanes write consecutive 16-byte chunks of a row
+        const int row_bytes = BN * out_bytes, chunks_per_row = row_bytes / 16;
+        unsigned char *cbase = reinterpret_cast<unsigned char *>(p.C);
+        for (int idx = tid; idx < BM * chunks_per_row; idx += 64 * NW) {
+            const int row = idx / chunks_per_row, ch = idx - row * chunks_per_row;
+            const int gm = m0 + row, gn = n0 + ch * (16 / out_bytes);
+            if (gm < p.M && gn < p.N)
+                *reinterpret_cast<v4i *>(cbase + ((size_t)gm * p.N + gn) * out_bytes) =
+                    *reinterpret_cast<const v4i *>(tile + (size_t)row * row_bytes + ch * 16);
+        }
+    }
 }
 
 // -------------------------------------------------------------------------------------------------
@@ -467,7 +567,7 @@ static int launch_gemm_cfg(const GemmArgs &a, hipStream_t st)
 {
     constexpr int BM = QB * WBM * WGM, BN = QB * WBN * WGN, NT = 64 * WGM * WGN;
     constexpr int RING = NSTAGE * (BM + BN) * ROW_BYTES + WGM * WGN * NSTAGE * 256;   // operand ring + per-wave scale patches
-    constexpr int PATCH = WGM * WGN * QB * EPI_LD * (int)sizeof(float);
+    constexpr int PATCH = WGM * WGN * QB * EPI_LD * (int)sizeof(float) + (EPI == EPI_S32 ? 0 : BM * BN * (EPI == EPI_Q ? 1 : 2));   // + tile image
     constexpr int SMEM = RING > PATCH ? RING : PATCH;
     GemmArgs p = a;
     p.tiles_m = (p.M + BM - 1) / BM;
