@@ -122,22 +122,96 @@ __global__ __launch_bounds__(NT) void dequantize_kernel(const int8_t *q, const S
     }
 }
 
+// GELU on a block tensor.  A block has ONE scale, so its 1024 inputs take at most 256 distinct values code*scale:
+// the wave evaluates the function once per code (4 codes per lane) into a 1 KiB LDS table and every element then
+// costs one LDS gather instead of ~40 vector instructions.  The table entry is computed from (float)code * scale,
+// the very expression a per-element evaluation would use, so the results are bit-identical to it.
+template <typename F>
+__device__ __forceinline__ void fill_code_table(float *table, int lane, float scale, F f)
+{
+    v4f t;
+    t.x = f((float)(int8_t)(4 * lane + 0) * scale);
+    t.y = f((float)(int8_t)(4 * lane + 1) * scale);
+    t.z = f((float)(int8_t)(4 * lane + 2) * scale);
+    t.w = f((float)(int8_t)(4 * lane + 3) * scale);
+    *reinterpret_cast<v4f *>(table + 4 * lane) = t;               // entry index = the code's byte value
+    __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
+    __builtin_amdgcn_wave_barrier();
+    __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
+}
+__device__ __forceinline__ void gather16(const float *table, v4i p, float x[16])
+{
+    const uint32_t w[4] = {(uint32_t)p.x, (uint32_t)p.y, (uint32_t)p.z, (uint32_t)p.w};
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+        x[4 * i + 0] = table[w[i] & 0xFF];
+        x[4 * i + 1] = table[(w[i] >> 8) & 0xFF];
+        x[4 * i + 2] = table[(w[i] >> 16) & 0xFF];
+        x[4 * i + 3] = table[w[i] >> 24];
+    }
+}
+__device__ __forceinline__ void table_done()
+{
+    __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
+    __builtin_amdgcn_wave_barrier();                               // all gathers done before the next block's fill
+}
+
+// A wave that loads one block (1 KiB of codes), waits, computes and stores keeps far too few bytes in flight to
+// cover the memory latency, so the GELU kernels run the block loop with the codes and scales of the next PF blocks
+// already requested.
+constexpr int PF = 3;
+template <typename ST> struct CodeStream {
+    const int8_t *q;
+    const ST *s;
+    int C, SC, nblk, stride, lane;
+    v4i codes[PF];
+    float scale[PF];
+    __device__ __forceinline__ void request(int slot, int blk)
+    {
+        if (blk < nblk) {
+            const int rb = blk / SC, cb = blk - rb * SC;
+            codes[slot] = *reinterpret_cast<const v4i *>(q + (size_t)(rb * QB + (lane >> 1)) * C + cb * QB + (lane & 1) * 16);
+            scale[slot] = load_scale(s, blk);
+        }
+    }
+    __device__ __forceinline__ CodeStream(const int8_t *q_, const ST *s_, int C_, int SC_, int nblk_, int stride_, int lane_, int blk0)
+        : q(q_), s(s_), C(C_), SC(SC_), nblk(nblk_), stride(stride_), lane(lane_)
+    {
+#pragma unroll
+        for (int i = 0; i < PF; ++i) request(i, blk0 + i * stride);
+    }
+    // hands out the oldest block and requests the one PF strides ahead
+    __device__ __forceinline__ void next(int blk, v4i &c, float &sc)
+    {
+        c = codes[0]; sc = scale[0];
+#pragma unroll
+        for (int i = 0; i + 1 < PF; ++i) { codes[i] = codes[i + 1]; scale[i] = scale[i + 1]; }
+        request(PF - 1, blk + PF * stride);
+    }
+};
+
 // gelu_fwd.py:34-126
 template <int APPROX, typename ST>
 __global__ __launch_bounds__(NT) void gelu_fwd_kernel(const int8_t *q, const ST *s, int R, int C, float amax_eps,
                                                       int8_t *qy, ST *sy)
 {
-    JF_FOR_EACH_BLOCK(R, C)
-    {
+    __shared__ __attribute__((aligned(16))) float table[WPB][256];
+    float *tab = table[threadIdx.x >> 6];
+    const int lane = threadIdx.x & 63, SC = C / QB, nblk = (R / QB) * SC, stride = gridDim.x * WPB;
+    const int blk0 = blockIdx.x * WPB + (threadIdx.x >> 6);
+    CodeStream<ST> in(q, s, C, SC, nblk, stride, lane, blk0);
+    for (int blk = blk0; blk < nblk; blk += stride) {
         BlockPos pos(blk, SC, C, lane);
+        v4i c; float sc;
+        in.next(blk, c, sc);
+        fill_code_table(tab, lane, sc, [](float v) { return gelu<APPROX>(v); });
         float x[16];
-        unpack16(*reinterpret_cast<const v4i *>(q + pos.e0), load_scale(s, pos.rb * SC + pos.cb), x);
-#pragma unroll
-        for (int k = 0; k < 16; ++k) x[k] = gelu<APPROX>(x[k]);
+        gather16(tab, c, x);
+        table_done();
         float scale;
         v4i codes = quantize16(x, amax_eps, JF_ROUND_NEAREST, 0, 0, pos.e0, &scale);
         *reinterpret_cast<v4i *>(qy + pos.e0) = codes;
-        if (lane == 0) store_scale(sy, pos.rb * SC + pos.cb, scale);
+        if (lane == 0) store_scale(sy, blk, scale);
     }
 }
 
@@ -147,18 +221,27 @@ __global__ __launch_bounds__(NT) void gelu_bwd_kernel(const int8_t *qx, const ST
                                                       int R, int C, int rounding, uint64_t seed, uint64_t offset,
                                                       int8_t *qy, ST *sy)
 {
-    JF_FOR_EACH_BLOCK(R, C)
-    {
+    __shared__ __attribute__((aligned(16))) float table[WPB][256];
+    float *tab = table[threadIdx.x >> 6];
+    const int lane = threadIdx.x & 63, SC = C / QB, nblk = (R / QB) * SC, stride = gridDim.x * WPB;
+    const int blk0 = blockIdx.x * WPB + (threadIdx.x >> 6);
+    CodeStream<ST> inx(qx, sx, C, SC, nblk, stride, lane, blk0), ing(qg, sg, C, SC, nblk, stride, lane, blk0);
+    for (int blk = blk0; blk < nblk; blk += stride) {
         BlockPos pos(blk, SC, C, lane);
+        v4i cx, cg; float scx, scg;
+        inx.next(blk, cx, scx);
+        ing.next(blk, cg, scg);
         float x[16], g[16];
-        unpack16(*reinterpret_cast<const v4i *>(qx + pos.e0), load_scale(sx, pos.rb * SC + pos.cb), x);
-        unpack16(*reinterpret_cast<const v4i *>(qg + pos.e0), load_scale(sg, pos.rb * SC + pos.cb), g);
+        unpack16(cg, scg, g);
+        fill_code_table(tab, lane, scx, [](float v) { return dgelu<APPROX>(v); });
+        gather16(tab, cx, x);
+        table_done();
 #pragma unroll
-        for (int k = 0; k < 16; ++k) x[k] = dgelu<APPROX>(x[k]) * g[k];
+        for (int k = 0; k < 16; ++k) x[k] = x[k] * g[k];
         float scale;
         v4i codes = quantize16(x, 0.0f, rounding, seed, offset, pos.e0, &scale);
         *reinterpret_cast<v4i *>(qy + pos.e0) = codes;
-        if (lane == 0) store_scale(sy, pos.rb * SC + pos.cb, scale);
+        if (lane == 0) store_scale(sy, blk, scale);
     }
 }
 

@@ -7,6 +7,7 @@
 #pragma once
 
 #include <hip/hip_runtime.h>
+#include <type_traits>
 #include <stdint.h>
 
 #include "../../include/jetfire_hip.h"
@@ -27,12 +28,24 @@ template <typename ST> __device__ __forceinline__ float load_scale(const ST *p, 
 template <typename ST> __device__ __forceinline__ void store_scale(ST *p, int i, float v) { p[i] = (ST)v; }
 
 // ---------------------------------------------------------------------------------------------
-// 64-lane max reduction; every lane returns the maximum.
+// 64-lane max reduction of NON-NEGATIVE values; every lane returns the maximum (it comes back through a scalar
+// register, so the compiler knows it is wave-uniform).  Data-parallel-primitive moves inside the vector ALU:
+// a shuffle through the LDS crossbar would cost six dependent LDS round trips.
 __device__ __forceinline__ float wave_max(float v)
 {
-#pragma unroll
-    for (int m = 32; m >= 1; m >>= 1) v = fmaxf(v, __shfl_xor(v, m, WAVE));
-    return v;
+    auto step = [](float x, auto ctrl_c, auto rows_c) {
+        const int t = __builtin_amdgcn_update_dpp(__float_as_int(x), __float_as_int(x), decltype(ctrl_c)::value,
+                                                  decltype(rows_c)::value, 0xF, false);
+        return fmaxf(x, __int_as_float(t));
+    };
+    using all = std::integral_constant<int, 0xF>;
+    v = step(v, std::integral_constant<int, 0xB1>{}, all{});     // quad_perm [1,0,3,2]
+    v = step(v, std::integral_constant<int, 0x4E>{}, all{});     // quad_perm [2,3,0,1]
+    v = step(v, std::integral_constant<int, 0x141>{}, all{});    // row_half_mirror: max of 8
+    v = step(v, std::integral_constant<int, 0x140>{}, all{});    // row_mirror: max of the 16-lane row, in all its lanes
+    v = step(v, std::integral_constant<int, 0x142>{}, std::integral_constant<int, 0xA>{});   // row_bcast15 into rows 1, 3
+    v = step(v, std::integral_constant<int, 0x143>{}, std::integral_constant<int, 0xC>{});   // row_bcast31 into rows 2, 3
+    return __int_as_float(__builtin_amdgcn_readlane(__float_as_int(v), 63));
 }
 
 // ---------------------------------------------------------------------------------------------
@@ -80,20 +93,26 @@ __device__ __forceinline__ void sr_noise16(uint64_t seed, uint64_t offset, uint6
 // caller takes this path only for s in [2^-60, 2^60] and falls back to the IEEE division otherwise.
 struct BlockDivisor {
     float s, r;
-    bool fast;
+    bool fast;                  // the same in all lanes (s is a block constant): kept in a scalar register
     __device__ __forceinline__ explicit BlockDivisor(float s_) : s(s_)
     {
-        fast = (s_ > 8.67361738e-19f) && (s_ < 1.15292150e+18f);
+        fast = __builtin_amdgcn_readfirstlane((s_ > 8.67361738e-19f) && (s_ < 1.15292150e+18f)) != 0;
         r = 1.0f / s_;
     }
-    __device__ __forceinline__ float div(float x) const
+    // y[i] = x[i] / s for 16 values; ONE uniform branch around the whole batch
+    __device__ __forceinline__ void div16(const float x[16], float y[16]) const
     {
         if (fast) {
-            float q0 = x * r;
-            float e = __builtin_fmaf(-q0, s, x);
-            return __builtin_fmaf(e, r, q0);
+#pragma unroll
+            for (int i = 0; i < 16; ++i) {
+                float q0 = x[i] * r;
+                float e = __builtin_fmaf(-q0, s, x[i]);
+                y[i] = __builtin_fmaf(e, r, q0);
+            }
+        } else {
+#pragma unroll
+            for (int i = 0; i < 16; ++i) y[i] = x[i] / s;
         }
-        return x / s;
     }
 };
 
@@ -126,8 +145,7 @@ __device__ __forceinline__ v4i quantize16(const float v[16], float amax_eps, int
     *scale_out = s;
     BlockDivisor d(s);
     float y[16];
-#pragma unroll
-    for (int i = 0; i < 16; ++i) y[i] = d.div(v[i]);
+    d.div16(v, y);
     if (rounding == JF_ROUND_STOCHASTIC || rounding == JF_ROUND_STOCHASTIC_TRUNC) {
         float n[16];
         sr_noise16(seed, offset, e0, n);
@@ -168,8 +186,8 @@ __device__ __forceinline__ void unpack16(v4i p, float scale, float x[16])
 // Elementary functions (same sequences as the host checker uses).
 __device__ __forceinline__ float expf_det(float x)
 {
-    if (x < -87.0f) return 0.0f;
-    x = fminf(x, 88.0f);
+    const bool tiny = x < -87.0f;                    // result 0; selected at the end so that the code stays branch-free
+    x = fmaxf(fminf(x, 88.0f), -87.0f);
     float n = __builtin_rintf(x * 1.44269504f);
     float r = __builtin_fmaf(n, -0.693145752f, x);
     r = __builtin_fmaf(n, -1.42860677e-06f, r);
@@ -181,7 +199,8 @@ __device__ __forceinline__ float expf_det(float x)
     p = __builtin_fmaf(p, r, 0.5f);
     p = __builtin_fmaf(p, r, 1.0f);
     p = __builtin_fmaf(p, r, 1.0f);
-    return __int_as_float(__float_as_int(p) + (((int)n) << 23));
+    const float r2 = __int_as_float(__float_as_int(p) + (((int)n) << 23));
+    return tiny ? 0.0f : r2;
 }
 
 // erfc(z), z >= 0: t*exp(-z^2 + P(t)), t = 1/(1+z/2) (Chebyshev fit of Numerical Recipes' erfcc).

@@ -231,7 +231,6 @@ __global__ __launch_bounds__(64 * WGM * WGN, WGPC * WGM * WGN / 4) void igemm_nt
     // of stage s has been read.  Operand fragments and scales of K block k+1 are read from LDS into a second set
     // of registers BEFORE the products of K block k are issued, so the LDS pipe works while the wave multiplies
     // and accumulates; without this all waves of a SIMD queue at the LDS together and then compute together.
-    constexpr int AHEAD = NSTAGE - 1;                         // stages in flight beyond the one being consumed
     constexpr int LOADS = LPW + (EPI != EPI_S32 ? 1 : 0);     // LDS-direct loads per wave and stage
     const int nfull = nkb / KB_STAGE;                         // stages with all KB_STAGE blocks
     const int ktail = nkb - nfull * KB_STAGE;                 // K blocks of the short last stage (0: none)
@@ -253,12 +252,15 @@ __global__ __launch_bounds__(64 * WGM * WGN, WGPC * WGM * WGN / 4) void igemm_nt
     auto fetch = [&](const unsigned pa, const unsigned pb, const unsigned psc, auto slot_bytes_c, auto slot_words_c, auto buf_c) {
         constexpr int BUF = decltype(buf_c)::value;
         constexpr int SB = decltype(slot_bytes_c)::value, SW = decltype(slot_words_c)::value;
+        // the instruction's offset field has 16 bits: slots beyond that are reached through the address register
+        constexpr int HI = (SB + (WBM > WBN ? WBM : WBN) * QB * ROW_BYTES) > 65535 ? SB : 0;
+        const unsigned pa2 = pa + HI, pb2 = pb + HI;
 #pragma unroll
         for (int i = 0; i < WBM; ++i)
-            asm volatile("ds_read_b128 %0, %1 offset:%2" : "=v"(fa_reg[BUF][i]) : "v"(pa), "n"(SB + i * (QB * ROW_BYTES)));
+            asm volatile("ds_read_b128 %0, %1 offset:%2" : "=v"(fa_reg[BUF][i]) : "v"(pa2), "n"(SB - HI + i * (QB * ROW_BYTES)));
 #pragma unroll
         for (int j = 0; j < WBN; ++j)
-            asm volatile("ds_read_b128 %0, %1 offset:%2" : "=v"(fb_reg[BUF][j]) : "v"(pb), "n"(SB + j * (QB * ROW_BYTES)));
+            asm volatile("ds_read_b128 %0, %1 offset:%2" : "=v"(fb_reg[BUF][j]) : "v"(pb2), "n"(SB - HI + j * (QB * ROW_BYTES)));
         if (EPI != EPI_S32) {
             scale_vec &dst = sc_raw[BUF];
             if (NSC == 3) asm volatile("ds_read_b96 %0, %1 offset:%2" : "=v"(dst) : "v"(psc), "n"(SW * 4));
@@ -341,7 +343,6 @@ __global__ __launch_bounds__(64 * WGM * WGN, WGPC * WGM * WGN / 4) void igemm_nt
         else JF_WAIT_VMCNT(0);
     };
     using c0 = std::integral_constant<int, 0>;
-    using c1 = std::integral_constant<int, 1>;
     wait_stage(0, NSTAGE - 1);
     asm volatile("" ::: "memory");
     __builtin_amdgcn_s_barrier();                              // bare: __syncthreads() would drain every load
@@ -493,7 +494,8 @@ __global__ __launch_bounds__(64 * WGM * WGN, WGPC * WGM * WGN / 4) void igemm_nt
                         for (int k = 0; k < 16; ++k) x[k] = x[k] + p.bias[bn + rcol + k];
                     }
 #pragma unroll
-                    for (int k = 0; k < 16; ++k) t[k] = d.div(127.0f * x[k]);
+                    for (int k = 0; k < 16; ++k) x[k] = 127.0f * x[k];
+                    d.div16(x, t);
                     if (p.rounding == JF_ROUND_STOCHASTIC) {
                         float n[16];
                         sr_noise16(p.seed, p.offset, (uint64_t)e0, n);
