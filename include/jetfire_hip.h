@@ -59,8 +59,9 @@ typedef void *jf_stream_t;
 
 const char *jf_error_string(int code);
 
-/* Bytes of device scratch the GEMM entry points need for this problem (0 for JF_B_NK; for
- * JF_B_KN the B operand is re-laid-out K-contiguous first). */
+/* Bytes of device scratch the GEMM entry points need for this problem.  Currently 0 for both layouts (a JF_B_KN
+ * operand is staged as it lies in memory and transposed by the LDS read); callers still ask, and pass what they get,
+ * so that a build that re-lays B out first (JF_ERR_WORKSPACE if the buffer is missing) stays a drop-in. */
 size_t jf_igemm_workspace_bytes(int M, int N, int K, int b_layout);
 
 /* C_s32[M,N] = A[M,K] * B.   Replaces igemm_basic_int8_gemm (include/igemm.h:3-12,

@@ -17,6 +17,7 @@ namespace jf {
 constexpr int QB = 32;        // quantisation block edge
 constexpr int WAVE = 64;
 
+typedef int v2i __attribute__((ext_vector_type(2)));
 typedef int v4i __attribute__((ext_vector_type(4)));
 typedef int v16i __attribute__((ext_vector_type(16)));
 typedef float v4f __attribute__((ext_vector_type(4)));

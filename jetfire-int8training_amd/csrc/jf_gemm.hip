@@ -31,7 +31,7 @@ enum Epilogue { EPI_S32 = 0, EPI_FP = 1, EPI_Q = 2 };
 
 struct GemmArgs {
     const int8_t *A;      // [M, lda]
-    const int8_t *B;      // [N, ldb]   (K-contiguous)
+    const int8_t *B;      // [N, ldb] (K-contiguous) or, for the BKN kernels, [K, ldb] (N-contiguous)
     const void *sa;       // [K/32, M/32]
     const void *sb;       // [K/32, N/32]
     void *C;              // s32 / fp / s8 [M, N]
@@ -79,7 +79,9 @@ template <int I, int N, typename F> __device__ __forceinline__ void static_for(F
 constexpr int WBM = 2, WBN = 1;
 // NSTAGE = depth of the LDS ring (one stage being computed, NSTAGE-1 in flight); WGPC = workgroups per CU
 // (the second launch bound counts waves per SIMD: WGPC workgroups of WGM*WGN waves over 4 SIMDs).
-template <int EPI, typename ST, int WGM, int WGN, int NSTAGE, int WGPC>
+// BKN = 0: B is [N, ldb] (K-contiguous rows, like A).  BKN = 1: B is [K, ldb] (N-contiguous rows); its tile is staged
+// as it lies in memory and the K-contiguous MFMA operand is produced by the transposing LDS read of gfx950.
+template <int EPI, typename ST, int WGM, int WGN, int NSTAGE, int WGPC, int BKN>
 __global__ __launch_bounds__(64 * WGM * WGN, WGPC * WGM * WGN / 4) void igemm_nt_kernel(GemmArgs p)
 {
     constexpr int NW = WGM * WGN;
@@ -90,7 +92,7 @@ __global__ __launch_bounds__(64 * WGM * WGN, WGPC * WGM * WGN / 4) void igemm_nt
     constexpr int LPW = GROUPS / NW;                         // LDS-direct loads per wave per stage
     static_assert(GROUPS % NW == 0, "stage must split evenly over the waves");
     static_assert(NSTAGE >= 2 && NSTAGE <= 5, "ring depth");
-    static_assert((BM + BN) / QB <= 16, "scale patch holds 16 blocks per K block");
+    static_assert(!BKN || (BN == ROW_BYTES && WBN == 1), "a staged [K,N] row is one 128-byte LDS row");
 
     extern __shared__ __attribute__((aligned(16))) unsigned char smem[];
     typedef __attribute__((address_space(3))) unsigned char lds_u8;
@@ -120,16 +122,26 @@ __global__ __launch_bounds__(64 * WGM * WGN, WGPC * WGM * WGN / 4) void igemm_nt
     const int lrow = lane >> 3;
     const int gchunk = (lane & 7) ^ (((wave & 1) * 4 + (lane >> 4)) & 7);     // global chunk this lane fetches
     const unsigned loff_a = (unsigned)lrow * (unsigned)p.lda + gchunk * 16;
-    const unsigned loff_b = (unsigned)lrow * (unsigned)p.ldb + gchunk * 16;
-    const int8_t *gbase[LPW];      // wave-uniform: first byte of the group's first row
+    // B as [K,N]: a load moves 8 K rows x 128 N bytes (group g of a stage = K rows 8g .. 8g+7 of the stage).  Slot c'
+    // of row r holds global chunk c' ^ r, which makes the transposing reads below conflict-free.  Chunks beyond N (partial
+    // tile) fetch the tile's first chunk instead (never used).
+    const int kn_chunk = (n0 + (((lane & 7) ^ lrow) << 4)) < p.N ? ((lane & 7) ^ lrow) : 0;
+    const unsigned loff_b = BKN ? (unsigned)lrow * (unsigned)p.ldb + kn_chunk * 16
+                                : (unsigned)lrow * (unsigned)p.ldb + gchunk * 16;
+    const int8_t *gbase[LPW];      // wave-uniform: first byte of the group's first row (stage 0)
     bool is_a[LPW];
 #pragma unroll
     for (int j = 0; j < LPW; ++j) {
         const int grp = wave + j * NW;
         is_a[j] = grp < BM / 8;
-        int r0 = (is_a[j] ? m0 : n0) + (is_a[j] ? grp : grp - BM / 8) * 8;
-        if (r0 >= (is_a[j] ? p.M : p.N)) r0 = is_a[j] ? m0 : n0;   // groups of a partial tile: any valid group
-        gbase[j] = (is_a[j] ? p.A : p.B) + (size_t)r0 * (size_t)(is_a[j] ? p.lda : p.ldb);
+        if (BKN && !is_a[j]) {
+            const int k0 = (grp - BM / 8) * 8;                     // K row of the stage (redirected at issue time if beyond K)
+            gbase[j] = p.B + (size_t)k0 * (size_t)p.ldb + n0;
+        } else {
+            int r0 = (is_a[j] ? m0 : n0) + (is_a[j] ? grp : grp - BM / 8) * 8;
+            if (r0 >= (is_a[j] ? p.M : p.N)) r0 = is_a[j] ? m0 : n0;   // groups of a partial tile: any valid group
+            gbase[j] = (is_a[j] ? p.A : p.B) + (size_t)r0 * (size_t)(is_a[j] ? p.lda : p.ldb);
+        }
     }
     // Scales of a stage: every wave fetches, again LDS-direct, the scales it needs itself into a private 256-byte
     // patch (lane l: K block l/16; word l%16 = the wave's WBM A-side scales, then its WBN B-side scales, the rest
@@ -175,12 +187,19 @@ __global__ __launch_bounds__(64 * WGM * WGN, WGPC * WGM * WGN / 4) void igemm_nt
         unsigned la = loff_a, lb = loff_b;
         if (!FULL && kb0 + (gchunk >> 1) >= nkb) {            // chunks of missing K blocks: the stage's first block again
             la -= (unsigned)(gchunk >> 1) * QB;
-            lb -= (unsigned)(gchunk >> 1) * QB;
+            if (!BKN) lb -= (unsigned)(gchunk >> 1) * QB;
         }
 #pragma unroll
         for (int j = 0; j < LPW; ++j) {
             const int grp = wave + j * NW;
-            const int8_t *base = gbase[j] + (size_t)kb0 * QB;  // wave-uniform
+            const int8_t *base;                                // wave-uniform
+            if (BKN && j >= A_LOADS) {
+                base = gbase[j] + (size_t)kb0 * QB * (size_t)p.ldb;
+                // K rows of a missing K block: the stage's first group again
+                if (!FULL && kb0 * QB + (grp - BM / 8) * 8 >= p.K) base -= (size_t)((grp - BM / 8) * 8) * (size_t)p.ldb;
+            } else {
+                base = gbase[j] + (size_t)kb0 * QB;
+            }
             asm volatile("s_mov_b32 m0, %2\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %0, %1"
                          ::"v"(j < A_LOADS ? la : lb), "s"(base), "s"(slot_lds + (unsigned)grp * 1024u) : "memory", "m0");
         }
@@ -201,6 +220,17 @@ __global__ __launch_bounds__(64 * WGM * WGN, WGPC * WGM * WGN / 4) void igemm_nt
         const unsigned fo = (lane & 31) * ROW_BYTES + (((2 * kb + (lane >> 5)) ^ ((lane >> 1) & 7)) << 4);
         fa_u[kb] = (unsigned)(uintptr_t)lds + fo + (wm * WBM * QB) * ROW_BYTES;
         fb_u[kb] = (unsigned)(uintptr_t)lds + A_BYTES + fo + (wn * WBN * QB) * ROW_BYTES;
+    }
+    // B staged as [K,N]: ds_read_b64_tr_b8 works on groups of 16 lanes; lane i of a group receives byte (i & 7) of the
+    // 8-byte rows addressed by lanes (i>>3), (i>>3)+2, ... (i>>3)+14 of the group.  Lanes 2q and 2q+1 address K row q
+    // of an 8-row group at N bytes 0..7 and 8..15 of a 16-column strip, so lane i gets 8 consecutive K values of
+    // column i: the MFMA operand (lane l: column l%32, K bytes 16*(l/32) .. +15) is two such reads (K rows +0..7, +8..15).
+    // The K block and the half are immediates, so one address register serves all of a stage.
+    unsigned fb_kn = 0;
+    if (BKN) {
+        const int g = lane >> 4, r = lane & 15, rho = r >> 1;
+        const int c = 2 * wn * WBN + (g & 1);                                    // 16-byte chunk of the N strip
+        fb_kn = (unsigned)(uintptr_t)lds + A_BYTES + (g >> 1) * 2048 + ((rho * 8 + (c ^ rho)) << 4) + 8 * (r & 1);
     }
     // scale patch of this wave: a uniform address, parked in a vector register once (LDS reads take a VGPR address)
     unsigned sc_v;
@@ -245,11 +275,12 @@ __global__ __launch_bounds__(64 * WGM * WGN, WGPC * WGM * WGN / 4) void igemm_nt
     typedef float scale_vec __attribute__((ext_vector_type(NSC == 3 ? 3 : NSC <= 2 ? 2 : 4)));
     v4i fa_reg[2][WBM], fb_reg[2][WBN];
     scale_vec sc_raw[2];
-    constexpr int FETCH_OPS = WBM + WBN + (EPI != EPI_S32 ? 1 : 0);
+    constexpr int FETCH_OPS = WBM + (BKN ? 2 : 1) * WBN + (EPI != EPI_S32 ? 1 : 0);
     static_assert(2 * FETCH_OPS <= 15, "lgkmcnt is a 4-bit counter");
     // pa/pb: this lane's fragment addresses for the K block (ring slot 0); psc: the wave's scale patch;
     // slot_bytes / slot_words: compile-time offset of the ring slot in the tile ring and of the K block in the patch
-    auto fetch = [&](const unsigned pa, const unsigned pb, const unsigned psc, auto slot_bytes_c, auto slot_words_c, auto buf_c) {
+    auto fetch = [&](const unsigned pa, const unsigned pb, const unsigned pbkn, const unsigned psc, auto slot_bytes_c,
+                     auto kn_off_c, auto slot_words_c, auto buf_c) {
         constexpr int BUF = decltype(buf_c)::value;
         constexpr int SB = decltype(slot_bytes_c)::value, SW = decltype(slot_words_c)::value;
         // the instruction's offset field has 16 bits: slots beyond that are reached through the address register
@@ -258,9 +289,17 @@ __global__ __launch_bounds__(64 * WGM * WGN, WGPC * WGM * WGN / 4) void igemm_nt
 #pragma unroll
         for (int i = 0; i < WBM; ++i)
             asm volatile("ds_read_b128 %0, %1 offset:%2" : "=v"(fa_reg[BUF][i]) : "v"(pa2), "n"(SB - HI + i * (QB * ROW_BYTES)));
+        if (BKN) {
+            constexpr int KO = decltype(kn_off_c)::value;     // slot + K block offset of the [K,N] staging
+            v2i lo, hi;
+            asm volatile("ds_read_b64_tr_b8 %0, %1 offset:%2" : "=v"(lo) : "v"(pbkn), "n"(KO));
+            asm volatile("ds_read_b64_tr_b8 %0, %1 offset:%2" : "=v"(hi) : "v"(pbkn), "n"(KO + 1024));
+            fb_reg[BUF][0] = v4i{lo.x, lo.y, hi.x, hi.y};
+        } else {
 #pragma unroll
-        for (int j = 0; j < WBN; ++j)
-            asm volatile("ds_read_b128 %0, %1 offset:%2" : "=v"(fb_reg[BUF][j]) : "v"(pb2), "n"(SB - HI + j * (QB * ROW_BYTES)));
+            for (int j = 0; j < WBN; ++j)
+                asm volatile("ds_read_b128 %0, %1 offset:%2" : "=v"(fb_reg[BUF][j]) : "v"(pb2), "n"(SB - HI + j * (QB * ROW_BYTES)));
+        }
         if (EPI != EPI_S32) {
             scale_vec &dst = sc_raw[BUF];
             if (NSC == 3) asm volatile("ds_read_b96 %0, %1 offset:%2" : "=v"(dst) : "v"(psc), "n"(SW * 4));
@@ -347,7 +386,7 @@ __global__ __launch_bounds__(64 * WGM * WGN, WGPC * WGM * WGN / 4) void igemm_nt
     asm volatile("" ::: "memory");
     __builtin_amdgcn_s_barrier();                              // bare: __syncthreads() would drain every load
     asm volatile("" ::: "memory");
-    fetch(fa_u[0], fb_u[0], sc_v, c0{}, c0{}, c0{});
+    fetch(fa_u[0], fb_u[0], fb_kn, sc_v, c0{}, c0{}, c0{}, c0{});
 
     for (int s0 = 0; s0 < nfull; s0 += NSTAGE) static_for<0, NSTAGE>([&](auto slot_c) {
         constexpr int SLOT = decltype(slot_c)::value;         // ring slot of this stage, a compile-time constant
@@ -370,10 +409,12 @@ __global__ __launch_bounds__(64 * WGM * WGN, WGPC * WGM * WGN / 4) void igemm_nt
                     if (s + NSTAGE < nstages) issue_stage(s + NSTAGE);
                 }
                 // unconditional: past the last stage it reads bytes of the ring that nobody uses
-                fetch(fa_u[0], fb_u[0], sc_v, std::integral_constant<int, NEXT_SLOT * STAGE_BYTES>{},
+                fetch(fa_u[0], fb_u[0], fb_kn, sc_v, std::integral_constant<int, NEXT_SLOT * STAGE_BYTES>{},
+                      std::integral_constant<int, NEXT_SLOT * STAGE_BYTES>{},
                       std::integral_constant<int, NEXT_SLOT * 64>{}, std::integral_constant<int, NXT>{});
             } else {
-                fetch(fa_u[kb + 1], fb_u[kb + 1], sc_v, std::integral_constant<int, SLOT * STAGE_BYTES>{},
+                fetch(fa_u[kb + 1], fb_u[kb + 1], fb_kn, sc_v, std::integral_constant<int, SLOT * STAGE_BYTES>{},
+                      std::integral_constant<int, SLOT * STAGE_BYTES + (kb + 1) * 4096>{},
                       std::integral_constant<int, SLOT * 64 + (kb + 1) * 16>{}, std::integral_constant<int, NXT>{});
             }
             fetched(std::integral_constant<int, FETCH_OPS>{}, std::integral_constant<int, CUR>{});
@@ -390,8 +431,9 @@ __global__ __launch_bounds__(64 * WGM * WGN, WGPC * WGM * WGN / 4) void igemm_nt
             constexpr int CUR = kb & 1;
             if (kb < ktail) {
                 if (kb > 0)
-                    fetch(fa_u[kb] + slot * STAGE_BYTES, fb_u[kb] + slot * STAGE_BYTES, sc_v + slot * 256,
-                          c0{}, std::integral_constant<int, kb * 16>{}, std::integral_constant<int, CUR>{});
+                    fetch(fa_u[kb] + slot * STAGE_BYTES, fb_u[kb] + slot * STAGE_BYTES, fb_kn + slot * STAGE_BYTES, sc_v + slot * 256,
+                          c0{}, std::integral_constant<int, kb * 4096>{}, std::integral_constant<int, kb * 16>{},
+                          std::integral_constant<int, CUR>{});
                 fetched(c0{}, std::integral_constant<int, CUR>{});
                 compute(std::integral_constant<int, CUR>{}, nfull * KB_STAGE + kb);
             }
@@ -564,7 +606,7 @@ static int launch_transpose(const int8_t *in, int R, int C, int8_t *out, hipStre
     return (int)hipGetLastError();
 }
 
-template <int EPI, typename ST, int WGM, int WGN, int NSTAGE, int WGPC>
+template <int EPI, typename ST, int WGM, int WGN, int NSTAGE, int WGPC, int BKN>
 static int launch_gemm_cfg(const GemmArgs &a, hipStream_t st)
 {
     constexpr int BM = QB * WBM * WGM, BN = QB * WBN * WGN, NT = 64 * WGM * WGN;
@@ -574,7 +616,7 @@ static int launch_gemm_cfg(const GemmArgs &a, hipStream_t st)
     GemmArgs p = a;
     p.tiles_m = (p.M + BM - 1) / BM;
     p.tiles_n = (p.N + BN - 1) / BN;
-    auto kern = igemm_nt_kernel<EPI, ST, WGM, WGN, NSTAGE, WGPC>;
+    auto kern = igemm_nt_kernel<EPI, ST, WGM, WGN, NSTAGE, WGPC, BKN>;
     // more than 64 KiB of dynamic LDS has to be opted into, per function
     hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void *>(kern), hipFuncAttributeMaxDynamicSharedMemorySize, SMEM);
     if (e != hipSuccess) return (int)e;
@@ -584,18 +626,22 @@ static int launch_gemm_cfg(const GemmArgs &a, hipStream_t st)
 
 // Tile configuration.  JF_GEMM_CFG selects it at build time (for experiments); the default is 128x128 tiles,
 // 8 waves, a 2-deep ring and two workgroups per CU (the epilogue of one overlaps the main loop of the other).
+// The default configuration reads a [K,N] B operand in place; the experimental one transposes it into the
+// caller's workspace first.
 #ifndef JF_GEMM_CFG
 #define JF_GEMM_CFG 0
 #endif
-template <int EPI, typename ST> static int launch_gemm(const GemmArgs &a, hipStream_t st)
+constexpr bool KN_NATIVE = (JF_GEMM_CFG == 0);
+template <int EPI, typename ST> static int launch_gemm(const GemmArgs &a, hipStream_t st, bool b_kn)
 {
 #if JF_GEMM_CFG == 0
-    return launch_gemm_cfg<EPI, ST, 2, 4, 2, 2>(a, st);
+    return b_kn ? launch_gemm_cfg<EPI, ST, 2, 4, 2, 2, 1>(a, st) : launch_gemm_cfg<EPI, ST, 2, 4, 2, 2, 0>(a, st);
 #else
     // 256x128 or 128x256, whichever pads the problem less (1600 = 12.5 x 128 but 6.25 x 256); 16 waves, 3-deep ring
+    (void)b_kn;
     auto padded = [](long d, long t) { return (d + t - 1) / t * t; };
     const long tall = padded(a.M, 256) * padded(a.N, 128), wide = padded(a.M, 128) * padded(a.N, 256);
-    return tall <= wide ? launch_gemm_cfg<EPI, ST, 4, 4, 3, 1>(a, st) : launch_gemm_cfg<EPI, ST, 2, 8, 3, 1>(a, st);
+    return tall <= wide ? launch_gemm_cfg<EPI, ST, 4, 4, 3, 1, 0>(a, st) : launch_gemm_cfg<EPI, ST, 2, 8, 3, 1, 0>(a, st);
 #endif
 }
 
@@ -606,20 +652,24 @@ static int check_gemm_common(const void *A, const void *B, const void *C, int M,
     if (!mult32(M) || !mult32(N) || !mult32(K)) return JF_ERR_SHAPE;
     if (b_layout != JF_B_NK && b_layout != JF_B_KN) return JF_ERR_ENUM;
     if (!aligned16(A) || !aligned16(B) || !aligned16(C)) return JF_ERR_ALIGN;
-    if (b_layout == JF_B_KN) {
+    if (b_layout == JF_B_KN && !KN_NATIVE) {
         if (!ws || ws_bytes < (size_t)N * (size_t)K) return JF_ERR_WORKSPACE;
         if (!aligned16(ws)) return JF_ERR_ALIGN;
     }
     return JF_OK;
 }
 
-// B as [N,K]: either the caller's buffer or its transpose in the workspace.
-static int b_as_nk(const int8_t *&B, int N, int K, int b_layout, void *ws, hipStream_t st)
+// Prepares the B operand: returns true if the kernel is to read it as [K,N] in place (leading dimension N);
+// otherwise B is [N,K] (the caller's buffer, or its transpose in the workspace) with leading dimension K.
+static bool prepare_b(const int8_t *&B, int &ldb, int N, int K, int b_layout, void *ws, hipStream_t st, int &rc)
 {
-    if (b_layout == JF_B_NK) return JF_OK;
-    int rc = launch_transpose(B, K, N, reinterpret_cast<int8_t *>(ws), st);
+    rc = JF_OK;
+    ldb = K;
+    if (b_layout == JF_B_NK) return false;
+    if (KN_NATIVE) { ldb = N; return true; }
+    rc = launch_transpose(B, K, N, reinterpret_cast<int8_t *>(ws), st);
     B = reinterpret_cast<const int8_t *>(ws);
-    return rc;
+    return false;
 }
 
 }  // namespace jf
@@ -645,7 +695,7 @@ const char *jf_error_string(int code)
 size_t jf_igemm_workspace_bytes(int M, int N, int K, int b_layout)
 {
     (void)M;
-    return b_layout == JF_B_KN ? (size_t)N * (size_t)K : 0;
+    return (b_layout == JF_B_KN && !KN_NATIVE) ? (size_t)N * (size_t)K : 0;
 }
 
 int jf_igemm_s32(const int8_t *A, const int8_t *B, int32_t *C, int M, int N, int K, int b_layout,
@@ -654,10 +704,12 @@ int jf_igemm_s32(const int8_t *A, const int8_t *B, int32_t *C, int M, int N, int
     int rc = check_gemm_common(A, B, C, M, N, K, b_layout, workspace, workspace_bytes);
     if (rc) return rc;
     hipStream_t st = (hipStream_t)stream;
-    if ((rc = b_as_nk(B, N, K, b_layout, workspace, st))) return rc;
+    int ldb;
+    const bool kn = prepare_b(B, ldb, N, K, b_layout, workspace, st, rc);
+    if (rc) return rc;
     GemmArgs a = {};
-    a.A = A; a.B = B; a.C = C; a.M = M; a.N = N; a.K = K; a.lda = K; a.ldb = K;
-    return launch_gemm<EPI_S32, float>(a, st);
+    a.A = A; a.B = B; a.C = C; a.M = M; a.N = N; a.K = K; a.lda = K; a.ldb = ldb;
+    return launch_gemm<EPI_S32, float>(a, st, kn);
 }
 
 int jf_igemm_block_acc(const int8_t *A, const int8_t *B, int32_t *acc, int M, int N, int K, int b_layout,
@@ -666,12 +718,14 @@ int jf_igemm_block_acc(const int8_t *A, const int8_t *B, int32_t *acc, int M, in
     int rc = check_gemm_common(A, B, acc, M, N, K, b_layout, workspace, workspace_bytes);
     if (rc) return rc;
     hipStream_t st = (hipStream_t)stream;
-    if ((rc = b_as_nk(B, N, K, b_layout, workspace, st))) return rc;
+    int ldb;
+    const bool kn = prepare_b(B, ldb, N, K, b_layout, workspace, st, rc);
+    if (rc) return rc;
     for (int kb = 0; kb < K / QB; ++kb) {
         GemmArgs a = {};
-        a.A = A + kb * QB; a.B = B + kb * QB; a.C = acc + (size_t)kb * M * N;
-        a.M = M; a.N = N; a.K = QB; a.lda = K; a.ldb = K;
-        if ((rc = launch_gemm<EPI_S32, float>(a, st))) return rc;
+        a.A = A + kb * QB; a.B = kn ? B + (size_t)kb * QB * N : B + kb * QB; a.C = acc + (size_t)kb * M * N;
+        a.M = M; a.N = N; a.K = QB; a.lda = K; a.ldb = ldb;
+        if ((rc = launch_gemm<EPI_S32, float>(a, st, kn))) return rc;
     }
     return JF_OK;
 }
@@ -686,11 +740,13 @@ int jf_igemm_block_fp(const int8_t *A, const int8_t *B, const void *sa, const vo
     if ((scale_dtype != JF_SCALE_F16 && scale_dtype != JF_SCALE_F32) ||
         (out_dtype != JF_FP_F16 && out_dtype != JF_FP_F32 && out_dtype != JF_FP_BF16)) return JF_ERR_ENUM;
     hipStream_t st = (hipStream_t)stream;
-    if ((rc = b_as_nk(B, N, K, b_layout, workspace, st))) return rc;
+    int ldb;
+    const bool kn = prepare_b(B, ldb, N, K, b_layout, workspace, st, rc);
+    if (rc) return rc;
     GemmArgs a = {};
-    a.A = A; a.B = B; a.sa = sa; a.sb = sb; a.C = C; a.M = M; a.N = N; a.K = K; a.lda = K; a.ldb = K;
+    a.A = A; a.B = B; a.sa = sa; a.sb = sb; a.C = C; a.M = M; a.N = N; a.K = K; a.lda = K; a.ldb = ldb;
     a.out_dtype = out_dtype;
-    return scale_dtype == JF_SCALE_F16 ? launch_gemm<EPI_FP, half_t>(a, st) : launch_gemm<EPI_FP, float>(a, st);
+    return scale_dtype == JF_SCALE_F16 ? launch_gemm<EPI_FP, half_t>(a, st, kn) : launch_gemm<EPI_FP, float>(a, st, kn);
 }
 
 int jf_igemm_block_q(const int8_t *A, const int8_t *B, const void *sa, const void *sb,
@@ -705,11 +761,13 @@ int jf_igemm_block_q(const int8_t *A, const int8_t *B, const void *sa, const voi
     if ((scale_dtype != JF_SCALE_F16 && scale_dtype != JF_SCALE_F32) ||
         (rounding != JF_ROUND_NEAREST && rounding != JF_ROUND_STOCHASTIC)) return JF_ERR_ENUM;
     hipStream_t st = (hipStream_t)stream;
-    if ((rc = b_as_nk(B, N, K, b_layout, workspace, st))) return rc;
+    int ldb;
+    const bool kn = prepare_b(B, ldb, N, K, b_layout, workspace, st, rc);
+    if (rc) return rc;
     GemmArgs a = {};
     a.A = A; a.B = B; a.sa = sa; a.sb = sb; a.C = C; a.sc = sc; a.bias = bias; a.biasmax = biasmax;
-    a.M = M; a.N = N; a.K = K; a.lda = K; a.ldb = K; a.rounding = rounding; a.seed = seed; a.offset = offset;
-    return scale_dtype == JF_SCALE_F16 ? launch_gemm<EPI_Q, half_t>(a, st) : launch_gemm<EPI_Q, float>(a, st);
+    a.M = M; a.N = N; a.K = K; a.lda = K; a.ldb = ldb; a.rounding = rounding; a.seed = seed; a.offset = offset;
+    return scale_dtype == JF_SCALE_F16 ? launch_gemm<EPI_Q, half_t>(a, st, kn) : launch_gemm<EPI_Q, float>(a, st, kn);
 }
 
 int jf_transpose_s8(const int8_t *in, int R, int C, int8_t *out, jf_stream_t stream)
