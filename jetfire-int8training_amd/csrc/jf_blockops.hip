@@ -315,40 +315,55 @@ __global__ __launch_bounds__(NT) void rowstats_kernel(const int8_t *q, const ST 
     }
 }
 
-// Sum of 32 per-lane values over the 32 lanes that share (lane & 1): a halving butterfly over lane bits 5..1.
-// On return lane l holds the total of value index  ((l>>5)&1)*16 + ((l>>4)&1)*8 + ((l>>3)&1)*4 + ((l>>2)&1)*2 + ((l>>1)&1).
-__device__ __forceinline__ float reduce32_over_rows(float (&v)[32], int lane)
+// Column sums over the 32 rows of a block: lane l holds row l/2 and 32 values (index i) of column set l%2.  The 8 lanes
+// of a 16-lane row that share l%2 are summed by rotations inside the vector ALU (+2, +4, +8 lanes), the four rows
+// through a small LDS patch.  On return lane l holds the total of value index l/2 for column set l%2
+// (a fixed tree: reproducible).  `patch` = 256 floats private to the wave.
+__device__ __forceinline__ float colsum32_over_rows(const float (&v)[32], int lane, float *patch)
 {
-#define JF_BFLY(N, MASK)                                                   \
-    {                                                                      \
-        const bool up = (lane & (MASK)) != 0;                              \
-        _Pragma("unroll") for (int i = 0; i < (N) / 2; ++i) {              \
-            const float send = up ? v[i] : v[(N) / 2 + i];                 \
-            const float keep = up ? v[(N) / 2 + i] : v[i];                 \
-            v[i] = keep + __shfl_xor(send, (MASK), WAVE);                  \
-        }                                                                  \
+    auto rot_add = [](float x, auto ctrl_c) {
+        const int t = __builtin_amdgcn_update_dpp(0, __float_as_int(x), decltype(ctrl_c)::value, 0xF, 0xF, false);
+        return x + __int_as_float(t);
+    };
+    const int row = lane >> 4, set = lane & 1;
+#pragma unroll
+    for (int i = 0; i < 32; ++i) {
+        float x = v[i];
+        x = rot_add(x, std::integral_constant<int, 0x122>{});      // row_ror:2
+        x = rot_add(x, std::integral_constant<int, 0x124>{});      // row_ror:4
+        x = rot_add(x, std::integral_constant<int, 0x128>{});      // row_ror:8
+        if ((lane & 15) < 2) patch[(row * 2 + set) * 32 + i] = x;  // one lane per (row of lanes, column set)
     }
-    JF_BFLY(32, 32) JF_BFLY(16, 16) JF_BFLY(8, 8) JF_BFLY(4, 4) JF_BFLY(2, 2)
-#undef JF_BFLY
-    return v[0];
+    __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
+    __builtin_amdgcn_wave_barrier();
+    __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
+    const int i = lane >> 1;
+    const float total = ((patch[(0 * 2 + set) * 32 + i] + patch[(1 * 2 + set) * 32 + i]) +
+                         (patch[(2 * 2 + set) * 32 + i] + patch[(3 * 2 + set) * 32 + i]));
+    __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
+    __builtin_amdgcn_wave_barrier();                               // the patch may be rewritten
+    return total;
 }
 
-// LayerNorm backward, pass 1.  One workgroup (16 waves) per 32-row strip; the waves take the column blocks
-// round-robin.  Per row: 16-column partial sums of xhat*wdy (fmaf chain) and wdy (add chain) go to LDS, then one
-// lane per row adds all C/16 partials in ascending order -> c1 = sum/C, c2 = sum/C (a defined order, so the
-// requantised dx is bit-reproducible).  Also the strip's column sums of dy*xhat and dy (partial dgamma / dbeta,
-// reduced over strips by colsum_kernel), by a butterfly over the 32 rows of the block.
 constexpr int LNB_THREADS = 1024;
+// LayerNorm backward in one launch (layernorm.py:197-402): one workgroup (16 waves) per 32-row strip; the waves take
+// the column blocks round-robin.  Row reductions in a defined order (per row: 16-column partial sums of xhat*wdy as an
+// fmaf chain and of wdy as an add chain go to LDS, then one lane per row adds all C/16 partials in ascending order ->
+// c1, c2, so the requantised dx is bit-reproducible); then dx is computed and requantised.  The strip (2 x 32 x C bytes) is read a second time for that, from the L2 it was just fetched
+// into (keeping it in registers instead does not fit next to the column-sum butterfly).  Also the strip's column sums
+// for dgamma / dbeta.
 template <typename ST>
-__global__ __launch_bounds__(LNB_THREADS) void layernorm_bwd_stats_kernel(const int8_t *qx, const ST *sx, const int8_t *qg,
+__global__ __launch_bounds__(LNB_THREADS) void layernorm_bwd_fused_kernel(const int8_t *qx, const ST *sx, const int8_t *qg,
                                                                           const ST *sg, const float *gamma, const float *mean,
-                                                                          const float *rstd, int R, int C, float *c1, float *c2,
+                                                                          const float *rstd, int R, int C, int rounding,
+                                                                          uint64_t seed, uint64_t offset, int8_t *qdx, ST *sdx,
                                                                           float *pdg, float *pdb)
 {
-    extern __shared__ float fsm[];                // part1[32][C/16], part2[32][C/16]
+    extern __shared__ float fsm[];                // part1[32][C/16], part2[32][C/16], c1[32], c2[32], column-sum patches
     const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
     const int SC = C / QB, H = C / 16, rb = blockIdx.x;
-    float *part1 = fsm, *part2 = fsm + QB * H;
+    float *part1 = fsm, *part2 = fsm + QB * H, *c1s = part2 + QB * H, *c2s = c1s + QB;
+    float *cpatch = c2s + QB + wave * 256;
     const int r = lane >> 1;
     const float mu = mean[rb * QB + r], rs = rstd[rb * QB + r];
     for (int cb = wave; cb < SC; cb += LNB_THREADS / WAVE) {
@@ -371,9 +386,8 @@ __global__ __launch_bounds__(LNB_THREADS) void layernorm_bwd_stats_kernel(const 
         part1[r * H + cb * 2 + (lane & 1)] = p1;
         part2[r * H + cb * 2 + (lane & 1)] = p2;
         if (pdg) {
-            const float total = reduce32_over_rows(v, lane);
-            const int idx = ((lane >> 5) & 1) * 16 + ((lane >> 4) & 1) * 8 + ((lane >> 3) & 1) * 4 + ((lane >> 2) & 1) * 2 +
-                            ((lane >> 1) & 1);
+            const float total = colsum32_over_rows(v, lane, cpatch);
+            const int idx = lane >> 1;                             // 0..15: sum of dy*xhat, 16..31: sum of dy
             float *dst = (idx & 16) ? pdb : pdg;
             dst[(size_t)rb * C + cb * QB + (lane & 1) * 16 + (idx & 15)] = total;
         }
@@ -383,27 +397,18 @@ __global__ __launch_bounds__(LNB_THREADS) void layernorm_bwd_stats_kernel(const 
         const int rr = threadIdx.x;
         float t1 = 0.0f, t2 = 0.0f;
         for (int h = 0; h < H; ++h) { t1 = t1 + part1[rr * H + h]; t2 = t2 + part2[rr * H + h]; }
-        c1[rb * QB + rr] = t1 / (float)C;
-        c2[rb * QB + rr] = t2 / (float)C;
+        c1s[rr] = t1 / (float)C;
+        c2s[rr] = t2 / (float)C;
     }
-}
-
-// LayerNorm backward, pass 2: dx = (wdy - fmaf(xhat, c1, c2)) * rstd, requantised (layernorm.py:197-402).
-template <typename ST>
-__global__ __launch_bounds__(NT) void layernorm_bwd_dx_kernel(const int8_t *qx, const ST *sx, const int8_t *qg,
-                                                              const ST *sg, const float *gamma, const float *mean,
-                                                              const float *rstd, const float *c1, const float *c2,
-                                                              int R, int C, int rounding, uint64_t seed, uint64_t offset,
-                                                              int8_t *qdx, ST *sdx)
-{
-    JF_FOR_EACH_BLOCK(R, C)
-    {
-        BlockPos pos(blk, SC, C, lane);
+    __syncthreads();
+    const float k1 = c1s[r], k2 = c2s[r];
+    for (int cb = wave; cb < SC; cb += LNB_THREADS / WAVE) {
+        const int col = cb * QB + (lane & 1) * 16;
+        const size_t e0 = (size_t)(rb * QB + r) * C + col;
         float x[16], g[16], w[16];
-        unpack16(*reinterpret_cast<const v4i *>(qx + pos.e0), load_scale(sx, pos.rb * SC + pos.cb), x);
-        unpack16(*reinterpret_cast<const v4i *>(qg + pos.e0), load_scale(sg, pos.rb * SC + pos.cb), g);
-        Load16<float>::run(gamma + pos.col, w);
-        const float mu = mean[pos.row], rs = rstd[pos.row], k1 = c1[pos.row], k2 = c2[pos.row];
+        unpack16(*reinterpret_cast<const v4i *>(qx + e0), load_scale(sx, rb * SC + cb), x);
+        unpack16(*reinterpret_cast<const v4i *>(qg + e0), load_scale(sg, rb * SC + cb), g);
+        Load16<float>::run(gamma + col, w);
 #pragma unroll
         for (int k = 0; k < 16; ++k) {
             const float xh = (x[k] - mu) * rs;
@@ -411,17 +416,21 @@ __global__ __launch_bounds__(NT) void layernorm_bwd_dx_kernel(const int8_t *qx, 
             x[k] = (wdy - __builtin_fmaf(xh, k1, k2)) * rs;
         }
         float scale;
-        v4i codes = quantize16(x, 0.0f, rounding, seed, offset, pos.e0, &scale);
-        *reinterpret_cast<v4i *>(qdx + pos.e0) = codes;
-        if (lane == 0) store_scale(sdx, pos.rb * SC + pos.cb, scale);
+        v4i codes = quantize16(x, 0.0f, rounding, seed, offset, e0, &scale);
+        *reinterpret_cast<v4i *>(qdx + e0) = codes;
+        if (lane == 0) store_scale(sdx, rb * SC + cb, scale);
     }
 }
 
 // out[c] = sum over strips of part[strip][c]   (layernorm.py:405-428).  64 columns per workgroup, 16 strip lanes
 // per column (fixed partition and a fixed tree, so the result is reproducible).
-__global__ __launch_bounds__(1024) void colsum_kernel(const float *part, int strips, int C, float *out)
+__global__ __launch_bounds__(1024) void colsum_kernel(const float *part0, float *out0, const float *part1, float *out1,
+                                                      int strips, int C)
 {
     __shared__ float red[16][65];
+    const float *part = blockIdx.y ? part1 : part0;
+    float *out = blockIdx.y ? out1 : out0;
+    if (!out) return;                                              // uniform
     const int tx = threadIdx.x & 63, ty = threadIdx.x >> 6;
     const int c = blockIdx.x * 64 + tx;
     float a = 0.0f;
@@ -586,25 +595,29 @@ int jf_layernorm_bwd(const int8_t *qx, const void *sx, const int8_t *qg, const v
     if (!aligned16(qdx) || !aligned16(gamma)) return JF_ERR_ALIGN;
     if (!workspace || workspace_bytes < jf_layernorm_bwd_workspace_bytes(R, C)) return JF_ERR_WORKSPACE;
     if (!aligned16(workspace)) return JF_ERR_ALIGN;
-    const size_t smem = (size_t)2 * QB * (C / 16) * sizeof(float);
-    if (smem > 64 * 1024) return JF_ERR_SHAPE;                 // rows of up to 4096 columns
+    // LDS: two [32][C/16] partial-sum arrays, c1/c2, one 1 KiB column-sum patch per wave
+    const size_t smem = ((size_t)2 * QB * (C / 16) + 2 * QB + (LNB_THREADS / WAVE) * 256) * sizeof(float);
+    if (smem > 160 * 1024 - 512) return JF_ERR_SHAPE;          // rows of up to ~8000 columns
     hipStream_t st = (hipStream_t)stream;
-    float *c1 = (float *)workspace, *c2 = c1 + R;
     const bool want_dw = dgamma || dbeta;
-    float *pdg = want_dw ? c2 + R : nullptr, *pdb = want_dw ? pdg + (size_t)(R / QB) * C : nullptr;
-    const int grid = grid_for_blocks(R, C);
-#define JF_LNB(ST)                                                                                                   \
-    do {                                                                                                             \
-        hipLaunchKernelGGL(layernorm_bwd_stats_kernel<ST>, dim3(R / QB), dim3(LNB_THREADS), smem, st, qx, (const ST *)sx, qg, \
-                           (const ST *)sg, gamma, mean, rstd, R, C, c1, c2, pdg, pdb);                               \
-        hipLaunchKernelGGL(layernorm_bwd_dx_kernel<ST>, dim3(grid), dim3(NT), 0, st, qx, (const ST *)sx, qg,          \
-                           (const ST *)sg, gamma, mean, rstd, c1, c2, R, C, rounding, seed, offset, qdx, (ST *)sdx);  \
+    // workspace: [2R floats, unused by this implementation][strips x C partial dgamma][strips x C partial dbeta]
+    float *pdg = want_dw ? (float *)workspace + (size_t)2 * R : nullptr, *pdb = want_dw ? pdg + (size_t)(R / QB) * C : nullptr;
+#define JF_LNF(ST)                                                                                                    \
+    do {                                                                                                              \
+        auto kern = layernorm_bwd_fused_kernel<ST>;                                                                   \
+        if (smem > 64 * 1024) {                                                                                       \
+            hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void *>(kern),                                  \
+                                               hipFuncAttributeMaxDynamicSharedMemorySize, (int)smem);                \
+            if (e != hipSuccess) return (int)e;                                                                       \
+        }                                                                                                             \
+        hipLaunchKernelGGL(kern, dim3(R / QB), dim3(LNB_THREADS), smem, st, qx, (const ST *)sx, qg, (const ST *)sg,   \
+                           gamma, mean, rstd, R, C, rounding, seed, offset, qdx, (ST *)sdx, pdg, pdb);                \
     } while (0)
-    if (scale_dtype == JF_SCALE_F16) JF_LNB(half_t);
-    else JF_LNB(float);
-#undef JF_LNB
-    if (dgamma) hipLaunchKernelGGL(colsum_kernel, dim3((C + 63) / 64), dim3(1024), 0, st, pdg, R / QB, C, dgamma);
-    if (dbeta) hipLaunchKernelGGL(colsum_kernel, dim3((C + 63) / 64), dim3(1024), 0, st, pdb, R / QB, C, dbeta);
+    if (scale_dtype == JF_SCALE_F16) JF_LNF(half_t);
+    else JF_LNF(float);
+#undef JF_LNF
+    if (want_dw)
+        hipLaunchKernelGGL(colsum_kernel, dim3((C + 63) / 64, 2), dim3(1024), 0, st, pdg, dgamma, pdb, dbeta, R / QB, C);
     return (int)hipGetLastError();
 }
 
