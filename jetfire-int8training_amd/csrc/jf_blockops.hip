@@ -126,15 +126,21 @@ __global__ __launch_bounds__(NT) void dequantize_kernel(const int8_t *q, const S
 // the wave evaluates the function once per code (4 codes per lane) into a 1 KiB LDS table and every element then
 // costs one LDS gather instead of ~40 vector instructions.  The table entry is computed from (float)code * scale,
 // the very expression a per-element evaluation would use, so the results are bit-identical to it.
-template <typename F>
-__device__ __forceinline__ void fill_code_table(float *table, int lane, float scale, F f)
+// PAIR(x, pos, neg) evaluates the function at +x and -x (x >= 0).  Lane l covers the magnitudes 2l+1 and 2l+2
+// (1 .. 128); entry index = the code's byte value, so -m sits at 256-m and index 128 is the code -128.  Entry 0
+// (the function at +0, the same for every block) is passed in.
+template <typename PAIR>
+__device__ __forceinline__ void fill_code_table(float *table, int lane, float scale, float f0, PAIR pair)
 {
-    v4f t;
-    t.x = f((float)(int8_t)(4 * lane + 0) * scale);
-    t.y = f((float)(int8_t)(4 * lane + 1) * scale);
-    t.z = f((float)(int8_t)(4 * lane + 2) * scale);
-    t.w = f((float)(int8_t)(4 * lane + 3) * scale);
-    *reinterpret_cast<v4f *>(table + 4 * lane) = t;               // entry index = the code's byte value
+    const int m = 2 * lane + 1;
+    float p0, n0, p1, n1;
+    pair((float)m * scale, p0, n0);
+    pair((float)(m + 1) * scale, p1, n1);
+    table[m] = p0;
+    if (lane < 63) table[m + 1] = p1;                              // +128 is not a code
+    table[256 - m] = n0;
+    table[255 - m] = n1;
+    if (lane == 0) table[0] = f0;
     __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
     __builtin_amdgcn_wave_barrier();
     __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
@@ -200,11 +206,14 @@ __global__ __launch_bounds__(NT) void gelu_fwd_kernel(const int8_t *q, const ST 
     const int lane = threadIdx.x & 63, SC = C / QB, nblk = (R / QB) * SC, stride = gridDim.x * WPB;
     const int blk0 = blockIdx.x * WPB + (threadIdx.x >> 6);
     CodeStream<ST> in(q, s, C, SC, nblk, stride, lane, blk0);
+    float zero = 0.0f;
+    asm volatile("" : "+v"(zero));                                 // evaluated on the device, like every other entry
+    const float f0 = gelu<APPROX>(zero);
     for (int blk = blk0; blk < nblk; blk += stride) {
         BlockPos pos(blk, SC, C, lane);
         v4i c; float sc;
         in.next(blk, c, sc);
-        fill_code_table(tab, lane, sc, [](float v) { return gelu<APPROX>(v); });
+        fill_code_table(tab, lane, sc, f0, [](float v, float &a, float &b) { gelu_pair<APPROX>(v, a, b); });
         float x[16];
         gather16(tab, c, x);
         table_done();
@@ -226,6 +235,9 @@ __global__ __launch_bounds__(NT) void gelu_bwd_kernel(const int8_t *qx, const ST
     const int lane = threadIdx.x & 63, SC = C / QB, nblk = (R / QB) * SC, stride = gridDim.x * WPB;
     const int blk0 = blockIdx.x * WPB + (threadIdx.x >> 6);
     CodeStream<ST> inx(qx, sx, C, SC, nblk, stride, lane, blk0), ing(qg, sg, C, SC, nblk, stride, lane, blk0);
+    float zero = 0.0f;
+    asm volatile("" : "+v"(zero));
+    const float f0 = dgelu<APPROX>(zero);
     for (int blk = blk0; blk < nblk; blk += stride) {
         BlockPos pos(blk, SC, C, lane);
         v4i cx, cg; float scx, scg;
@@ -233,7 +245,7 @@ __global__ __launch_bounds__(NT) void gelu_bwd_kernel(const int8_t *qx, const ST
         ing.next(blk, cg, scg);
         float x[16], g[16];
         unpack16(cg, scg, g);
-        fill_code_table(tab, lane, scx, [](float v) { return dgelu<APPROX>(v); });
+        fill_code_table(tab, lane, scx, f0, [](float v, float &a, float &b) { dgelu_pair<APPROX>(v, a, b); });
         gather16(tab, cx, x);
         table_done();
 #pragma unroll
@@ -487,6 +499,15 @@ static inline int grid_for_blocks(int R, int C)
     return (int)(g < cap ? g : cap);
 }
 
+// kernels that keep several blocks in flight per wave and have per-kernel setup: no more workgroups than are resident
+static inline int grid_for_resident(int R, int C)
+{
+    const long nblk = (long)(R / QB) * (C / QB);
+    long g = (nblk + WPB - 1) / WPB;
+    const long cap = 256L * 8;
+    return (int)(g < cap ? g : cap);
+}
+
 static int check_block_tensor(const void *q, const void *s, int R, int C, int scale_dtype)
 {
     if (!q || !s) return JF_ERR_NULL;
@@ -630,7 +651,7 @@ int jf_gelu_fwd(const int8_t *q, const void *s, int R, int C, int scale_dtype, i
     if (approx != JF_GELU_ERF && approx != JF_GELU_TANH) return JF_ERR_ENUM;
     if (!aligned16(qy)) return JF_ERR_ALIGN;
     hipStream_t st = (hipStream_t)stream;
-    const int grid = grid_for_blocks(R, C);
+    const int grid = grid_for_resident(R, C);
 #define JF_GF(A, ST) JF_LAUNCH((gelu_fwd_kernel<A, ST>), grid, 0, st, q, (const ST *)s, R, C, amax_eps, qy, (ST *)sy)
     if (scale_dtype == JF_SCALE_F16) {
         if (approx == JF_GELU_ERF) JF_GF(JF_GELU_ERF, half_t);
@@ -652,7 +673,7 @@ int jf_gelu_bwd(const int8_t *qx, const void *sx, const int8_t *qg, const void *
     if ((approx != JF_GELU_ERF && approx != JF_GELU_TANH) || !rounding_ok(rounding)) return JF_ERR_ENUM;
     if (!aligned16(qy)) return JF_ERR_ALIGN;
     hipStream_t st = (hipStream_t)stream;
-    const int grid = grid_for_blocks(R, C);
+    const int grid = grid_for_resident(R, C);
 #define JF_GB(A, ST)                                                                                              \
     JF_LAUNCH((gelu_bwd_kernel<A, ST>), grid, 0, st, qx, (const ST *)sx, qg, (const ST *)sg, R, C, rounding, seed, \
               offset, qy, (ST *)sy)

@@ -259,6 +259,44 @@ template <int APPROX> __device__ __forceinline__ float dgelu(float x)
     return __builtin_fmaf((0.5f * x) * sech2, dinner, 0.5f * (1.0f + t));
 }
 
+// gelu / dgelu at +x and -x (x >= 0) from one evaluation of the expensive part.  Every operation below is the one
+// gelu<>/dgelu<> performs at that argument, or differs from it by exact sign symmetries only (x*x, |x|, a product with one
+// factor negated, 1 + (-t)), so the pair is bit-identical to two separate evaluations.
+template <int APPROX> __device__ __forceinline__ void gelu_pair(float x, float &pos, float &neg)
+{
+    if (APPROX == JF_GELU_ERF) {
+        const float h = 0.5f * erfc_pos(x * 0.707106781f);
+        pos = x * (x > 0.0f ? 1.0f - h : h);
+        neg = (-x) * h;
+        return;
+    }
+    const float x2 = x * x;
+    const float inner = 0.797884561f * (x * __builtin_fmaf(0.044715f, x2, 1.0f));
+    const float t = tanhf_det(inner);                      // inner >= 0, so t >= 0 and tanh(-inner) = -t
+    const float hx = 0.5f * x;
+    pos = hx * (1.0f + t);
+    neg = (-hx) * (1.0f - t);
+}
+
+template <int APPROX> __device__ __forceinline__ void dgelu_pair(float x, float &pos, float &neg)
+{
+    if (APPROX == JF_GELU_ERF) {
+        const float pdf = 0.398942280f * expf_det(-0.5f * (x * x));
+        const float h = 0.5f * erfc_pos(x * 0.707106781f);
+        pos = __builtin_fmaf(x, pdf, x > 0.0f ? 1.0f - h : h);
+        neg = __builtin_fmaf(-x, pdf, h);
+        return;
+    }
+    const float x2 = x * x;
+    const float inner = 0.797884561f * (x * __builtin_fmaf(0.044715f, x2, 1.0f));
+    const float t = tanhf_det(inner);
+    const float dinner = 0.797884561f * __builtin_fmaf(0.134145f, x2, 1.0f);
+    const float sech2 = __builtin_fmaf(-t, t, 1.0f);
+    const float a = (0.5f * x) * sech2;
+    pos = __builtin_fmaf(a, dinner, 0.5f * (1.0f + t));
+    neg = __builtin_fmaf(-a, dinner, 0.5f * (1.0f - t));
+}
+
 // ---------------------------------------------------------------------------------------------
 // host-side argument checks shared by the entry points
 static inline bool mult32(int v) { return v > 0 && (v % QB) == 0; }
