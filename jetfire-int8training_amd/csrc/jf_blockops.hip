@@ -166,33 +166,49 @@ __device__ __forceinline__ void table_done()
 // cover the memory latency, so the GELU kernels run the block loop with the codes and scales of the next PF blocks
 // already requested.
 constexpr int PF = 3;
+// Walks the blocks blk0, blk0 + stride, ... of a wave without a division per block: (row block, column block) advance
+// by (stride / SC, stride % SC) with a carry.
+struct BlockWalk {
+    int rb, cb, drb, dcb, SC;
+    __device__ __forceinline__ BlockWalk(int blk0, int stride, int SC_) : SC(SC_)
+    {
+        rb = blk0 / SC; cb = blk0 - rb * SC;
+        drb = stride / SC; dcb = stride - drb * SC;
+    }
+    __device__ __forceinline__ void step()
+    {
+        rb += drb; cb += dcb;
+        if (cb >= SC) { cb -= SC; ++rb; }
+    }
+};
 template <typename ST> struct CodeStream {
     const int8_t *q;
     const ST *s;
-    int C, SC, nblk, stride, lane;
+    int C, RB, lane;
+    BlockWalk at;                 // the next block to request
     v4i codes[PF];
     float scale[PF];
-    __device__ __forceinline__ void request(int slot, int blk)
+    __device__ __forceinline__ void request(int slot)
     {
-        if (blk < nblk) {
-            const int rb = blk / SC, cb = blk - rb * SC;
-            codes[slot] = *reinterpret_cast<const v4i *>(q + (size_t)(rb * QB + (lane >> 1)) * C + cb * QB + (lane & 1) * 16);
-            scale[slot] = load_scale(s, blk);
+        if (at.rb < RB) {
+            codes[slot] = *reinterpret_cast<const v4i *>(q + (size_t)(at.rb * QB + (lane >> 1)) * C + at.cb * QB + (lane & 1) * 16);
+            scale[slot] = load_scale(s, at.rb * at.SC + at.cb);
         }
+        at.step();
     }
-    __device__ __forceinline__ CodeStream(const int8_t *q_, const ST *s_, int C_, int SC_, int nblk_, int stride_, int lane_, int blk0)
-        : q(q_), s(s_), C(C_), SC(SC_), nblk(nblk_), stride(stride_), lane(lane_)
+    __device__ __forceinline__ CodeStream(const int8_t *q_, const ST *s_, int R, int C_, int stride, int lane_, int blk0)
+        : q(q_), s(s_), C(C_), RB(R / QB), lane(lane_), at(blk0, stride, C_ / QB)
     {
 #pragma unroll
-        for (int i = 0; i < PF; ++i) request(i, blk0 + i * stride);
+        for (int i = 0; i < PF; ++i) request(i);
     }
     // hands out the oldest block and requests the one PF strides ahead
-    __device__ __forceinline__ void next(int blk, v4i &c, float &sc)
+    __device__ __forceinline__ void next(v4i &c, float &sc)
     {
         c = codes[0]; sc = scale[0];
 #pragma unroll
         for (int i = 0; i + 1 < PF; ++i) { codes[i] = codes[i + 1]; scale[i] = scale[i + 1]; }
-        request(PF - 1, blk + PF * stride);
+        request(PF - 1);
     }
 };
 
@@ -202,25 +218,53 @@ __global__ __launch_bounds__(NT) void gelu_fwd_kernel(const int8_t *q, const ST 
                                                       int8_t *qy, ST *sy)
 {
     __shared__ __attribute__((aligned(16))) float table[WPB][256];
+    __shared__ __attribute__((aligned(16))) int qtable[WPB][256];
     float *tab = table[threadIdx.x >> 6];
-    const int lane = threadIdx.x & 63, SC = C / QB, nblk = (R / QB) * SC, stride = gridDim.x * WPB;
-    const int blk0 = blockIdx.x * WPB + (threadIdx.x >> 6);
-    CodeStream<ST> in(q, s, C, SC, nblk, stride, lane, blk0);
+    int *qtab = qtable[threadIdx.x >> 6];
+    const int lane = threadIdx.x & 63, SC = C / QB, RB = R / QB, stride = gridDim.x * WPB;
+    const int blk0 = __builtin_amdgcn_readfirstlane(blockIdx.x * WPB + (threadIdx.x >> 6));
+    CodeStream<ST> in(q, s, R, C, stride, lane, blk0);
     float zero = 0.0f;
     asm volatile("" : "+v"(zero));                                 // evaluated on the device, like every other entry
     const float f0 = gelu<APPROX>(zero);
-    for (int blk = blk0; blk < nblk; blk += stride) {
-        BlockPos pos(blk, SC, C, lane);
+    for (BlockWalk w(blk0, stride, SC); w.rb < RB; w.step()) {
+        const size_t e0 = (size_t)(w.rb * QB + (lane >> 1)) * C + w.cb * QB + (lane & 1) * 16;
         v4i c; float sc;
-        in.next(blk, c, sc);
+        in.next(c, sc);
         fill_code_table(tab, lane, sc, f0, [](float v, float &a, float &b) { gelu_pair<APPROX>(v, a, b); });
+        // The outputs take at most 256 distinct values too, so the requantisation (exact division, rounding, clamp) is
+        // done on the table, 4 entries per lane, once the block's absmax is known; an element costs two gathers.
         float x[16];
         gather16(tab, c, x);
+        float m = 0.0f;
+#pragma unroll
+        for (int k = 0; k < 16; ++k) m = fmaxf(m, fabsf(x[k]));
+        const float amax = wave_max(m) + amax_eps;
+        float scale = 0.0f;
+        v4i codes = {0, 0, 0, 0};
+        if (amax > 0.0f) {                                         // uniform
+            scale = amax / 127.0f;
+            BlockDivisor d(scale);
+            const v4f t4 = *reinterpret_cast<const v4f *>(tab + 4 * lane);
+            const float t[4] = {t4.x, t4.y, t4.z, t4.w};
+            float y[4];
+            d.divn<4>(t, y);
+            v4i q4 = {clamp127(__builtin_rintf(y[0])), clamp127(__builtin_rintf(y[1])), clamp127(__builtin_rintf(y[2])),
+                      clamp127(__builtin_rintf(y[3]))};
+            *reinterpret_cast<v4i *>(qtab + 4 * lane) = q4;
+            __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
+            __builtin_amdgcn_wave_barrier();
+            __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
+            const uint32_t wd[4] = {(uint32_t)c.x, (uint32_t)c.y, (uint32_t)c.z, (uint32_t)c.w};
+            int o[4];
+#pragma unroll
+            for (int i = 0; i < 4; ++i)
+                o[i] = (int)pack4(qtab[wd[i] & 0xFF], qtab[(wd[i] >> 8) & 0xFF], qtab[(wd[i] >> 16) & 0xFF], qtab[wd[i] >> 24]);
+            codes = v4i{o[0], o[1], o[2], o[3]};
+        }
         table_done();
-        float scale;
-        v4i codes = quantize16(x, amax_eps, JF_ROUND_NEAREST, 0, 0, pos.e0, &scale);
-        *reinterpret_cast<v4i *>(qy + pos.e0) = codes;
-        if (lane == 0) store_scale(sy, blk, scale);
+        *reinterpret_cast<v4i *>(qy + e0) = codes;
+        if (lane == 0) store_scale(sy, w.rb * SC + w.cb, scale);
     }
 }
 
@@ -232,17 +276,17 @@ __global__ __launch_bounds__(NT) void gelu_bwd_kernel(const int8_t *qx, const ST
 {
     __shared__ __attribute__((aligned(16))) float table[WPB][256];
     float *tab = table[threadIdx.x >> 6];
-    const int lane = threadIdx.x & 63, SC = C / QB, nblk = (R / QB) * SC, stride = gridDim.x * WPB;
-    const int blk0 = blockIdx.x * WPB + (threadIdx.x >> 6);
-    CodeStream<ST> inx(qx, sx, C, SC, nblk, stride, lane, blk0), ing(qg, sg, C, SC, nblk, stride, lane, blk0);
+    const int lane = threadIdx.x & 63, SC = C / QB, RB = R / QB, stride = gridDim.x * WPB;
+    const int blk0 = __builtin_amdgcn_readfirstlane(blockIdx.x * WPB + (threadIdx.x >> 6));
+    CodeStream<ST> inx(qx, sx, R, C, stride, lane, blk0), ing(qg, sg, R, C, stride, lane, blk0);
     float zero = 0.0f;
     asm volatile("" : "+v"(zero));
     const float f0 = dgelu<APPROX>(zero);
-    for (int blk = blk0; blk < nblk; blk += stride) {
-        BlockPos pos(blk, SC, C, lane);
+    for (BlockWalk w(blk0, stride, SC); w.rb < RB; w.step()) {
+        const size_t e0 = (size_t)(w.rb * QB + (lane >> 1)) * C + w.cb * QB + (lane & 1) * 16;
         v4i cx, cg; float scx, scg;
-        inx.next(blk, cx, scx);
-        ing.next(blk, cg, scg);
+        inx.next(cx, scx);
+        ing.next(cg, scg);
         float x[16], g[16];
         unpack16(cg, scg, g);
         fill_code_table(tab, lane, scx, f0, [](float v, float &a, float &b) { dgelu_pair<APPROX>(v, a, b); });
@@ -251,9 +295,9 @@ __global__ __launch_bounds__(NT) void gelu_bwd_kernel(const int8_t *qx, const ST
 #pragma unroll
         for (int k = 0; k < 16; ++k) x[k] = x[k] * g[k];
         float scale;
-        v4i codes = quantize16(x, 0.0f, rounding, seed, offset, pos.e0, &scale);
-        *reinterpret_cast<v4i *>(qy + pos.e0) = codes;
-        if (lane == 0) store_scale(sy, blk, scale);
+        v4i codes = quantize16(x, 0.0f, rounding, seed, offset, e0, &scale);
+        *reinterpret_cast<v4i *>(qy + e0) = codes;
+        if (lane == 0) store_scale(sy, w.rb * SC + w.cb, scale);
     }
 }
 

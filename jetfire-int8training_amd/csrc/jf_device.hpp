@@ -100,21 +100,22 @@ struct BlockDivisor {
         fast = __builtin_amdgcn_readfirstlane((s_ > 8.67361738e-19f) && (s_ < 1.15292150e+18f)) != 0;
         r = 1.0f / s_;
     }
-    // y[i] = x[i] / s for 16 values; ONE uniform branch around the whole batch
-    __device__ __forceinline__ void div16(const float x[16], float y[16]) const
+    // y[i] = x[i] / s for N values; ONE uniform branch around the whole batch
+    template <int N> __device__ __forceinline__ void divn(const float *x, float *y) const
     {
         if (fast) {
 #pragma unroll
-            for (int i = 0; i < 16; ++i) {
+            for (int i = 0; i < N; ++i) {
                 float q0 = x[i] * r;
                 float e = __builtin_fmaf(-q0, s, x[i]);
                 y[i] = __builtin_fmaf(e, r, q0);
             }
         } else {
 #pragma unroll
-            for (int i = 0; i < 16; ++i) y[i] = x[i] / s;
+            for (int i = 0; i < N; ++i) y[i] = x[i] / s;
         }
     }
+    __device__ __forceinline__ void div16(const float x[16], float y[16]) const { divn<16>(x, y); }
 };
 
 __device__ __forceinline__ int clamp127(float y_rounded)
