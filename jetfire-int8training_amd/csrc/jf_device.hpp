@@ -82,8 +82,10 @@ __device__ __forceinline__ void sr_noise16(uint64_t seed, uint64_t offset, uint6
         philox4x32_10((uint32_t)cc, (uint32_t)(cc >> 32), 0u, 0u, (uint32_t)seed, (uint32_t)(seed >> 32), o);
 #pragma unroll
         for (int w = 0; w < 4; ++w) {
-            n[call * 8 + 2 * w]     = ((float)(o[w] & 0xFFFFu) + 0.5f) * 1.52587890625e-05f - 0.5f;
-            n[call * 8 + 2 * w + 1] = ((float)(o[w] >> 16) + 0.5f) * 1.52587890625e-05f - 0.5f;
+            // (h + 0.5) * 2^-16 - 0.5 = h * 2^-16 + (2^-17 - 0.5): every step of either form is exact (17 significant
+            // bits at most), so the single fma gives the same value
+            n[call * 8 + 2 * w]     = __builtin_fmaf((float)(o[w] & 0xFFFFu), 1.52587890625e-05f, -0.49999237060546875f);
+            n[call * 8 + 2 * w + 1] = __builtin_fmaf((float)(o[w] >> 16), 1.52587890625e-05f, -0.49999237060546875f);
         }
     }
 }
@@ -129,6 +131,20 @@ __device__ __forceinline__ uint32_t pack4(int a, int b, int c, int d)
     return (uint32_t)(a & 0xFF) | ((uint32_t)(b & 0xFF) << 8) | ((uint32_t)(c & 0xFF) << 16) | ((uint32_t)d << 24);
 }
 
+// Round-to-nearest-even codes of 4 values, clamped to +-127, packed into one word.  Clamping first and rounding
+// second gives the same integers as rounding first (the bounds are integers).  Adding 1.5*2^23 rounds to an
+// integer in the addition itself and leaves its two's-complement low byte in the low byte of the bit pattern.
+__device__ __forceinline__ uint32_t round_clamp_pack4(float a, float b, float c, float d)
+{
+    auto code_bits = [](float y) {
+        const float yc = __builtin_amdgcn_fmed3f(y, -127.0f, 127.0f);
+        return __float_as_uint(yc + 12582912.0f);
+    };
+    const uint32_t ab = __builtin_amdgcn_perm(code_bits(b), code_bits(a), 0x0c0c0400u);   // bytes: a, b, 0, 0
+    const uint32_t cd = __builtin_amdgcn_perm(code_bits(d), code_bits(c), 0x0c0c0400u);
+    return __builtin_amdgcn_perm(cd, ab, 0x05040100u);                                    // bytes: a, b, c, d
+}
+
 // ---------------------------------------------------------------------------------------------
 // Block quantisation of 16 values per lane, one wave = one 32x32 block (lane l: row l/2,
 // columns 16*(l%2) .. +15).  Returns the packed codes; *scale_out = amax/127 (all lanes).
@@ -157,18 +173,20 @@ __device__ __forceinline__ v4i quantize16(const float v[16], float amax_eps, int
             y[i] = __builtin_copysignf(a, y[i]);
         }
     }
-    int c[16];
     if (rounding == JF_ROUND_TRUNC || rounding == JF_ROUND_STOCHASTIC_TRUNC) {
+        int c[16];
 #pragma unroll
         for (int i = 0; i < 16; ++i) c[i] = clamp127(__builtin_truncf(y[i]));
+        out.x = (int)pack4(c[0], c[1], c[2], c[3]);
+        out.y = (int)pack4(c[4], c[5], c[6], c[7]);
+        out.z = (int)pack4(c[8], c[9], c[10], c[11]);
+        out.w = (int)pack4(c[12], c[13], c[14], c[15]);
     } else {
-#pragma unroll
-        for (int i = 0; i < 16; ++i) c[i] = clamp127(__builtin_rintf(y[i]));
+        out.x = (int)round_clamp_pack4(y[0], y[1], y[2], y[3]);
+        out.y = (int)round_clamp_pack4(y[4], y[5], y[6], y[7]);
+        out.z = (int)round_clamp_pack4(y[8], y[9], y[10], y[11]);
+        out.w = (int)round_clamp_pack4(y[12], y[13], y[14], y[15]);
     }
-    out.x = (int)pack4(c[0], c[1], c[2], c[3]);
-    out.y = (int)pack4(c[4], c[5], c[6], c[7]);
-    out.z = (int)pack4(c[8], c[9], c[10], c[11]);
-    out.w = (int)pack4(c[12], c[13], c[14], c[15]);
     return out;
 }
 

@@ -544,13 +544,10 @@ __global__ __launch_bounds__(64 * WGM * WGN, WGPC * WGM * WGN / 4) void igemm_nt
 #pragma unroll
                         for (int k = 0; k < 16; ++k) t[k] = t[k] + n[k];
                     }
-                    int c[16];
-#pragma unroll
-                    for (int k = 0; k < 16; ++k) c[k] = clamp127(__builtin_rintf(t[k]));
-                    codes.x = (int)pack4(c[0], c[1], c[2], c[3]);
-                    codes.y = (int)pack4(c[4], c[5], c[6], c[7]);
-                    codes.z = (int)pack4(c[8], c[9], c[10], c[11]);
-                    codes.w = (int)pack4(c[12], c[13], c[14], c[15]);
+                    codes.x = (int)round_clamp_pack4(t[0], t[1], t[2], t[3]);
+                    codes.y = (int)round_clamp_pack4(t[4], t[5], t[6], t[7]);
+                    codes.z = (int)round_clamp_pack4(t[8], t[9], t[10], t[11]);
+                    codes.w = (int)round_clamp_pack4(t[12], t[13], t[14], t[15]);
                 }
                 *reinterpret_cast<v4i *>(tile + (size_t)trow * BN + tcol) = codes;
                 if (lane == 0) store_scale(reinterpret_cast<ST *>(p.sc), (bm / QB) * SN + bn / QB, scale);
