@@ -12,7 +12,8 @@
  *     All of R, C, M, N, K must be positive multiples of 32.  Data pointers must be 16-byte aligned.
  *   - `scale_dtype` selects the element type of EVERY scale pointer of the call
  *     (JF_SCALE_F16 = IEEE binary16, what the reference stores; JF_SCALE_F32 = binary32).
- *   - GEMM scale operands are K-major: sa[kb*(M/32)+mb], sb[kb*(N/32)+nb]; output scales are
+ *   - GEMM scale operands are K-major (JF_SCALES_KMAJOR): sa[kb*(M/32)+mb], sb[kb*(N/32)+nb], or, per operand, the
+ *     block tensor's own row-major scale array (JF_SCALES_ROWMAJOR): sa[mb*(K/32)+kb]; output scales are
  *     sc[mb*(N/32)+nb]  (reference: …/igemm/igemm_BlockSquare32OutputIntQuantizeBiasRowCol.cu:110-111,
  *     187-188, 297-304; paths below are relative to JetfireGEMMKernel/BlockQuantize/cpp_extension/).
  *   - stochastic rounding draws Philox4x32-10 noise keyed by (seed, offset + flat output index / 8),
@@ -42,6 +43,10 @@ extern "C" {
 
 #define JF_SCALE_F16 0
 #define JF_SCALE_F32 1
+
+/* Where the scale of block (row block r, K block kb) of a GEMM operand lives */
+#define JF_SCALES_KMAJOR   0      /* s[kb*(rows/32) + r]: what the reference kernels take (callers transpose)        */
+#define JF_SCALES_ROWMAJOR 1      /* s[r*(K/32) + kb]: the block tensor's own scale array, no transposed copy needed */
 
 #define JF_FP_F16  0
 #define JF_FP_F32  1
@@ -77,7 +82,7 @@ int jf_igemm_block_acc(const int8_t *A, const int8_t *B, int32_t *acc, int M, in
 /* C_fp[M,N] = sum_kb sa*sb*(A_kb*B_kb), fp32 accumulate in ascending kb, stored as out_dtype.
  * Replaces igemm_output_fp_no_quantize (include/igemm.h:14-25, igemm/igemm_BlockSquare32OutputFp.cu:340-382). */
 int jf_igemm_block_fp(const int8_t *A, const int8_t *B, const void *sa, const void *sb, void *C,
-                      int M, int N, int K, int b_layout, int scale_dtype, int out_dtype,
+                      int M, int N, int K, int b_layout, int scale_dtype, int sa_layout, int sb_layout, int out_dtype,
                       void *workspace, size_t workspace_bytes, jf_stream_t stream);
 
 /* (C_s8[M,N], sc[M/32,N/32]) = per-32x32-block requantisation of the same accumulation.
@@ -89,7 +94,7 @@ int jf_igemm_block_fp(const int8_t *A, const int8_t *B, const void *sa, const vo
  * bias ([N] fp32) and biasmax ([1] fp32, device) may be NULL (= zeros). */
 int jf_igemm_block_q(const int8_t *A, const int8_t *B, const void *sa, const void *sb,
                      const float *bias, const float *biasmax, int8_t *C, void *sc,
-                     int M, int N, int K, int b_layout, int scale_dtype, int rounding,
+                     int M, int N, int K, int b_layout, int scale_dtype, int sa_layout, int sb_layout, int rounding,
                      uint64_t seed, uint64_t offset,
                      void *workspace, size_t workspace_bytes, jf_stream_t stream);
 

@@ -1,8 +1,10 @@
 """int8_linear_forward / int8_linear_backward on top of the BlockQuantizeCUDA extension.
 
 Data format everywhere: codes int8 [..., R, C] with one scale per 32x32 tile, scales [..., R/32, C/32]
-(float16 as in the reference, float32 accepted).  The GEMM entry points want both scale operands K-major
-([K/32, rows/32]), hence the small transposes below (reference: linear_fwd.py:17-18, linear_bwd.py:11).
+(float16 as in the reference, float32 accepted).  The GEMM entry points take their scale operands as [K/32, rows/32];
+the reference makes transposed copies for that (linear_fwd.py:17-18, linear_bwd.py:11), here the .t() VIEW of the
+block tensor's own scale array is passed and the kernel reads it in place.  The zero bias the reference allocates on
+every call (linear_fwd.py:20-21) is kept per device and width.
 """
 import os
 import sys
@@ -23,7 +25,18 @@ def _flat2(t):
 
 
 def _k_major(s2d):
-    return s2d.t().contiguous()
+    """[rows/32, K/32] -> [K/32, rows/32] without a copy (the extension accepts this view)."""
+    return s2d.contiguous().t()
+
+
+_ZERO_BIAS = {}
+
+
+def _zero_bias(n, device):
+    key = (str(device), n)
+    if key not in _ZERO_BIAS:
+        _ZERO_BIAS[key] = (torch.zeros(n, dtype=torch.float32, device=device), torch.zeros(1, dtype=torch.float32, device=device))
+    return _ZERO_BIAS[key]
 
 
 def _check_block(B):
@@ -47,8 +60,7 @@ def int8_linear_forward(X8_3D, SX16_3D, W8, SW16, output_quantized, B):
     sx2 = _flat2(SX16_3D)
     n_out = W8.shape[0]
     m, k = x2.shape
-    zero_bias = torch.zeros(n_out, dtype=torch.float32, device=W8.device)
-    zero_biasmax = torch.zeros(1, dtype=torch.float32, device=W8.device)
+    zero_bias, zero_biasmax = _zero_bias(n_out, W8.device)
     o8, so = BQC.igemm_output_int_quantize_bias_rowcol(x2.contiguous(), W8.t(), zero_bias, zero_biasmax,
                                                        _k_major(sx2), _k_major(SW16), m, n_out, k)
     if not output_quantized:

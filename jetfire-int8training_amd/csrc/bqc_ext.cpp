@@ -73,16 +73,28 @@ void check_b_nk(const torch::Tensor &W, const torch::Tensor &X, int64_t K, int64
                 W.sizes(), " strides ", W.strides());
 }
 
-int check_scales(const torch::Tensor &SX, const torch::Tensor &SW, const torch::Tensor &X, int64_t M, int64_t N, int64_t K)
+// A GEMM scale operand is [K/32, rows/32]: either contiguous (what the reference kernels need, JF_SCALES_KMAJOR) or the
+// .t() view of a contiguous [rows/32, K/32] tensor, i.e. the block tensor's own scale array without the transposed
+// copy (JF_SCALES_ROWMAJOR; strides (1, K/32)).
+int scale_layout(const torch::Tensor &S, int64_t K, int64_t rows, const char *name)
+{
+    TORCH_CHECK(S.dim() == 2 && S.size(0) == K / QB && S.size(1) == rows / QB, name, " must be [K/32,rows/32] = [", K / QB,
+                ",", rows / QB, "], got ", S.sizes());
+    if (S.is_contiguous()) return JF_SCALES_KMAJOR;
+    TORCH_CHECK(S.stride(0) == 1 && S.stride(1) == K / QB, name,
+                " must be contiguous or the .t() view of a contiguous [rows/32,K/32] tensor, got strides ", S.strides());
+    return JF_SCALES_ROWMAJOR;
+}
+
+int check_scales(const torch::Tensor &SX, const torch::Tensor &SW, const torch::Tensor &X, int64_t M, int64_t N, int64_t K,
+                 int &sx_layout, int &sw_layout)
 {
     const int code = scale_code(SX, "SX");
     TORCH_CHECK(SW.scalar_type() == SX.scalar_type(), "SX and SW must have the same dtype");
     TORCH_CHECK(SX.is_cuda() && SW.is_cuda() && SX.device() == X.device() && SW.device() == X.device(),
                 "scales must be on the same GPU as X");
-    TORCH_CHECK(SX.dim() == 2 && SX.size(0) == K / QB && SX.size(1) == M / QB && SX.is_contiguous(),
-                "SX must be contiguous [K/32,M/32] = [", K / QB, ",", M / QB, "], got ", SX.sizes());
-    TORCH_CHECK(SW.dim() == 2 && SW.size(0) == K / QB && SW.size(1) == N / QB && SW.is_contiguous(),
-                "SW must be contiguous [K/32,N/32] = [", K / QB, ",", N / QB, "], got ", SW.sizes());
+    sx_layout = scale_layout(SX, K, M, "SX");
+    sw_layout = scale_layout(SW, K, N, "SW");
     return code;
 }
 
@@ -161,7 +173,8 @@ std::tuple<torch::Tensor, torch::Tensor> block_q(const torch::Tensor &X, const t
     check_dims(M, N, K);
     check_a(X, M, K);
     if (layout == JF_B_NK) check_b_nk(W, X, K, N); else check_b_kn(W, X, K, N);
-    const int code = check_scales(SX, SW, X, M, N, K);
+    int sxl, swl;
+    const int code = check_scales(SX, SW, X, M, N, K, sxl, swl);
     const float *bias_p = nullptr, *biasmax_p = nullptr;
     if (bias) {
         TORCH_CHECK(bias->is_cuda() && bias->device() == X.device() && bias->scalar_type() == torch::kFloat32 &&
@@ -174,14 +187,14 @@ std::tuple<torch::Tensor, torch::Tensor> block_q(const torch::Tensor &X, const t
     }
     c10::DeviceGuard guard(X.device());
     torch::Tensor O = torch::empty({M, N}, X.options().dtype(torch::kInt8));
-    torch::Tensor SO = torch::empty({M / QB, N / QB}, SX.options());
+    torch::Tensor SO = torch::empty({M / QB, N / QB}, SX.options().memory_format(c10::MemoryFormat::Contiguous));
     Workspace ws(X, M, N, K, layout);
     uint64_t seed = 0, offset = 0;
     if (rounding == JF_ROUND_STOCHASTIC) std::tie(seed, offset) = next_philox(X, (int64_t)M * N);
     {
         pybind11::gil_scoped_release nogil;
         check_rc(jf_igemm_block_q((const int8_t *)X.data_ptr(), (const int8_t *)W.data_ptr(), SX.data_ptr(), SW.data_ptr(),
-                                  bias_p, biasmax_p, (int8_t *)O.data_ptr(), SO.data_ptr(), M, N, K, layout, code, rounding,
+                                  bias_p, biasmax_p, (int8_t *)O.data_ptr(), SO.data_ptr(), M, N, K, layout, code, sxl, swl, rounding,
                                   seed, offset, ws.ptr, ws.bytes, current_stream(X)),
                  "igemm_block_q");
     }
@@ -215,13 +228,14 @@ torch::Tensor igemm_output_fp_no_quantize(torch::Tensor X, torch::Tensor W, torc
     check_dims(M, N, K);
     check_a(X, M, K);
     check_b_kn(W, X, K, N);
-    const int code = check_scales(SX, SW, X, M, N, K);
+    int sxl, swl;
+    const int code = check_scales(SX, SW, X, M, N, K, sxl, swl);
     c10::DeviceGuard guard(X.device());
     torch::Tensor O = torch::empty({M, N}, X.options().dtype(torch::kFloat16));
     Workspace ws(X, M, N, K, JF_B_KN);
     pybind11::gil_scoped_release nogil;
     check_rc(jf_igemm_block_fp((const int8_t *)X.data_ptr(), (const int8_t *)W.data_ptr(), SX.data_ptr(), SW.data_ptr(),
-                               O.data_ptr(), M, N, K, JF_B_KN, code, JF_FP_F16, ws.ptr, ws.bytes, current_stream(X)),
+                               O.data_ptr(), M, N, K, JF_B_KN, code, sxl, swl, JF_FP_F16, ws.ptr, ws.bytes, current_stream(X)),
              "igemm_output_fp_no_quantize");
     return O;
 }

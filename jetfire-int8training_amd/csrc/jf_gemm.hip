@@ -32,8 +32,9 @@ enum Epilogue { EPI_S32 = 0, EPI_FP = 1, EPI_Q = 2 };
 struct GemmArgs {
     const int8_t *A;      // [M, lda]
     const int8_t *B;      // [N, ldb] (K-contiguous) or, for the BKN kernels, [K, ldb] (N-contiguous)
-    const void *sa;       // [K/32, M/32]
-    const void *sb;       // [K/32, N/32]
+    const void *sa;       // scale of A block (mb, kb) at sa[kb * sa_ks + mb * sa_is]
+    const void *sb;       // scale of B block (nb, kb) at sb[kb * sb_ks + nb * sb_is]
+    int sa_ks, sa_is, sb_ks, sb_is;
     void *C;              // s32 / fp / s8 [M, N]
     void *sc;             // [M/32, N/32]   (EPI_Q)
     const float *bias;    // [N] or null   (EPI_Q)
@@ -156,14 +157,14 @@ __global__ __launch_bounds__(64 * WGM * WGN, WGPC * WGM * WGN / 4) void igemm_nt
     const bool s_is_a = !(s_blk >= WBM && s_blk < NSC);       // padding lanes repeat the first A-side scale
     int s_idx = s_is_a ? m0 / QB + wm * WBM + (s_blk < WBM ? s_blk : 0) : n0 / QB + wn * WBN + s_blk - WBM;
     { const int lim = s_is_a ? SM : SN; s_idx = s_idx < lim ? s_idx : lim - 1; }
-    const int s_ld = s_is_a ? SM : SN;
+    const int s_ks = s_is_a ? p.sa_ks : p.sb_ks, s_is = s_is_a ? p.sa_is : p.sb_is;   // element strides: K block, tile block
     const unsigned char *const s_base = reinterpret_cast<const unsigned char *>(s_is_a ? p.sa : p.sb);
     auto scale_addr = [&](int kbg) {
-        const unsigned e = (unsigned)(kbg * s_ld + s_idx);
+        const unsigned e = (unsigned)(kbg * s_ks + s_idx * s_is);
         return s_base + (sizeof(ST) == 4 ? e * 4u : (e >> 1) * 4u);
     };
     const unsigned char *s_ptr = scale_addr((lane >> 4) < nkb ? (lane >> 4) : nkb - 1);
-    const unsigned s_step = (unsigned)(KB_STAGE * s_ld) * (unsigned)sizeof(ST);   // KB_STAGE*s_ld is even: exact for binary16
+    const unsigned s_step = (unsigned)(KB_STAGE * s_ks) * (unsigned)sizeof(ST);   // KB_STAGE*s_ks is even: exact for binary16
 
     constexpr int A_LOADS = (BM / 8) / NW;                    // loads 0 .. A_LOADS-1 of a wave fetch A rows, the rest B rows
     static_assert((BM / 8) % NW == 0, "a load instruction fetches rows of one operand");
@@ -356,9 +357,9 @@ __global__ __launch_bounds__(64 * WGM * WGN, WGPC * WGM * WGN / 4) void igemm_nt
                 return (float)__builtin_bit_cast(half_t, h);
             };
 #pragma unroll
-            for (int i = 0; i < WBM; ++i) fa[i] = scale_of(sc_raw[CUR][i], kbg * SM + mb[i]);
+            for (int i = 0; i < WBM; ++i) fa[i] = scale_of(sc_raw[CUR][i], kbg * p.sa_ks + mb[i] * p.sa_is);
 #pragma unroll
-            for (int j = 0; j < WBN; ++j) fb[j] = scale_of(sc_raw[CUR][WBM + j], kbg * SN + nb[j]);
+            for (int j = 0; j < WBN; ++j) fb[j] = scale_of(sc_raw[CUR][WBM + j], kbg * p.sb_ks + nb[j] * p.sb_is);
             static_for<0, NBLK>([&](auto n_c) {
                 constexpr int n = decltype(n_c)::value, i = n / WBN, j = n % WBN;
                 const v16i z = {0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0};
@@ -727,8 +728,16 @@ int jf_igemm_block_acc(const int8_t *A, const int8_t *B, int32_t *acc, int M, in
     return JF_OK;
 }
 
+// element strides (K block, tile block) of a scale operand with `blocks` tile blocks
+static bool scale_strides(int layout, int K, int blocks, int &ks, int &is)
+{
+    if (layout == JF_SCALES_KMAJOR) { ks = blocks; is = 1; return true; }
+    if (layout == JF_SCALES_ROWMAJOR) { ks = 1; is = K / QB; return true; }
+    return false;
+}
+
 int jf_igemm_block_fp(const int8_t *A, const int8_t *B, const void *sa, const void *sb, void *C,
-                      int M, int N, int K, int b_layout, int scale_dtype, int out_dtype,
+                      int M, int N, int K, int b_layout, int scale_dtype, int sa_layout, int sb_layout, int out_dtype,
                       void *workspace, size_t workspace_bytes, jf_stream_t stream)
 {
     int rc = check_gemm_common(A, B, C, M, N, K, b_layout, workspace, workspace_bytes);
@@ -742,13 +751,15 @@ int jf_igemm_block_fp(const int8_t *A, const int8_t *B, const void *sa, const vo
     if (rc) return rc;
     GemmArgs a = {};
     a.A = A; a.B = B; a.sa = sa; a.sb = sb; a.C = C; a.M = M; a.N = N; a.K = K; a.lda = K; a.ldb = ldb;
+    if (!scale_strides(sa_layout, K, M / QB, a.sa_ks, a.sa_is) || !scale_strides(sb_layout, K, N / QB, a.sb_ks, a.sb_is))
+        return JF_ERR_ENUM;
     a.out_dtype = out_dtype;
     return scale_dtype == JF_SCALE_F16 ? launch_gemm<EPI_FP, half_t>(a, st, kn) : launch_gemm<EPI_FP, float>(a, st, kn);
 }
 
 int jf_igemm_block_q(const int8_t *A, const int8_t *B, const void *sa, const void *sb,
                      const float *bias, const float *biasmax, int8_t *C, void *sc,
-                     int M, int N, int K, int b_layout, int scale_dtype, int rounding,
+                     int M, int N, int K, int b_layout, int scale_dtype, int sa_layout, int sb_layout, int rounding,
                      uint64_t seed, uint64_t offset,
                      void *workspace, size_t workspace_bytes, jf_stream_t stream)
 {
@@ -764,6 +775,8 @@ int jf_igemm_block_q(const int8_t *A, const int8_t *B, const void *sa, const voi
     GemmArgs a = {};
     a.A = A; a.B = B; a.sa = sa; a.sb = sb; a.C = C; a.sc = sc; a.bias = bias; a.biasmax = biasmax;
     a.M = M; a.N = N; a.K = K; a.lda = K; a.ldb = ldb; a.rounding = rounding; a.seed = seed; a.offset = offset;
+    if (!scale_strides(sa_layout, K, M / QB, a.sa_ks, a.sa_is) || !scale_strides(sb_layout, K, N / QB, a.sb_ks, a.sb_is))
+        return JF_ERR_ENUM;
     return scale_dtype == JF_SCALE_F16 ? launch_gemm<EPI_Q, half_t>(a, st, kn) : launch_gemm<EPI_Q, float>(a, st, kn);
 }
 

@@ -18,6 +18,7 @@ QB = 32
 
 B_NK, B_KN = 0, 1
 SCALE_F16, SCALE_F32 = 0, 1
+SCALES_KMAJOR, SCALES_ROWMAJOR = 0, 1
 FP_F16, FP_F32, FP_BF16 = 0, 1, 2
 ROUND_NEAREST, ROUND_STOCHASTIC, ROUND_TRUNC, ROUND_STOCHASTIC_TRUNC = 0, 1, 2, 3
 GELU_ERF, GELU_TANH = 0, 1
@@ -45,8 +46,8 @@ def lib():
         L.jf_igemm_workspace_bytes.restype = _sz
         L.jf_igemm_s32.argtypes = [_p, _p, _p, _i, _i, _i, _i, _p, _sz, _p]
         L.jf_igemm_block_acc.argtypes = [_p, _p, _p, _i, _i, _i, _i, _p, _sz, _p]
-        L.jf_igemm_block_fp.argtypes = [_p, _p, _p, _p, _p, _i, _i, _i, _i, _i, _i, _p, _sz, _p]
-        L.jf_igemm_block_q.argtypes = [_p, _p, _p, _p, _p, _p, _p, _p, _i, _i, _i, _i, _i, _i, _u64, _u64, _p, _sz, _p]
+        L.jf_igemm_block_fp.argtypes = [_p, _p, _p, _p, _p, _i, _i, _i, _i, _i, _i, _i, _i, _p, _sz, _p]
+        L.jf_igemm_block_q.argtypes = [_p, _p, _p, _p, _p, _p, _p, _p, _i, _i, _i, _i, _i, _i, _i, _i, _u64, _u64, _p, _sz, _p]
         L.jf_quantize.argtypes = [_p, _i, _i, _i, _p, _p, _p, _i, _i, _u64, _u64, _f, _p]
         L.jf_dequantize.argtypes = [_p, _p, _i, _i, _i, _p, _p]
         L.jf_transpose_s8.argtypes = [_p, _i, _i, _p, _p]
@@ -157,14 +158,24 @@ def _gemm_operands(A, B, b_layout):
     return M, N, K, ws, nbytes
 
 
+def _scale_layout(s, K, rows, name):
+    """[K/32, rows/32] contiguous (K-major) or the .t() view of a contiguous [rows/32, K/32] tensor (row-major)."""
+    if not isinstance(s, torch.Tensor) or not s.is_cuda or s.dim() != 2:
+        raise RuntimeError(f"{name}: expected a 2-D GPU tensor")
+    if tuple(s.shape) != (K // QB, rows // QB):
+        raise RuntimeError(f"{name}: scale shape must be [K/32,rows/32]={K // QB, rows // QB}, got {tuple(s.shape)}")
+    if s.is_contiguous():
+        return SCALES_KMAJOR
+    if s.stride() == (1, K // QB):
+        return SCALES_ROWMAJOR
+    raise RuntimeError(f"{name}: expected a contiguous tensor or the .t() view of one, got strides {s.stride()}")
+
+
 def _gemm_scales(sa, sb, M, N, K):
     code = _scale_code(sa, "sa")
-    _need(sa, None, "sa")
-    _need(sb, sa.dtype, "sb")
-    if tuple(sa.shape) != (K // QB, M // QB) or tuple(sb.shape) != (K // QB, N // QB):
-        raise RuntimeError(f"scale shapes must be [K/32,M/32]={K // QB, M // QB} and [K/32,N/32]={K // QB, N // QB}, "
-                           f"got {tuple(sa.shape)} and {tuple(sb.shape)}")
-    return code
+    if sb.dtype != sa.dtype:
+        raise RuntimeError(f"sb: expected dtype {sa.dtype}, got {sb.dtype}")
+    return code, _scale_layout(sa, K, M, "sa"), _scale_layout(sb, K, N, "sb")
 
 
 def igemm_s32(A, B, b_layout=B_KN):
@@ -183,16 +194,16 @@ def igemm_block_acc(A, B, b_layout=B_KN):
 
 def igemm_block_fp(A, B, sa, sb, b_layout=B_KN, out_dtype=torch.float16):
     M, N, K, ws, nb = _gemm_operands(A, B, b_layout)
-    code = _gemm_scales(sa, sb, M, N, K)
+    code, la, lb = _gemm_scales(sa, sb, M, N, K)
     out = torch.empty((M, N), dtype=out_dtype, device=A.device)
-    check(lib().jf_igemm_block_fp(_ptr(A), _ptr(B), _ptr(sa), _ptr(sb), _ptr(out), M, N, K, b_layout, code,
+    check(lib().jf_igemm_block_fp(_ptr(A), _ptr(B), _ptr(sa), _ptr(sb), _ptr(out), M, N, K, b_layout, code, la, lb,
                                   _FP_CODE[out_dtype], _ptr(ws), nb, _stream()))
     return out
 
 
 def igemm_block_q(A, B, sa, sb, b_layout=B_KN, bias=None, biasmax=None, rounding=ROUND_NEAREST, seed=None, offset=None):
     M, N, K, ws, nb = _gemm_operands(A, B, b_layout)
-    code = _gemm_scales(sa, sb, M, N, K)
+    code, la, lb = _gemm_scales(sa, sb, M, N, K)
     if bias is not None:
         _need(bias, torch.float32, "bias", 1)
         if bias.numel() != N:
@@ -205,7 +216,7 @@ def igemm_block_q(A, B, sa, sb, b_layout=B_KN, bias=None, biasmax=None, rounding
     out = torch.empty((M, N), dtype=torch.int8, device=A.device)
     sc = torch.empty((M // QB, N // QB), dtype=sa.dtype, device=A.device)
     check(lib().jf_igemm_block_q(_ptr(A), _ptr(B), _ptr(sa), _ptr(sb), _ptr(bias), _ptr(biasmax), _ptr(out), _ptr(sc),
-                                 M, N, K, b_layout, code, rounding, seed, offset, _ptr(ws), nb, _stream()))
+                                 M, N, K, b_layout, code, la, lb, rounding, seed, offset, _ptr(ws), nb, _stream()))
     return out, sc
 
 

@@ -117,6 +117,29 @@ def test_block_q_deterministic_and_stochastic(jf, oracle, M, N, K, layout, f16):
         same(sc, wsc, "SR scales")
 
 
+@pytest.mark.parametrize("f16", [True, False])
+@pytest.mark.parametrize("layout", [0, 1])
+def test_row_major_scale_operands(jf, oracle, layout, f16):
+    """The scale operands may be the .t() views of the block tensors' own [rows/32, K/32] scale arrays (no transposed
+    copy): same bits as with K-major copies, for each operand separately and for both."""
+    M, N, K = 160, 352, 544
+    A, Bkn, sa, sb = make_problem(99 + layout, M, N, K, f16)
+    B = b_of(Bkn, layout)
+    st = np.float16 if f16 else np.float32
+    dA, dB = dev(A), dev(B)
+    ka, kb = dev(sa.astype(st)), dev(sb.astype(st))                                  # [K/32, rows/32] contiguous
+    ra, rb = dev(np.ascontiguousarray(sa.astype(st).T)).t(), dev(np.ascontiguousarray(sb.astype(st).T)).t()   # views
+    assert not ra.is_contiguous() and not rb.is_contiguous()
+    want = oracle.igemm_block_f32(A, B, sa, sb, layout)
+    for xa, xb in ((ra, kb), (ka, rb), (ra, rb)):
+        same(jf.igemm_block_fp(dA, dB, xa, xb, layout, torch.float32), want, "fp32 accumulators")
+        q0, s0 = jf.igemm_block_q(dA, dB, ka, kb, layout, rounding=jf.ROUND_STOCHASTIC, seed=3, offset=5)
+        q1, s1 = jf.igemm_block_q(dA, dB, xa, xb, layout, rounding=jf.ROUND_STOCHASTIC, seed=3, offset=5)
+        assert torch.equal(q0, q1) and torch.equal(s0, s1)
+    with pytest.raises(RuntimeError):
+        jf.igemm_block_fp(dA, dB, ka[:, ::2].repeat_interleave(2, 1)[:, : M // QB].t().t()[::1].as_strided((K // QB, M // QB), (M // QB * 2, 2)), kb, layout)
+
+
 def test_block_q_bias(jf, oracle):
     """The forward kernel's bias / biasmax inputs (…BiasRowCol.cu:313,341,357)."""
     M, N, K = 128, 256, 96
