@@ -3,18 +3,26 @@
 //   acc[m,n] = sum over 32-deep K blocks kb (ascending) of  (sa[kb,m/32]*sb[kb,n/32]) * d_kb[m,n]
 //   d_kb     = exact INT32 dot product of the kb-th 32-wide slices of A[m,:] and B[n,:]
 //
-// One v_mfma_i32_32x32x32_i8 with a zero accumulator input produces d_kb for a whole 32x32 output
-// block, i.e. exactly one Jetfire quantisation-block product; the fp32 scale-accumulate is one
-// v_cvt_f32_i32 + one v_fma_f32 per value.  (Reference kernels: igemm_BlockSquare32OutputIntQuantize
-// BiasRowCol.cu:134-225 and its siblings under JetfireGEMMKernel/BlockQuantize/cpp_extension/igemm/.)
+// One v_mfma_i32_32x32x32_i8 produces d_kb for a whole 32x32 output block, i.e. exactly one Jetfire
+// quantisation-block product.  (Reference kernels: igemm_BlockSquare32OutputIntQuantizeBiasRowCol.cu:134-225 and
+// its siblings under JetfireGEMMKernel/BlockQuantize/cpp_extension/igemm/.)
 //
-// Work decomposition: workgroup = 512 threads = 8 waves, tile 256x128 (or 128x256), each wave owns a
-// 64x64 sub-tile = 2x2 quantisation blocks (64 fp32 accumulators per lane).  K is consumed in stages
-// of 4 blocks (128 bytes per row) through a 3-deep LDS ring filled by LDS-direct loads
-// (global_load_lds_dwordx4: no register staging, two stages in flight while one is computed).  LDS rows
-// are 128 bytes with an XOR chunk swizzle, so the 16-byte MFMA operand reads are conflict-free.  Both
-// operands are K-contiguous ("NT"); a [K,N] B operand is transposed into a caller-provided workspace
-// first.  Scales are wave-uniform and come in through scalar loads.
+// Scale-accumulate.  The vector ALU is the bottleneck of this kernel, and on this part it runs plain fp32
+// add/mul/fma at twice the rate of conversions (v_cvt_f32_i32 included).  So the product is not converted:
+// the MFMA's accumulator input is the inline constant 0x3e22f983 (the bit pattern of 1/(2 pi)) in every
+// element.  |d| <= 32*127^2 < 2^21 keeps 0x3e22f983 + d inside the binade [1/8, 1/4), whose unit in the last
+// place is 2^-26, so  as_float(0x3e22f983 + d) - as_float(0x3e22f983) = d * 2^-26  exactly (one v_sub_f32),
+// and  fma(sa*sb*2^26, d*2^-26, acc)  has the same exact product, hence the same rounding, as
+// fma(sa*sb, float(d), acc).  The only way the two differ is an overflow of sa*sb*2^26; that is detected
+// after the K loop and the wave then recomputes its blocks with the plain sequence (see there).
+//
+// Work decomposition: workgroup = 8 waves (2 x 4), tile 128x128, each wave owns 64x32 = 2 quantisation
+// blocks (32 fp32 accumulators per lane); two workgroups per CU.  K is consumed in stages of 4 blocks (128
+// bytes per row) through an LDS ring filled by LDS-direct loads (global_load_lds_dwordx4: no register
+// staging).  LDS rows are 128 bytes with an XOR chunk swizzle, so the 16-byte MFMA operand reads are
+// conflict-free.  A is K-contiguous; B is either K-contiguous ([N,K]) or [K,N], which is staged as it lies
+// in memory and read with the transposing LDS read.  Scales are wave-uniform and are fetched by each wave
+// into a private LDS patch.
 #include "jf_device.hpp"
 
 #include <type_traits>
@@ -324,13 +332,14 @@ __global__ __launch_bounds__(64 * WGM * WGN, WGPC * WGM * WGN / 4) void igemm_nt
     // product n-1 (long finished) is converted and accumulated.  (d_pend, sab_pend) carry the lagging product across
     // K blocks and stages; the first accumulation adds 0*0 and the last product is accumulated after the loop.
     constexpr int NBLK = WBM * WBN;
+    constexpr int C_MAGIC = 0x3e22f983;                        // accumulator input of the MFMAs (file header)
     v16i d_pend = {0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0};
     float sab_pend = 0.0f;
     auto accumulate = [&](auto blk_c) {
         constexpr int i = decltype(blk_c)::value / WBN, j = decltype(blk_c)::value % WBN;
         float t[16];
 #pragma unroll
-        for (int v = 0; v < 16; ++v) t[v] = (float)d_pend[v];          // exact: |d| <= 32*127^2
+        for (int v = 0; v < 16; ++v) t[v] = __int_as_float(d_pend[v]) - __int_as_float(C_MAGIC);   // = d * 2^-26, exactly
 #pragma unroll
         for (int v = 0; v < 16; ++v) acc[i][j][v] = __builtin_fmaf(sab_pend, t[v], acc[i][j][v]);
         // pin the accumulation here: the optimiser would otherwise postpone it past the next K blocks and keep their
@@ -362,9 +371,13 @@ __global__ __launch_bounds__(64 * WGM * WGN, WGPC * WGM * WGN / 4) void igemm_nt
             for (int j = 0; j < WBN; ++j) fb[j] = scale_of(sc_raw[CUR][WBM + j], kbg * p.sb_ks + nb[j] * p.sb_is);
             static_for<0, NBLK>([&](auto n_c) {
                 constexpr int n = decltype(n_c)::value, i = n / WBN, j = n % WBN;
-                const v16i z = {0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0};
-                const v16i d_new = __builtin_amdgcn_mfma_i32_32x32x32_i8(fa_reg[CUR][i], fb_reg[CUR][j], z, 0, 0, 0);
-                const float sab_new = fa[i] * fb[j];
+                // asm: as a builtin operand the constant is hoisted into 16 registers instead of being encoded inline.
+                // The compiler therefore does not know this is an MFMA; its result is first read by the accumulate()
+                // AFTER the one below (32 vector instructions and another MFMA later), far beyond the wait states
+                // a vector read of an MFMA result needs.
+                v16i d_new;
+                asm volatile("v_mfma_i32_32x32x32_i8 %0, %1, %2, 0x3e22f983" : "=&v"(d_new) : "v"(fa_reg[CUR][i]), "v"(fb_reg[CUR][j]));
+                const float sab_new = (fa[i] * fb[j]) * 67108864.0f;       // * 2^26, see accumulate()
                 __builtin_amdgcn_sched_barrier(0);
                 accumulate(std::integral_constant<int, (n + NBLK - 1) % NBLK>{});
                 __builtin_amdgcn_sched_barrier(0);
@@ -441,7 +454,61 @@ __global__ __launch_bounds__(64 * WGM * WGN, WGPC * WGM * WGN / 4) void igemm_nt
         });
     }
     __builtin_amdgcn_s_waitcnt(0xC07F);                        // the last, unused prefetch must land before its registers are reused
-    if (EPI != EPI_S32) accumulate(std::integral_constant<int, NBLK - 1>{});
+    if (EPI != EPI_S32) {
+        accumulate(std::integral_constant<int, NBLK - 1>{});
+        // The scaled factor sa*sb*2^26 overflows when sa*sb >= 2^102.  An infinite factor leaves every accumulator
+        // it touches infinite or NaN (inf*0 included), so "some accumulator of the wave is not finite" catches all such
+        // cases; the wave then recomputes its blocks the plain way (operands straight from memory, zero accumulator
+        // input, v_cvt_f32_i32, unscaled factor), which also reproduces results that really are infinite.
+        float chk = 0.0f;
+#pragma unroll
+        for (int i = 0; i < WBM; ++i)
+#pragma unroll
+            for (int j = 0; j < WBN; ++j)
+#pragma unroll
+                for (int v = 0; v < 16; ++v) chk = __builtin_fmaf(acc[i][j][v], 0.0f, chk);
+        if (__builtin_expect(__ballot(chk != chk) != 0, 0)) {
+            const ST *const sa_t = reinterpret_cast<const ST *>(p.sa), *const sb_t = reinterpret_cast<const ST *>(p.sb);
+#pragma unroll 1
+            for (int blk = 0; blk < NBLK; ++blk) {
+                const int i = blk / WBN, j = blk % WBN;
+                const size_t arow = (size_t)(mb[i] * QB + (lane & 31)), bcol = (size_t)(nb[j] * QB + (lane & 31));
+                float r[16];
+#pragma unroll
+                for (int v = 0; v < 16; ++v) r[v] = 0.0f;
+#pragma unroll 1
+                for (int kb = 0; kb < nkb; ++kb) {
+                    const int k0 = kb * QB + 16 * (lane >> 5);
+                    const v4i fa = *reinterpret_cast<const v4i *>(p.A + arow * (size_t)p.lda + k0);
+                    v4i fb;
+                    if (BKN) {
+                        const int8_t *src = p.B + (size_t)k0 * (size_t)p.ldb + bcol;
+#pragma unroll
+                        for (int c = 0; c < 4; ++c) {
+                            unsigned w = 0;
+#pragma unroll 1
+                            for (int q = 0; q < 4; ++q, src += p.ldb) w |= (unsigned)(uint8_t)*src << (8 * q);
+                            fb[c] = (int)w;
+                        }
+                    } else {
+                        fb = *reinterpret_cast<const v4i *>(p.B + bcol * (size_t)p.ldb + k0);
+                    }
+                    const v16i z = {0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0};
+                    const v16i d = __builtin_amdgcn_mfma_i32_32x32x32_i8(fa, fb, z, 0, 0, 0);
+                    const float sab = (float)sa_t[kb * p.sa_ks + mb[i] * p.sa_is] * (float)sb_t[kb * p.sb_ks + nb[j] * p.sb_is];
+#pragma unroll
+                    for (int v = 0; v < 16; ++v) r[v] = __builtin_fmaf(sab, (float)d[v], r[v]);
+                }
+                static_for<0, NBLK>([&](auto n_c) {
+                    constexpr int n = decltype(n_c)::value;
+                    if (n == blk) {
+#pragma unroll
+                        for (int v = 0; v < 16; ++v) acc[n / WBN][n % WBN][v] = r[v];
+                    }
+                });
+            }
+        }
+    }
     __syncthreads();           // the epilogue reuses the ring as scratch
 
     // ---- epilogue ------------------------------------------------------------------------------------------

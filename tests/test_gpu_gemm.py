@@ -140,6 +140,37 @@ def test_row_major_scale_operands(jf, oracle, layout, f16):
         jf.igemm_block_fp(dA, dB, ka[:, ::2].repeat_interleave(2, 1)[:, : M // QB].t().t()[::1].as_strided((K // QB, M // QB), (M // QB * 2, 2)), kb, layout)
 
 
+@pytest.mark.parametrize("layout", [0, 1])
+@pytest.mark.parametrize("regime", ["huge_everywhere", "huge_one_block", "huge_last_kblock", "denormal_products"])
+def test_extreme_scale_products(jf, oracle, regime, layout):
+    """Scale products at the ends of the fp32 range.  sa*sb >= 2^102 is where the kernel's pre-scaled factor
+    (sa*sb*2^26) overflows and the wave must fall back to the plain conversion; products in the denormal range
+    must keep their (reduced) precision.  Results are finite in every regime, and bit-exact like everywhere else."""
+    M, N, K = 160, 288, 160
+    A, Bkn, sa, sb = make_problem(1234 + layout, M, N, K, f16=False)
+    B = b_of(Bkn, layout)
+    sa = (sa / sa.max()).astype(np.float32)
+    sb = (sb / sb.max()).astype(np.float32)                      # all in (0, 1]
+    if regime == "huge_everywhere":
+        sa, sb = sa * np.float32(2.0 ** 53), sb * np.float32(2.0 ** 52)
+    elif regime == "huge_one_block":                             # one output block (one wave) takes the fallback
+        sa[:, 2] *= np.float32(2.0 ** 53)
+        sb[:, 5] *= np.float32(2.0 ** 52)
+    elif regime == "huge_last_kblock":
+        sa[-1, :] *= np.float32(2.0 ** 53)
+        sb[-1, :] *= np.float32(2.0 ** 52)
+    else:
+        sa, sb = sa * np.float32(2.0 ** -70), sb * np.float32(2.0 ** -70)
+    want = oracle.igemm_block_f32(A, B, sa, sb, layout)
+    assert np.isfinite(want).all() and np.abs(want).max() > 0
+    dA, dB, dsa, dsb = dev(A), dev(B), dev(sa), dev(sb)
+    same(jf.igemm_block_fp(dA, dB, dsa, dsb, layout, torch.float32), want, f"{regime}: fp32 accumulators")
+    q, sc = jf.igemm_block_q(dA, dB, dsa, dsb, layout)
+    wq, wsc = oracle.igemm_block_q(A, B, sa, sb, layout, scale_dtype="f32")
+    same(q, wq, f"{regime}: codes")
+    same(sc, wsc, f"{regime}: scales")
+
+
 def test_block_q_bias(jf, oracle):
     """The forward kernel's bias / biasmax inputs (…BiasRowCol.cu:313,341,357)."""
     M, N, K = 128, 256, 96
