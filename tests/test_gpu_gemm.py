@@ -264,3 +264,47 @@ def test_full_size_xl_fc_slabs(jf, oracle):
         rb = slice(r0 // 32, r0 // 32 + 1)
         want = oracle.igemm_block_f32(GT[rows], A, np.ascontiguousarray(SG[:, rb]), SX, 1)
         same(dw[rows], want, f"wgrad rows {r0}")
+
+
+def test_full_size_stress_cube_slabs(jf, oracle):
+    """BASELINE config 5: M = N = K = 8192, heavy-tailed A (Student-t, 3 degrees of freedom), B ~ N(0, 0.02);
+    requantised output in deterministic and stochastic mode, checked bit-exactly on row slabs."""
+    n = 8192
+    g = torch.Generator().manual_seed(0)
+    a = torch.randn(n, n, generator=g) / torch.sqrt(torch.randn(3, n, n, generator=g).pow_(2).mean(0))   # t(3) = z / sqrt(chi2_3 / 3)
+    b = torch.randn(n, n, generator=g) * 0.02
+    qa, sa = jf.quantize(a.cuda(), scale_dtype=torch.float32)
+    qb, sb = jf.quantize(b.cuda(), scale_dtype=torch.float32)
+    del a, b
+    y, sy = jf.igemm_block_q(qa, qb, sa.t(), sb.t(), jf.B_NK)
+    z, sz = jf.igemm_block_q(qa, qb, sa.t(), sb.t(), jf.B_NK, rounding=jf.ROUND_STOCHASTIC, seed=5, offset=11)
+    torch.cuda.synchronize()
+    A, B, SA, SB = (t.cpu().numpy() for t in (qa, qb, sa, sb))
+    SBt = np.ascontiguousarray(SB.T)
+    for r0 in (0, 5088, 8160):
+        rows, rb = slice(r0, r0 + 32), slice(r0 // 32, r0 // 32 + 1)
+        acc = oracle.igemm_block_f32(A[rows], B, np.ascontiguousarray(SA[rb].T), SBt, 0)
+        wq, wsc = oracle.requant(acc)
+        same(y[rows], wq, f"det codes rows {r0}")
+        same(sy[rb], wsc, f"det scales rows {r0}")
+        wq, wsc = oracle.requant(acc, stochastic=True, seed=5, offset=11 + r0 * n // 8)
+        same(z[rows], wq, f"SR codes rows {r0}")
+        same(sz[rb], wsc, f"SR scales rows {r0}")
+
+
+def test_full_size_small_wgrad_deep_k(jf, oracle):
+    """BASELINE config 2 (GPT-2 small, 12288 tokens): the weight gradient of the qkv layer, K = 12288 deep with few
+    output tiles (2304 x 768), both operands read in place from their token-major arrays' natural layouts."""
+    T, Cin, Cout = 12288, 768, 2304
+    g = torch.Generator().manual_seed(0)
+    x = torch.randn(T, Cin, generator=g)
+    dy = torch.randn(T, Cout, generator=g) * 1e-3
+    qx, sx = jf.quantize(x.cuda(), scale_dtype=torch.float32)
+    qg, sg, qgT = jf.quantize(dy.cuda(), rounding=jf.ROUND_STOCHASTIC, scale_dtype=torch.float32, transpose=True, seed=0, offset=0)
+    dw = jf.igemm_block_fp(qgT, qx, sg, sx, jf.B_KN, torch.float32)
+    torch.cuda.synchronize()
+    GT, X, SG, SX = (t.cpu().numpy() for t in (qgT, qx, sg, sx))
+    for r0 in (0, 1120, 2272):
+        rows, rb = slice(r0, r0 + 32), slice(r0 // 32, r0 // 32 + 1)
+        want = oracle.igemm_block_f32(GT[rows], X, np.ascontiguousarray(SG[:, rb]), SX, 1)
+        same(dw[rows], want, f"wgrad rows {r0}")

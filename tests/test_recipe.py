@@ -66,6 +66,6 @@ def test_small_stack_trains():
         loss = F.mse_loss(model(x), target)
         loss.backward()
         opt.step()
-        losses.append(float(loss))
+        losses.append(float(loss.detach()))
     assert losses[-1] < 0.8 * losses[0], losses
     assert all(torch.isfinite(p).all() for p in model.parameters())
