@@ -469,9 +469,8 @@ __global__ __launch_bounds__(64 * WGM * WGN, WGPC * WGM * WGN / 4) void igemm_nt
                 for (int v = 0; v < 16; ++v) chk = __builtin_fmaf(acc[i][j][v], 0.0f, chk);
         if (__builtin_expect(__ballot(chk != chk) != 0, 0)) {
             const ST *const sa_t = reinterpret_cast<const ST *>(p.sa), *const sb_t = reinterpret_cast<const ST *>(p.sb);
-#pragma unroll 1
-            for (int blk = 0; blk < NBLK; ++blk) {
-                const int i = blk / WBN, j = blk % WBN;
+            static_for<0, NBLK>([&](auto blk_c) {              // compile-time block index: no indexed register arrays
+                constexpr int blk = decltype(blk_c)::value, i = blk / WBN, j = blk % WBN;
                 const size_t arow = (size_t)(mb[i] * QB + (lane & 31)), bcol = (size_t)(nb[j] * QB + (lane & 31));
                 float r[16];
 #pragma unroll
@@ -499,14 +498,9 @@ __global__ __launch_bounds__(64 * WGM * WGN, WGPC * WGM * WGN / 4) void igemm_nt
 #pragma unroll
                     for (int v = 0; v < 16; ++v) r[v] = __builtin_fmaf(sab, (float)d[v], r[v]);
                 }
-                static_for<0, NBLK>([&](auto n_c) {
-                    constexpr int n = decltype(n_c)::value;
-                    if (n == blk) {
 #pragma unroll
-                        for (int v = 0; v < 16; ++v) acc[n / WBN][n % WBN][v] = r[v];
-                    }
-                });
-            }
+                for (int v = 0; v < 16; ++v) acc[i][j][v] = r[v];
+            });
         }
     }
     __syncthreads();           // the epilogue reuses the ring as scratch
