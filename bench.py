@@ -24,7 +24,7 @@ for p in (ROOT, PKG):
         sys.path.insert(0, p)
 
 INT8_PEAK_TOPS = 5000.0      # MI355X dense INT8 MFMA peak, tera-ops/s
-MEASURED_TRAFFIC_BYTES = 150.1e6   # fc forward GEMM: 97.3 MB fetched + 52.8 MB written per launch (counter run)
+MEASURED_TRAFFIC_BYTES = 150.2e6   # fc forward GEMM: 97.3 MB fetched + 52.8 MB written per launch (counter run)
 TOKENS = 8192
 LAYERS = [("qkv", 1600, 4800), ("proj", 1600, 1600), ("fc", 1600, 6400), ("fc2", 6400, 1600)]
 

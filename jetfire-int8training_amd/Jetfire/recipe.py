@@ -8,6 +8,8 @@ float8_e4m3fn (same bytes), exactly as the reference does (qmodel.py:131,153,230
 
 Linear biases are not part of the data flow (the reference ignores them as well); LayerNorm has a weight only.
 """
+import weakref
+
 import torch
 import torch.nn as nn
 import torch.nn.functional as F
@@ -19,6 +21,36 @@ from Nonlinear import (int8_add_Ifp_Ig16_Ofp_Og, int8_add_Ifp_Ig16_Ofp_Og_MeanVa
 
 QB = 32
 _F8 = torch.float8_e4m3fn
+
+
+class WeightCodes:
+    """INT8 codes and scales of weights, made once per weight VERSION instead of once per forward.
+
+    The reference re-quantises every weight in every forward (qmodel.py:92,139,199-200) although a weight only changes
+    in the optimizer step.  A tensor's version counter is bumped by every in-place update (optimizer steps, `copy_`,
+    `add_` under no_grad), so (tensor identity, version) names the weight's current value; deterministic rounding makes
+    the cached codes identical to re-quantised ones.  Entries die with their tensors."""
+
+    def __init__(self):
+        self._entries = {}
+        self.hits = self.misses = 0
+
+    def get(self, w):
+        key = id(w)
+        e = self._entries.get(key)
+        if e is not None and e[0]() is w and e[1] == w._version and e[2] == w.data_ptr():
+            self.hits += 1
+            return e[3], e[4]
+        self.misses += 1
+        q, s = int8_quantize(w.detach(), QB)
+        self._entries[key] = (weakref.ref(w, lambda _r, k=key, d=self._entries: d.pop(k, None)), w._version, w.data_ptr(), q, s)
+        return q, s
+
+    def clear(self):
+        self._entries.clear()
+
+
+weight_codes = WeightCodes()
 
 
 def _as_f8(q):
@@ -61,7 +93,7 @@ class AttentionIn(torch.autograd.Function):
 
     @staticmethod
     def forward(ctx, residual, qx, sx, w_qkv, ln_w, mean, rstd):
-        qw, sw = int8_quantize(w_qkv, QB)
+        qw, sw = weight_codes.get(w_qkv)
         qx = _as_s8(qx)
         qn, sn, _ = int8_layernorm_forward(qx, sx, ln_w, mean, rstd, QB)
         qkv = int8_linear_forward(qn, sn, qw, sw, False, QB)
@@ -83,7 +115,7 @@ class AttentionOut(torch.autograd.Function):
 
     @staticmethod
     def forward(ctx, residual, y, w_proj):
-        qw, sw = int8_quantize(w_proj, QB)
+        qw, sw = weight_codes.get(w_proj)
         qy, sy = int8_quantize(y.contiguous(), QB)
         qo, so = int8_linear_forward(qy, sy, qw, sw, True, QB)
         fp, q, s, mean, rstd = int8_add_Ifp_Ig16_Ofp_Og_MeanVar(residual.contiguous(), qo, so, QB)
@@ -105,8 +137,8 @@ class MLPResidual(torch.autograd.Function):
     @staticmethod
     def forward(ctx, residual, qx, sx, w_fc, w_proj, ln_w, mean, rstd):
         qx = _as_s8(qx)
-        qw1, sw1 = int8_quantize(w_fc, QB)
-        qw2, sw2 = int8_quantize(w_proj, QB)
+        qw1, sw1 = weight_codes.get(w_fc)
+        qw2, sw2 = weight_codes.get(w_proj)
         qn, sn, _ = int8_layernorm_forward(qx, sx, ln_w, mean, rstd, QB)
         qh, sh = int8_linear_forward(qn, sn, qw1, sw1, True, QB)
         qa, sa = int8_gelu_forward(qh, sh, QB)

@@ -371,34 +371,29 @@ __global__ __launch_bounds__(NT) void rowstats_kernel(const int8_t *q, const ST 
     }
 }
 
-// Column sums over the 32 rows of a block: lane l holds row l/2 and 32 values (index i) of column set l%2.  The 8 lanes
-// of a 16-lane row that share l%2 are summed by rotations inside the vector ALU (+2, +4, +8 lanes), the four rows
-// through a small LDS patch.  On return lane l holds the total of value index l/2 for column set l%2
-// (a fixed tree: reproducible).  `patch` = 256 floats private to the wave.
-__device__ __forceinline__ float colsum32_over_rows(const float (&v)[32], int lane, float *patch)
+// Column sums over the 32 rows of a block: lane l holds row l/2 and 16 values (index k) of column set l%2.  The values
+// go through a wave-private LDS patch, value k of lane l at word 66*k + l; lane j then adds rows 16*(j%2) .. +15 of
+// output j/2 = (value index k = j/4, column set (j/2)%2) and the two halves are combined with one lane swap.  The pitch
+// of 66 words puts the 64 lanes of every read (and of every write) on 64 different banks.  Plain adds in a fixed order
+// (reproducible); moving data through LDS costs this kernel's bottleneck, the vector ALU, 17 instructions where a
+// cross-lane butterfly costs 3 per value.  On return lanes with j%2 == 0 hold the total of output j/2.
+constexpr int COLSUM_PITCH = 66, COLSUM_PATCH = 16 * COLSUM_PITCH;   // floats per wave
+__device__ __forceinline__ float colsum16_over_rows(const float (&v)[16], int lane, float *patch)
 {
-    auto rot_add = [](float x, auto ctrl_c) {
-        const int t = __builtin_amdgcn_update_dpp(0, __float_as_int(x), decltype(ctrl_c)::value, 0xF, 0xF, false);
-        return x + __int_as_float(t);
-    };
-    const int row = lane >> 4, set = lane & 1;
 #pragma unroll
-    for (int i = 0; i < 32; ++i) {
-        float x = v[i];
-        x = rot_add(x, std::integral_constant<int, 0x122>{});      // row_ror:2
-        x = rot_add(x, std::integral_constant<int, 0x124>{});      // row_ror:4
-        x = rot_add(x, std::integral_constant<int, 0x128>{});      // row_ror:8
-        if ((lane & 15) < 2) patch[(row * 2 + set) * 32 + i] = x;  // one lane per (row of lanes, column set)
-    }
+    for (int k = 0; k < 16; ++k) patch[k * COLSUM_PITCH + lane] = v[k];
     __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
     __builtin_amdgcn_wave_barrier();
     __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
-    const int i = lane >> 1;
-    const float total = ((patch[(0 * 2 + set) * 32 + i] + patch[(1 * 2 + set) * 32 + i]) +
-                         (patch[(2 * 2 + set) * 32 + i] + patch[(3 * 2 + set) * 32 + i]));
+    const float *src = patch + (lane >> 2) * COLSUM_PITCH + ((lane >> 1) & 1) + 32 * (lane & 1);
+    float t = src[0];
+#pragma unroll
+    for (int i = 1; i < 16; ++i) t = t + src[2 * i];
+    const int o = __builtin_amdgcn_update_dpp(0, __float_as_int(t), 0xB1, 0xF, 0xF, false);   // quad_perm [1,0,3,2]
+    t = t + __int_as_float(o);                                     // both lanes of the pair: same two operands
     __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
     __builtin_amdgcn_wave_barrier();                               // the patch may be rewritten
-    return total;
+    return t;
 }
 
 constexpr int LNB_THREADS = 1024;
@@ -419,13 +414,13 @@ __global__ __launch_bounds__(LNB_THREADS) void layernorm_bwd_fused_kernel(const 
     const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
     const int SC = C / QB, H = C / 16, rb = blockIdx.x;
     float *part1 = fsm, *part2 = fsm + QB * H, *c1s = part2 + QB * H, *c2s = c1s + QB;
-    float *cpatch = c2s + QB + wave * 256;
+    float *cpatch = c2s + QB + wave * COLSUM_PATCH;
     const int r = lane >> 1;
     const float mu = mean[rb * QB + r], rs = rstd[rb * QB + r];
     for (int cb = wave; cb < SC; cb += LNB_THREADS / WAVE) {
         const int col = cb * QB + (lane & 1) * 16;
         const size_t e0 = (size_t)(rb * QB + r) * C + col;
-        float x[16], g[16], w[16], v[32];
+        float x[16], g[16], w[16], v[16];
         unpack16(*reinterpret_cast<const v4i *>(qx + e0), load_scale(sx, rb * SC + cb), x);
         unpack16(*reinterpret_cast<const v4i *>(qg + e0), load_scale(sg, rb * SC + cb), g);
         Load16<float>::run(gamma + col, w);
@@ -437,15 +432,16 @@ __global__ __launch_bounds__(LNB_THREADS) void layernorm_bwd_fused_kernel(const 
             p1 = __builtin_fmaf(xh, wdy, p1);
             p2 = p2 + wdy;
             v[k] = g[k] * xh;
-            v[16 + k] = g[k];
         }
         part1[r * H + cb * 2 + (lane & 1)] = p1;
         part2[r * H + cb * 2 + (lane & 1)] = p2;
         if (pdg) {
-            const float total = colsum32_over_rows(v, lane, cpatch);
-            const int idx = lane >> 1;                             // 0..15: sum of dy*xhat, 16..31: sum of dy
-            float *dst = (idx & 16) ? pdb : pdg;
-            dst[(size_t)rb * C + cb * QB + (lane & 1) * 16 + (idx & 15)] = total;
+            // output of lane j (j even): value index j/4 of column set (j/2)%2
+            const size_t dst = (size_t)rb * C + cb * QB + ((lane >> 1) & 1) * 16 + (lane >> 2);
+            const float tg = colsum16_over_rows(v, lane, cpatch);  // sum of dy*xhat
+            if ((lane & 1) == 0) pdg[dst] = tg;
+            const float tb = colsum16_over_rows(g, lane, cpatch);  // sum of dy
+            if ((lane & 1) == 0) pdb[dst] = tb;
         }
     }
     __syncthreads();
@@ -660,9 +656,9 @@ int jf_layernorm_bwd(const int8_t *qx, const void *sx, const int8_t *qg, const v
     if (!aligned16(qdx) || !aligned16(gamma)) return JF_ERR_ALIGN;
     if (!workspace || workspace_bytes < jf_layernorm_bwd_workspace_bytes(R, C)) return JF_ERR_WORKSPACE;
     if (!aligned16(workspace)) return JF_ERR_ALIGN;
-    // LDS: two [32][C/16] partial-sum arrays, c1/c2, one 1 KiB column-sum patch per wave
-    const size_t smem = ((size_t)2 * QB * (C / 16) + 2 * QB + (LNB_THREADS / WAVE) * 256) * sizeof(float);
-    if (smem > 160 * 1024 - 512) return JF_ERR_SHAPE;          // rows of up to ~8000 columns
+    // LDS: two [32][C/16] partial-sum arrays, c1/c2, one column-sum patch per wave
+    const size_t smem = ((size_t)2 * QB * (C / 16) + 2 * QB + (LNB_THREADS / WAVE) * COLSUM_PATCH) * sizeof(float);
+    if (smem > 160 * 1024 - 512) return JF_ERR_SHAPE;          // rows of up to ~5700 columns
     hipStream_t st = (hipStream_t)stream;
     const bool want_dw = dgamma || dbeta;
     // workspace: [2R floats, unused by this implementation][strips x C partial dgamma][strips x C partial dbeta]

@@ -69,3 +69,35 @@ def test_small_stack_trains():
         losses.append(float(loss.detach()))
     assert losses[-1] < 0.8 * losses[0], losses
     assert all(torch.isfinite(p).all() for p in model.parameters())
+
+
+def test_weight_codes_are_cached_per_weight_version():
+    """A weight is quantised once per value: repeated forwards reuse its codes, an optimizer-style in-place update
+    re-quantises it, and cached codes are the ones a fresh quantisation gives."""
+    import recipe
+    from Nonlinear import int8_quantize
+    torch.manual_seed(2)
+    model = recipe.QStack(1, 128, 4).cuda()
+    x = torch.randn(2, 64, 128, device="cuda")
+    recipe.weight_codes.clear()
+    recipe.weight_codes.hits = recipe.weight_codes.misses = 0
+    with torch.no_grad():
+        y0 = model(x)
+        assert (recipe.weight_codes.misses, recipe.weight_codes.hits) == (4, 0)
+        y1 = model(x)
+        assert (recipe.weight_codes.misses, recipe.weight_codes.hits) == (4, 4)
+        assert torch.equal(y0, y1)
+        w = model.blocks[0].w_fc
+        q, s = recipe.weight_codes.get(w)
+        q2, s2 = int8_quantize(w.detach(), 32)
+        assert torch.equal(q, q2) and torch.equal(s, s2)
+        w.mul_(2.0)                                               # what an optimizer step does: in place, new version
+        q3, s3 = recipe.weight_codes.get(w)
+        assert recipe.weight_codes.misses == 5
+        assert torch.equal(q3, q) and not torch.equal(s3, s)      # same codes (exact rescale by 2), doubled scales
+        y2 = model(x)
+        assert not torch.equal(y2, y1)
+    del model, w
+    import gc
+    gc.collect()
+    assert len(recipe.weight_codes._entries) == 0
