@@ -36,6 +36,12 @@ extern "C" {
 #define JF_ERR_ALIGN         -4   /* pointer or leading dimension not 16-byte aligned */
 #define JF_ERR_WORKSPACE     -5   /* workspace missing or smaller than required      */
 #define JF_ERR_DEVICE        -6   /* the current device is not gfx950                */
+#define JF_ERR_UNSUPPORTED   -7   /* valid codes, but this combination of layouts is not implemented */
+
+/* A operand layout of jf_igemm_block_fp (every other GEMM entry point takes A as [M,K]) */
+#define JF_A_MK 0                 /* A is [M,K] row-major                                                          */
+#define JF_A_KM 1                 /* A is [K,M] row-major: the un-transposed gradient [tokens, C_out] of a weight
+                                     gradient; implemented together with JF_B_KN (else JF_ERR_UNSUPPORTED)         */
 
 /* B operand layout of the GEMMs */
 #define JF_B_NK 0                 /* B is [N,K] row-major ("row x col", forward)      */
@@ -80,10 +86,12 @@ int jf_igemm_block_acc(const int8_t *A, const int8_t *B, int32_t *acc, int M, in
                        void *workspace, size_t workspace_bytes, jf_stream_t stream);
 
 /* C_fp[M,N] = sum_kb sa*sb*(A_kb*B_kb), fp32 accumulate in ascending kb, stored as out_dtype.
- * Replaces igemm_output_fp_no_quantize (include/igemm.h:14-25, igemm/igemm_BlockSquare32OutputFp.cu:340-382). */
+ * Replaces igemm_output_fp_no_quantize (include/igemm.h:14-25, igemm/igemm_BlockSquare32OutputFp.cu:340-382).
+ * With a_layout = JF_A_KM the weight gradient dW = dY^T X is computed from dY [tokens, C_out] as it lies in memory:
+ * the reference's callers materialise dY^T first (Linear/linear_bwd.py:21, Nonlinear/transpose.py:69-97). */
 int jf_igemm_block_fp(const int8_t *A, const int8_t *B, const void *sa, const void *sb, void *C,
-                      int M, int N, int K, int b_layout, int scale_dtype, int sa_layout, int sb_layout, int out_dtype,
-                      void *workspace, size_t workspace_bytes, jf_stream_t stream);
+                      int M, int N, int K, int a_layout, int b_layout, int scale_dtype, int sa_layout, int sb_layout,
+                      int out_dtype, void *workspace, size_t workspace_bytes, jf_stream_t stream);
 
 /* (C_s8[M,N], sc[M/32,N/32]) = per-32x32-block requantisation of the same accumulation.
  *   rounding JF_ROUND_NEAREST : q = clamp(rn(127*(acc+bias[n]) / (amax+biasmax)), +-127)

@@ -4,7 +4,9 @@ Data format everywhere: codes int8 [..., R, C] with one scale per 32x32 tile, sc
 (float16 as in the reference, float32 accepted).  The GEMM entry points take their scale operands as [K/32, rows/32];
 the reference makes transposed copies for that (linear_fwd.py:17-18, linear_bwd.py:11), here the .t() VIEW of the
 block tensor's own scale array is passed and the kernel reads it in place.  The zero bias the reference allocates on
-every call (linear_fwd.py:20-21) is kept per device and width.
+every call (linear_fwd.py:20-21) is kept per device and width.  The weight-gradient GEMM reads the gradient
+[tokens, C_out] in place as its [K, M] operand when no pre-transposed copy is supplied (G8T=None); the reference needs
+the copy (linear_bwd.py:21, made by int8_transpose / int8_quantize_transpose).
 """
 import os
 import sys
@@ -70,7 +72,8 @@ def int8_linear_forward(X8_3D, SX16_3D, W8, SW16, output_quantized, B):
 
 def int8_linear_backward(X8_3D, SX16_3D, G8_3D, SG16_3D, G8T, W8, SW16, B, stochastic=True, dgrad_quantize=True):
     """dX = dY W (requantised with stochastic rounding) and dW = dY^T X (fp16).
-    G8 [BS,T,N] with SG [BS,T/32,N/32]; G8T = G8 transposed to [N, BS*T]; W8 [N,K], SW [N/32,K/32].
+    G8 [BS,T,N] with SG [BS,T/32,N/32]; G8T = G8 transposed to [N, BS*T], or None (then G8 itself is read, no copy);
+    W8 [N,K], SW [N/32,K/32].
     Returns (GX8, GSX, GW) or (GX_fp, GW) when dgrad_quantize=False (reference: linear_bwd.py:4-29; like
     there, the activation gradient is always rounded stochastically)."""
     _check_block(B)
@@ -79,6 +82,8 @@ def int8_linear_backward(X8_3D, SX16_3D, G8_3D, SG16_3D, G8T, W8, SW16, B, stoch
     tokens, c_out = g2.shape
     c_in = W8.shape[1]
     gx8, gsx = BQC.igemm_output_int_quantize_stochastic(g2, W8, _k_major(sg2), SW16, tokens, c_in, c_out)
+    if G8T is None:
+        G8T = g2.t()                                               # a view: the extension reads g2 as the [K, M] operand
     gw = BQC.igemm_output_fp_no_quantize(G8T, x2, sg2, sx2, G8T.shape[0], c_in, G8T.shape[1])
     if not dgrad_quantize:
         return _dequant_like(gx8, gsx, tuple(G8_3D.shape[:-1])), gw

@@ -6,6 +6,10 @@ Counterpart of the autograd Functions of the reference recipe (INT8_GPT2/qmodel.
 scales).  Autograd only carries floating tensors, so the INT8 codes cross Function boundaries re-viewed as
 float8_e4m3fn (same bytes), exactly as the reference does (qmodel.py:131,153,230,266).
 
+Two per-call costs of the reference are gone: weights are quantised once per weight version (WeightCodes below), and no
+transposed gradient is materialised for the weight-gradient GEMMs (the reference calls int8_transpose /
+int8_quantize_transpose before every one, qmodel.py:156,237,250; here the GEMM reads the gradient in place).
+
 Linear biases are not part of the data flow (the reference ignores them as well); LayerNorm has a weight only.
 """
 import weakref
@@ -16,8 +20,7 @@ import torch.nn.functional as F
 
 from Linear import int8_linear_backward, int8_linear_forward
 from Nonlinear import (int8_add_Ifp_Ig16_Ofp_Og, int8_add_Ifp_Ig16_Ofp_Og_MeanVar, int8_gelu_backward, int8_gelu_forward,
-                       int8_layernorm_backward, int8_layernorm_forward, int8_quantize, int8_quantize_transpose,
-                       int8_transpose)
+                       int8_layernorm_backward, int8_layernorm_forward, int8_quantize)
 
 QB = 32
 _F8 = torch.float8_e4m3fn
@@ -103,8 +106,8 @@ class AttentionIn(torch.autograd.Function):
     @staticmethod
     def backward(ctx, fpg, g):
         qx, sx, qn, sn, qw, sw, ln_w, mean, rstd = ctx.saved_tensors
-        qg, sg, qgt = int8_quantize_transpose(g.contiguous(), QB, stochastic=True, transpose_output_2d=True)
-        qg, sg, gw = int8_linear_backward(qn, sn, qg, sg, qgt, qw, sw, QB, stochastic=True)
+        qg, sg = int8_quantize(g.contiguous(), QB, stochastic=True)
+        qg, sg, gw = int8_linear_backward(qn, sn, qg, sg, None, qw, sw, QB, stochastic=True)
         qg, sg, g_ln = int8_layernorm_backward(qx, sx, qg, sg, ln_w, QB, mean, rstd, stochastic=True)
         res_g, qg, sg = int8_add_Ifp_Ig16_Ofp_Og(fpg.contiguous(), qg, sg, QB, stochastic=True)
         return res_g, _as_f8(qg), sg, gw, g_ln, None, None
@@ -126,8 +129,7 @@ class AttentionOut(torch.autograd.Function):
     def backward(ctx, fpg, qg, sg, _m, _r):
         qy, sy, qw, sw = ctx.saved_tensors
         qg = _as_s8(qg)
-        qgt = int8_transpose(qg, transpose_output_2d=True)
-        g, gw = int8_linear_backward(qy, sy, qg, sg, qgt, qw, sw, QB, stochastic=True, dgrad_quantize=False)
+        g, gw = int8_linear_backward(qy, sy, qg, sg, None, qw, sw, QB, stochastic=True, dgrad_quantize=False)
         return fpg, g, gw
 
 
@@ -151,11 +153,9 @@ class MLPResidual(torch.autograd.Function):
     def backward(ctx, fpg, qg, sg, _m, _r):
         qx, sx, qn, sn, qh, sh, qa, sa, qw1, sw1, qw2, sw2, ln_w, mean, rstd = ctx.saved_tensors
         qg = _as_s8(qg)
-        qgt = int8_transpose(qg, transpose_output_2d=True)
-        qg, sg, gw2 = int8_linear_backward(qa, sa, qg, sg, qgt, qw2, sw2, QB, stochastic=True)
+        qg, sg, gw2 = int8_linear_backward(qa, sa, qg, sg, None, qw2, sw2, QB, stochastic=True)
         qg, sg = int8_gelu_backward(qh, sh, qg, sg, QB, stochastic=True)
-        qgt = int8_transpose(qg, transpose_output_2d=True)
-        qg, sg, gw1 = int8_linear_backward(qn, sn, qg, sg, qgt, qw1, sw1, QB, stochastic=True)
+        qg, sg, gw1 = int8_linear_backward(qn, sn, qg, sg, None, qw1, sw1, QB, stochastic=True)
         qg, sg, g_ln = int8_layernorm_backward(qx, sx, qg, sg, ln_w, QB, mean, rstd, stochastic=True)
         res_g, qg, sg = int8_add_Ifp_Ig16_Ofp_Og(fpg.contiguous(), qg, sg, QB, stochastic=True)
         return res_g, _as_f8(qg), sg, gw1, gw2, g_ln, None, None

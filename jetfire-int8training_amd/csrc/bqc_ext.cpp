@@ -49,6 +49,19 @@ void check_a(const torch::Tensor &X, int64_t M, int64_t K)
     TORCH_CHECK(X.is_contiguous(), "X must be contiguous");
 }
 
+// A of the weight-gradient GEMM: [M,K] contiguous (the reference's pre-transposed gradient G8T), or the .t() view
+// of a contiguous [K,M] tensor (strides (1,M)), i.e. the gradient [tokens, C_out] as it lies in memory: JF_A_KM.
+int check_a_any_layout(const torch::Tensor &X, int64_t M, int64_t K)
+{
+    TORCH_CHECK(X.is_cuda(), "X must be a GPU tensor");
+    TORCH_CHECK(X.scalar_type() == torch::kInt8, "X must be int8, got ", X.scalar_type());
+    TORCH_CHECK(X.dim() == 2 && X.size(0) == M && X.size(1) == K, "X must be [M,K] = [", M, ",", K, "], got ", X.sizes());
+    if (X.is_contiguous()) return JF_A_MK;
+    TORCH_CHECK(X.stride(0) == 1 && X.stride(1) == M,
+                "X must be contiguous or the .t() view of a contiguous [K,M] tensor, got strides ", X.strides());
+    return JF_A_KM;
+}
+
 // B as [K,N] row-major ("row x row" functions).
 void check_b_kn(const torch::Tensor &W, const torch::Tensor &X, int64_t K, int64_t N)
 {
@@ -226,7 +239,7 @@ torch::Tensor igemm_output_fp_no_quantize(torch::Tensor X, torch::Tensor W, torc
                                           const int M, const int N, const int K)
 {
     check_dims(M, N, K);
-    check_a(X, M, K);
+    const int a_layout = check_a_any_layout(X, M, K);
     check_b_kn(W, X, K, N);
     int sxl, swl;
     const int code = check_scales(SX, SW, X, M, N, K, sxl, swl);
@@ -235,7 +248,8 @@ torch::Tensor igemm_output_fp_no_quantize(torch::Tensor X, torch::Tensor W, torc
     Workspace ws(X, M, N, K, JF_B_KN);
     pybind11::gil_scoped_release nogil;
     check_rc(jf_igemm_block_fp((const int8_t *)X.data_ptr(), (const int8_t *)W.data_ptr(), SX.data_ptr(), SW.data_ptr(),
-                               O.data_ptr(), M, N, K, JF_B_KN, code, sxl, swl, JF_FP_F16, ws.ptr, ws.bytes, current_stream(X)),
+                               O.data_ptr(), M, N, K, a_layout, JF_B_KN, code, sxl, swl, JF_FP_F16, ws.ptr, ws.bytes,
+                               current_stream(X)),
              "igemm_output_fp_no_quantize");
     return O;
 }

@@ -38,7 +38,7 @@ constexpr int EPI_LD = 36;                          // floats per staged row (32
 enum Epilogue { EPI_S32 = 0, EPI_FP = 1, EPI_Q = 2 };
 
 struct GemmArgs {
-    const int8_t *A;      // [M, lda]
+    const int8_t *A;      // [M, lda] (K-contiguous) or, for the AKM kernels, [K, lda] (M-contiguous rows)
     const int8_t *B;      // [N, ldb] (K-contiguous) or, for the BKN kernels, [K, ldb] (N-contiguous)
     const void *sa;       // scale of A block (mb, kb) at sa[kb * sa_ks + mb * sa_is]
     const void *sb;       // scale of B block (nb, kb) at sb[kb * sb_ks + nb * sb_is]
@@ -88,9 +88,10 @@ template <int I, int N, typename F> __device__ __forceinline__ void static_for(F
 constexpr int WBM = 2, WBN = 1;
 // NSTAGE = depth of the LDS ring (one stage being computed, NSTAGE-1 in flight); WGPC = workgroups per CU
 // (the second launch bound counts waves per SIMD: WGPC workgroups of WGM*WGN waves over 4 SIMDs).
+// AKM = 1: A is [K, lda] (M-contiguous rows), staged and read like a [K,N] B operand (below).
 // BKN = 0: B is [N, ldb] (K-contiguous rows, like A).  BKN = 1: B is [K, ldb] (N-contiguous rows); its tile is staged
 // as it lies in memory and the K-contiguous MFMA operand is produced by the transposing LDS read of gfx950.
-template <int EPI, typename ST, int WGM, int WGN, int NSTAGE, int WGPC, int BKN>
+template <int EPI, typename ST, int WGM, int WGN, int NSTAGE, int WGPC, int BKN, int AKM = 0>
 __global__ __launch_bounds__(64 * WGM * WGN, WGPC * WGM * WGN / 4) void igemm_nt_kernel(GemmArgs p)
 {
     constexpr int NW = WGM * WGN;
@@ -102,6 +103,7 @@ __global__ __launch_bounds__(64 * WGM * WGN, WGPC * WGM * WGN / 4) void igemm_nt
     static_assert(GROUPS % NW == 0, "stage must split evenly over the waves");
     static_assert(NSTAGE >= 2 && NSTAGE <= 5, "ring depth");
     static_assert(!BKN || (BN == ROW_BYTES && WBN == 1), "a staged [K,N] row is one 128-byte LDS row");
+    static_assert(!AKM || BM == ROW_BYTES, "a staged [K,M] row is one 128-byte LDS row");
 
     extern __shared__ __attribute__((aligned(16))) unsigned char smem[];
     typedef __attribute__((address_space(3))) unsigned char lds_u8;
@@ -130,7 +132,10 @@ __global__ __launch_bounds__(64 * WGM * WGN, WGPC * WGM * WGN / 4) void igemm_nt
     static_assert(NW % 2 == 0, "the chunk swizzle of a lane must not depend on the load index");
     const int lrow = lane >> 3;
     const int gchunk = (lane & 7) ^ (((wave & 1) * 4 + (lane >> 4)) & 7);     // global chunk this lane fetches
-    const unsigned loff_a = (unsigned)lrow * (unsigned)p.lda + gchunk * 16;
+    // A as [K,M]: as for B as [K,N] below (8 K rows x 128 M bytes per load, slot c' of row r holds chunk c' ^ r)
+    const int km_chunk = (m0 + (((lane & 7) ^ lrow) << 4)) < p.M ? ((lane & 7) ^ lrow) : 0;
+    const unsigned loff_a = AKM ? (unsigned)lrow * (unsigned)p.lda + km_chunk * 16
+                                : (unsigned)lrow * (unsigned)p.lda + gchunk * 16;
     // B as [K,N]: a load moves 8 K rows x 128 N bytes (group g of a stage = K rows 8g .. 8g+7 of the stage).  Slot c'
     // of row r holds global chunk c' ^ r, which makes the transposing reads below conflict-free.  Chunks beyond N (partial
     // tile) fetch the tile's first chunk instead (never used).
@@ -146,6 +151,8 @@ __global__ __launch_bounds__(64 * WGM * WGN, WGPC * WGM * WGN / 4) void igemm_nt
         if (BKN && !is_a[j]) {
             const int k0 = (grp - BM / 8) * 8;                     // K row of the stage (redirected at issue time if beyond K)
             gbase[j] = p.B + (size_t)k0 * (size_t)p.ldb + n0;
+        } else if (AKM && is_a[j]) {
+            gbase[j] = p.A + (size_t)(grp * 8) * (size_t)p.lda + m0;
         } else {
             int r0 = (is_a[j] ? m0 : n0) + (is_a[j] ? grp : grp - BM / 8) * 8;
             if (r0 >= (is_a[j] ? p.M : p.N)) r0 = is_a[j] ? m0 : n0;   // groups of a partial tile: any valid group
@@ -195,7 +202,7 @@ __global__ __launch_bounds__(64 * WGM * WGN, WGPC * WGM * WGN / 4) void igemm_nt
         }
         unsigned la = loff_a, lb = loff_b;
         if (!FULL && kb0 + (gchunk >> 1) >= nkb) {            // chunks of missing K blocks: the stage's first block again
-            la -= (unsigned)(gchunk >> 1) * QB;
+            if (!AKM) la -= (unsigned)(gchunk >> 1) * QB;
             if (!BKN) lb -= (unsigned)(gchunk >> 1) * QB;
         }
 #pragma unroll
@@ -206,6 +213,9 @@ __global__ __launch_bounds__(64 * WGM * WGN, WGPC * WGM * WGN / 4) void igemm_nt
                 base = gbase[j] + (size_t)kb0 * QB * (size_t)p.ldb;
                 // K rows of a missing K block: the stage's first group again
                 if (!FULL && kb0 * QB + (grp - BM / 8) * 8 >= p.K) base -= (size_t)((grp - BM / 8) * 8) * (size_t)p.ldb;
+            } else if (AKM && j < A_LOADS) {
+                base = gbase[j] + (size_t)kb0 * QB * (size_t)p.lda;
+                if (!FULL && kb0 * QB + grp * 8 >= p.K) base -= (size_t)(grp * 8) * (size_t)p.lda;
             } else {
                 base = gbase[j] + (size_t)kb0 * QB;
             }
@@ -240,6 +250,13 @@ __global__ __launch_bounds__(64 * WGM * WGN, WGPC * WGM * WGN / 4) void igemm_nt
         const int g = lane >> 4, r = lane & 15, rho = r >> 1;
         const int c = 2 * wn * WBN + (g & 1);                                    // 16-byte chunk of the N strip
         fb_kn = (unsigned)(uintptr_t)lds + A_BYTES + (g >> 1) * 2048 + ((rho * 8 + (c ^ rho)) << 4) + 8 * (r & 1);
+    }
+    unsigned fa_km[WBM];                                                             // A staged as [K,M]: the same, per block
+#pragma unroll
+    for (int i = 0; i < WBM; ++i) {
+        const int g = lane >> 4, r = lane & 15, rho = r >> 1;
+        const int c = 2 * (wm * WBM + i) + (g & 1);
+        fa_km[i] = AKM ? (unsigned)(uintptr_t)lds + (g >> 1) * 2048 + ((rho * 8 + (c ^ rho)) << 4) + 8 * (r & 1) : 0u;
     }
     // scale patch of this wave: a uniform address, parked in a vector register once (LDS reads take a VGPR address)
     unsigned sc_v;
@@ -284,22 +301,35 @@ __global__ __launch_bounds__(64 * WGM * WGN, WGPC * WGM * WGN / 4) void igemm_nt
     typedef float scale_vec __attribute__((ext_vector_type(NSC == 3 ? 3 : NSC <= 2 ? 2 : 4)));
     v4i fa_reg[2][WBM], fb_reg[2][WBN];
     scale_vec sc_raw[2];
-    constexpr int FETCH_OPS = WBM + (BKN ? 2 : 1) * WBN + (EPI != EPI_S32 ? 1 : 0);
+    constexpr int FETCH_OPS = (AKM ? 2 : 1) * WBM + (BKN ? 2 : 1) * WBN + (EPI != EPI_S32 ? 1 : 0);
     static_assert(2 * FETCH_OPS <= 15, "lgkmcnt is a 4-bit counter");
     // pa/pb: this lane's fragment addresses for the K block (ring slot 0); psc: the wave's scale patch;
     // slot_bytes / slot_words: compile-time offset of the ring slot in the tile ring and of the K block in the patch
-    auto fetch = [&](const unsigned pa, const unsigned pb, const unsigned pbkn, const unsigned psc, auto slot_bytes_c,
+    // kn_base: runtime offset of the ring slot for the transposing reads (0 where the slot is in the immediates)
+    auto fetch = [&](const unsigned pa, const unsigned pb, const unsigned kn_base, const unsigned psc, auto slot_bytes_c,
                      auto kn_off_c, auto slot_words_c, auto buf_c) {
         constexpr int BUF = decltype(buf_c)::value;
         constexpr int SB = decltype(slot_bytes_c)::value, SW = decltype(slot_words_c)::value;
         // the instruction's offset field has 16 bits: slots beyond that are reached through the address register
         constexpr int HI = (SB + (WBM > WBN ? WBM : WBN) * QB * ROW_BYTES) > 65535 ? SB : 0;
         const unsigned pa2 = pa + HI, pb2 = pb + HI;
+        constexpr int KO = decltype(kn_off_c)::value;         // slot + K block offset of a [K,N] / [K,M] staging
+        if (AKM) {
 #pragma unroll
-        for (int i = 0; i < WBM; ++i)
-            asm volatile("ds_read_b128 %0, %1 offset:%2" : "=v"(fa_reg[BUF][i]) : "v"(pa2), "n"(SB - HI + i * (QB * ROW_BYTES)));
+            for (int i = 0; i < WBM; ++i) {
+                const unsigned pakm = fa_km[i] + kn_base;
+                v2i lo, hi;
+                asm volatile("ds_read_b64_tr_b8 %0, %1 offset:%2" : "=v"(lo) : "v"(pakm), "n"(KO));
+                asm volatile("ds_read_b64_tr_b8 %0, %1 offset:%2" : "=v"(hi) : "v"(pakm), "n"(KO + 1024));
+                fa_reg[BUF][i] = v4i{lo.x, lo.y, hi.x, hi.y};
+            }
+        } else {
+#pragma unroll
+            for (int i = 0; i < WBM; ++i)
+                asm volatile("ds_read_b128 %0, %1 offset:%2" : "=v"(fa_reg[BUF][i]) : "v"(pa2), "n"(SB - HI + i * (QB * ROW_BYTES)));
+        }
         if (BKN) {
-            constexpr int KO = decltype(kn_off_c)::value;     // slot + K block offset of the [K,N] staging
+            const unsigned pbkn = fb_kn + kn_base;
             v2i lo, hi;
             asm volatile("ds_read_b64_tr_b8 %0, %1 offset:%2" : "=v"(lo) : "v"(pbkn), "n"(KO));
             asm volatile("ds_read_b64_tr_b8 %0, %1 offset:%2" : "=v"(hi) : "v"(pbkn), "n"(KO + 1024));
@@ -400,7 +430,7 @@ __global__ __launch_bounds__(64 * WGM * WGN, WGPC * WGM * WGN / 4) void igemm_nt
     asm volatile("" ::: "memory");
     __builtin_amdgcn_s_barrier();                              // bare: __syncthreads() would drain every load
     asm volatile("" ::: "memory");
-    fetch(fa_u[0], fb_u[0], fb_kn, sc_v, c0{}, c0{}, c0{}, c0{});
+    fetch(fa_u[0], fb_u[0], 0u, sc_v, c0{}, c0{}, c0{}, c0{});
 
     for (int s0 = 0; s0 < nfull; s0 += NSTAGE) static_for<0, NSTAGE>([&](auto slot_c) {
         constexpr int SLOT = decltype(slot_c)::value;         // ring slot of this stage, a compile-time constant
@@ -423,11 +453,11 @@ __global__ __launch_bounds__(64 * WGM * WGN, WGPC * WGM * WGN / 4) void igemm_nt
                     if (s + NSTAGE < nstages) issue_stage(s + NSTAGE);
                 }
                 // unconditional: past the last stage it reads bytes of the ring that nobody uses
-                fetch(fa_u[0], fb_u[0], fb_kn, sc_v, std::integral_constant<int, NEXT_SLOT * STAGE_BYTES>{},
+                fetch(fa_u[0], fb_u[0], 0u, sc_v, std::integral_constant<int, NEXT_SLOT * STAGE_BYTES>{},
                       std::integral_constant<int, NEXT_SLOT * STAGE_BYTES>{},
                       std::integral_constant<int, NEXT_SLOT * 64>{}, std::integral_constant<int, NXT>{});
             } else {
-                fetch(fa_u[kb + 1], fb_u[kb + 1], fb_kn, sc_v, std::integral_constant<int, SLOT * STAGE_BYTES>{},
+                fetch(fa_u[kb + 1], fb_u[kb + 1], 0u, sc_v, std::integral_constant<int, SLOT * STAGE_BYTES>{},
                       std::integral_constant<int, SLOT * STAGE_BYTES + (kb + 1) * 4096>{},
                       std::integral_constant<int, SLOT * 64 + (kb + 1) * 16>{}, std::integral_constant<int, NXT>{});
             }
@@ -445,7 +475,7 @@ __global__ __launch_bounds__(64 * WGM * WGN, WGPC * WGM * WGN / 4) void igemm_nt
             constexpr int CUR = kb & 1;
             if (kb < ktail) {
                 if (kb > 0)
-                    fetch(fa_u[kb] + slot * STAGE_BYTES, fb_u[kb] + slot * STAGE_BYTES, fb_kn + slot * STAGE_BYTES, sc_v + slot * 256,
+                    fetch(fa_u[kb] + slot * STAGE_BYTES, fb_u[kb] + slot * STAGE_BYTES, slot * STAGE_BYTES, sc_v + slot * 256,
                           c0{}, std::integral_constant<int, kb * 4096>{}, std::integral_constant<int, kb * 16>{},
                           std::integral_constant<int, CUR>{});
                 fetched(c0{}, std::integral_constant<int, CUR>{});
@@ -478,7 +508,19 @@ __global__ __launch_bounds__(64 * WGM * WGN, WGPC * WGM * WGN / 4) void igemm_nt
 #pragma unroll 1
                 for (int kb = 0; kb < nkb; ++kb) {
                     const int k0 = kb * QB + 16 * (lane >> 5);
-                    const v4i fa = *reinterpret_cast<const v4i *>(p.A + arow * (size_t)p.lda + k0);
+                    v4i fa;
+                    if (AKM) {
+                        const int8_t *src = p.A + (size_t)k0 * (size_t)p.lda + arow;
+#pragma unroll
+                        for (int c = 0; c < 4; ++c) {
+                            unsigned w = 0;
+#pragma unroll 1
+                            for (int q = 0; q < 4; ++q, src += p.lda) w |= (unsigned)(uint8_t)*src << (8 * q);
+                            fa[c] = (int)w;
+                        }
+                    } else {
+                        fa = *reinterpret_cast<const v4i *>(p.A + arow * (size_t)p.lda + k0);
+                    }
                     v4i fb;
                     if (BKN) {
                         const int8_t *src = p.B + (size_t)k0 * (size_t)p.ldb + bcol;
@@ -665,7 +707,7 @@ static int launch_transpose(const int8_t *in, int R, int C, int8_t *out, hipStre
     return (int)hipGetLastError();
 }
 
-template <int EPI, typename ST, int WGM, int WGN, int NSTAGE, int WGPC, int BKN>
+template <int EPI, typename ST, int WGM, int WGN, int NSTAGE, int WGPC, int BKN, int AKM = 0>
 static int launch_gemm_cfg(const GemmArgs &a, hipStream_t st)
 {
     constexpr int BM = QB * WBM * WGM, BN = QB * WBN * WGN, NT = 64 * WGM * WGN;
@@ -675,7 +717,7 @@ static int launch_gemm_cfg(const GemmArgs &a, hipStream_t st)
     GemmArgs p = a;
     p.tiles_m = (p.M + BM - 1) / BM;
     p.tiles_n = (p.N + BN - 1) / BN;
-    auto kern = igemm_nt_kernel<EPI, ST, WGM, WGN, NSTAGE, WGPC, BKN>;
+    auto kern = igemm_nt_kernel<EPI, ST, WGM, WGN, NSTAGE, WGPC, BKN, AKM>;
     // more than 64 KiB of dynamic LDS has to be opted into, per function
     hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void *>(kern), hipFuncAttributeMaxDynamicSharedMemorySize, SMEM);
     if (e != hipSuccess) return (int)e;
@@ -691,13 +733,21 @@ static int launch_gemm_cfg(const GemmArgs &a, hipStream_t st)
 #define JF_GEMM_CFG 0
 #endif
 constexpr bool KN_NATIVE = (JF_GEMM_CFG == 0);
-template <int EPI, typename ST> static int launch_gemm(const GemmArgs &a, hipStream_t st, bool b_kn)
+// a_km (A given as [K,M]) exists for the weight-gradient form only: fp output, B as [K,N].
+template <int EPI, typename ST> static int launch_gemm(const GemmArgs &a, hipStream_t st, bool b_kn, bool a_km = false)
 {
 #if JF_GEMM_CFG == 0
+    if (a_km) {
+        if constexpr (EPI == EPI_FP) {
+            if (b_kn) return launch_gemm_cfg<EPI, ST, 2, 4, 2, 2, 1, 1>(a, st);
+        }
+        return JF_ERR_UNSUPPORTED;
+    }
     return b_kn ? launch_gemm_cfg<EPI, ST, 2, 4, 2, 2, 1>(a, st) : launch_gemm_cfg<EPI, ST, 2, 4, 2, 2, 0>(a, st);
 #else
     // 256x128 or 128x256, whichever pads the problem less (1600 = 12.5 x 128 but 6.25 x 256); 16 waves, 3-deep ring
     (void)b_kn;
+    if (a_km) return JF_ERR_UNSUPPORTED;
     auto padded = [](long d, long t) { return (d + t - 1) / t * t; };
     const long tall = padded(a.M, 256) * padded(a.N, 128), wide = padded(a.M, 128) * padded(a.N, 256);
     return tall <= wide ? launch_gemm_cfg<EPI, ST, 4, 4, 3, 1, 0>(a, st) : launch_gemm_cfg<EPI, ST, 2, 8, 3, 1, 0>(a, st);
@@ -747,6 +797,7 @@ const char *jf_error_string(int code)
     case JF_ERR_ALIGN: return "jetfire_hip: pointer not 16-byte aligned";
     case JF_ERR_WORKSPACE: return "jetfire_hip: workspace missing or too small";
     case JF_ERR_DEVICE: return "jetfire_hip: device is not gfx950";
+    case JF_ERR_UNSUPPORTED: return "jetfire_hip: this combination of operand layouts is not implemented";
     default: return code > 0 ? hipGetErrorString((hipError_t)code) : "jetfire_hip: unknown error";
     }
 }
@@ -798,11 +849,12 @@ static bool scale_strides(int layout, int K, int blocks, int &ks, int &is)
 }
 
 int jf_igemm_block_fp(const int8_t *A, const int8_t *B, const void *sa, const void *sb, void *C,
-                      int M, int N, int K, int b_layout, int scale_dtype, int sa_layout, int sb_layout, int out_dtype,
-                      void *workspace, size_t workspace_bytes, jf_stream_t stream)
+                      int M, int N, int K, int a_layout, int b_layout, int scale_dtype, int sa_layout, int sb_layout,
+                      int out_dtype, void *workspace, size_t workspace_bytes, jf_stream_t stream)
 {
     int rc = check_gemm_common(A, B, C, M, N, K, b_layout, workspace, workspace_bytes);
     if (rc) return rc;
+    if (a_layout != JF_A_MK && a_layout != JF_A_KM) return JF_ERR_ENUM;
     if (!sa || !sb) return JF_ERR_NULL;
     if ((scale_dtype != JF_SCALE_F16 && scale_dtype != JF_SCALE_F32) ||
         (out_dtype != JF_FP_F16 && out_dtype != JF_FP_F32 && out_dtype != JF_FP_BF16)) return JF_ERR_ENUM;
@@ -811,11 +863,12 @@ int jf_igemm_block_fp(const int8_t *A, const int8_t *B, const void *sa, const vo
     const bool kn = prepare_b(B, ldb, N, K, b_layout, workspace, st, rc);
     if (rc) return rc;
     GemmArgs a = {};
-    a.A = A; a.B = B; a.sa = sa; a.sb = sb; a.C = C; a.M = M; a.N = N; a.K = K; a.lda = K; a.ldb = ldb;
+    const bool a_km = a_layout == JF_A_KM;
+    a.A = A; a.B = B; a.sa = sa; a.sb = sb; a.C = C; a.M = M; a.N = N; a.K = K; a.lda = a_km ? M : K; a.ldb = ldb;
     if (!scale_strides(sa_layout, K, M / QB, a.sa_ks, a.sa_is) || !scale_strides(sb_layout, K, N / QB, a.sb_ks, a.sb_is))
         return JF_ERR_ENUM;
     a.out_dtype = out_dtype;
-    return scale_dtype == JF_SCALE_F16 ? launch_gemm<EPI_FP, half_t>(a, st, kn) : launch_gemm<EPI_FP, float>(a, st, kn);
+    return scale_dtype == JF_SCALE_F16 ? launch_gemm<EPI_FP, half_t>(a, st, kn, a_km) : launch_gemm<EPI_FP, float>(a, st, kn, a_km);
 }
 
 int jf_igemm_block_q(const int8_t *A, const int8_t *B, const void *sa, const void *sb,

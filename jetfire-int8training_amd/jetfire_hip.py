@@ -17,6 +17,7 @@ LIB_PATH = os.path.join(_HERE, "libjetfire_hip.so")
 QB = 32
 
 B_NK, B_KN = 0, 1
+A_MK, A_KM = 0, 1
 SCALE_F16, SCALE_F32 = 0, 1
 SCALES_KMAJOR, SCALES_ROWMAJOR = 0, 1
 FP_F16, FP_F32, FP_BF16 = 0, 1, 2
@@ -46,7 +47,7 @@ def lib():
         L.jf_igemm_workspace_bytes.restype = _sz
         L.jf_igemm_s32.argtypes = [_p, _p, _p, _i, _i, _i, _i, _p, _sz, _p]
         L.jf_igemm_block_acc.argtypes = [_p, _p, _p, _i, _i, _i, _i, _p, _sz, _p]
-        L.jf_igemm_block_fp.argtypes = [_p, _p, _p, _p, _p, _i, _i, _i, _i, _i, _i, _i, _i, _p, _sz, _p]
+        L.jf_igemm_block_fp.argtypes = [_p, _p, _p, _p, _p, _i, _i, _i, _i, _i, _i, _i, _i, _i, _p, _sz, _p]
         L.jf_igemm_block_q.argtypes = [_p, _p, _p, _p, _p, _p, _p, _p, _i, _i, _i, _i, _i, _i, _i, _i, _u64, _u64, _p, _sz, _p]
         L.jf_quantize.argtypes = [_p, _i, _i, _i, _p, _p, _p, _i, _i, _u64, _u64, _f, _p]
         L.jf_dequantize.argtypes = [_p, _p, _i, _i, _i, _p, _p]
@@ -138,10 +139,15 @@ def _rng(rounding, numel, seed, offset):
 
 
 # ------------------------------------------------------------------------------------------------ GEMMs
-def _gemm_operands(A, B, b_layout):
+def _gemm_operands(A, B, b_layout, a_layout=0):
     _need(A, torch.int8, "A")
     _need(B, torch.int8, "B")
-    M, K = A.shape
+    if a_layout == A_MK:
+        M, K = A.shape
+    elif a_layout == A_KM:
+        K, M = A.shape
+    else:
+        raise RuntimeError("a_layout must be A_MK or A_KM")
     if b_layout == B_NK:
         N, K2 = B.shape
     elif b_layout == B_KN:
@@ -192,12 +198,13 @@ def igemm_block_acc(A, B, b_layout=B_KN):
     return out
 
 
-def igemm_block_fp(A, B, sa, sb, b_layout=B_KN, out_dtype=torch.float16):
-    M, N, K, ws, nb = _gemm_operands(A, B, b_layout)
+def igemm_block_fp(A, B, sa, sb, b_layout=B_KN, out_dtype=torch.float16, a_layout=A_MK):
+    """a_layout=A_KM: A is given as [K, M] (the un-transposed gradient of a weight-gradient GEMM)."""
+    M, N, K, ws, nb = _gemm_operands(A, B, b_layout, a_layout)
     code, la, lb = _gemm_scales(sa, sb, M, N, K)
     out = torch.empty((M, N), dtype=out_dtype, device=A.device)
-    check(lib().jf_igemm_block_fp(_ptr(A), _ptr(B), _ptr(sa), _ptr(sb), _ptr(out), M, N, K, b_layout, code, la, lb,
-                                  _FP_CODE[out_dtype], _ptr(ws), nb, _stream()))
+    check(lib().jf_igemm_block_fp(_ptr(A), _ptr(B), _ptr(sa), _ptr(sb), _ptr(out), M, N, K, a_layout, b_layout, code, la,
+                                  lb, _FP_CODE[out_dtype], _ptr(ws), nb, _stream()))
     return out
 
 

@@ -191,6 +191,14 @@ def test_linear_package_3d_shapes_and_values(oracle):
     assert eq(gw, wgw)
     gx, gw2 = int8_linear_backward(qx, sx, qg, sg, qgt, qw, sw, 32, stochastic=True, dgrad_quantize=False)
     assert gx.dtype == torch.float16 and tuple(gx.shape) == (BS, T, Cin) and torch.equal(gw2, gw)
+    # without a materialised transpose: G8T=None, or the .t() view of the gradient handed to the extension
+    _, gw3 = int8_linear_backward(qx, sx, qg, sg, None, qw, sw, 32, stochastic=True, dgrad_quantize=False)
+    gw4 = BQC.igemm_output_fp_no_quantize(qg.reshape(-1, Cout).t(), qx.reshape(-1, Cin), sg.reshape(-1, Cout // 32),
+                                          sx2, Cout, Cin, BS * T)
+    assert torch.equal(gw3, gw) and torch.equal(gw4, gw)
+    with pytest.raises(RuntimeError, match="contiguous or the .t\\(\\) view"):
+        BQC.igemm_output_fp_no_quantize(qgt[:, ::2], qx.reshape(-1, Cin)[: BS * T // 2], sg.reshape(-1, Cout // 32)[: BS * T // 64],
+                                        sx2[: BS * T // 64], Cout, Cin, BS * T // 2)
     ref_gx = g.reshape(-1, Cout).float() @ w
     assert torch.nn.functional.cosine_similarity(gx.reshape(-1).float(), ref_gx.reshape(-1), dim=0) > 0.99
     ref_gw = g.reshape(-1, Cout).float().t() @ x.reshape(-1, Cin)

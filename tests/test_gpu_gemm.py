@@ -171,6 +171,25 @@ def test_extreme_scale_products(jf, oracle, regime, layout):
     same(sc, wsc, f"{regime}: scales")
 
 
+@pytest.mark.parametrize("f16", [True, False])
+@pytest.mark.parametrize("M,N,K", SHAPES + [(160, 288, 1056)])
+def test_block_fp_a_given_as_km(jf, oracle, M, N, K, f16):
+    """Weight-gradient form with the A operand as it lies in memory ([K, M], e.g. the gradient [tokens, C_out]) and
+    B as [K, N]: the same bits as with a materialised transpose."""
+    print(f"case fp A_KM M={M} N={N} K={K} f16={f16}", flush=True)
+    A, Bkn, sa, sb = make_problem(M + 2 * N + K, M, N, K, f16)
+    st = np.float16 if f16 else np.float32
+    Akm = np.ascontiguousarray(A.T)
+    want32 = oracle.igemm_block_f32(A, Bkn, sa, sb, 1)
+    dsa, dsb = dev(sa.astype(st)), dev(sb.astype(st))
+    same(jf.igemm_block_fp(dev(Akm), dev(Bkn), dsa, dsb, jf.B_KN, torch.float32, a_layout=jf.A_KM), want32, "fp32 accumulators")
+    got16 = jf.igemm_block_fp(dev(Akm), dev(Bkn), dsa, dsb, jf.B_KN, torch.float16, a_layout=jf.A_KM)
+    with np.errstate(over="ignore"):
+        same(got16, want32.astype(np.float16), "fp16 output")
+    with pytest.raises(RuntimeError, match="not implemented"):
+        jf.igemm_block_fp(dev(Akm), dev(np.ascontiguousarray(Bkn.T)), dsa, dsb, jf.B_NK, torch.float32, a_layout=jf.A_KM)
+
+
 def test_block_q_bias(jf, oracle):
     """The forward kernel's bias / biasmax inputs (…BiasRowCol.cu:313,341,357)."""
     M, N, K = 128, 256, 96
