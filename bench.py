@@ -217,6 +217,7 @@ def main():
     ap.add_argument("--no-extras", action="store_true")
     ap.add_argument("--pmc-probe", action="store_true", help="copy kernel + 3 GEMM launches only (for rocprofv3 --pmc)")
     ap.add_argument("--roofline-only", action="store_true", help="only the dominant-kernel measurement (for rocprofv3 --stats)")
+    ap.add_argument("--extras-only", action="store_true", help="only the block-kernel section (for rocprofv3 --pmc)")
     a = ap.parse_args()
     if a.gpus != 1:
         sys.exit("bench.py: this build measures one GPU only (--gpus 1); nothing here uses a second GPU")
@@ -233,6 +234,9 @@ def main():
         return
     if a.roofline_only:
         print(json.dumps({"roofline": dominant_kernel_roofline(jf, torch, ops)}))
+        return
+    if a.extras_only:
+        print(json.dumps({"memory_bound_kernels": nonlinear_extras(jf, torch)}))
         return
 
     for i in range(a.warmup):
