@@ -90,6 +90,34 @@ def dominant_kernel_roofline(jf, torch, ops, iters=20):
             "traffic": MEASURED_TRAFFIC_BYTES}
 
 
+def deep_k_weight_gradients(jf, torch):
+    """Weight gradients of BASELINE config 2 (GPT-2 small, 12288 tokens) and the smallest one of the XL set: few output
+    tiles over a deep K.  One accumulation chain per output (the reference's arithmetic) against the library's K split
+    (ordered fp32 partial sums, `splitk=0`); both read the gradient [tokens, C_out] in place."""
+    out = {}
+    for name, T, cout, cin in (("gpt2small_qkv", 12288, 2304, 768), ("gpt2small_proj", 12288, 768, 768),
+                               ("gpt2small_fc", 12288, 3072, 768), ("gpt2small_fc2", 12288, 768, 3072),
+                               ("xl_proj", TOKENS, 1600, 1600)):
+        g = torch.randint(-127, 128, (T, cout), dtype=torch.int8, device="cuda")
+        x = torch.randint(-127, 128, (T, cin), dtype=torch.int8, device="cuda")
+        sg = torch.rand(T // 32, cout // 32, device="cuda") + 0.5
+        sx = torch.rand(T // 32, cin // 32, device="cuda") + 0.5
+        r = {"parts": jf.splitk_plan(cout, cin, T, 0)[0]}
+        for key, sk in (("one_chain", 1), ("split_k", 0)):
+            for _ in range(3):
+                jf.igemm_block_fp(g, x, sg, sx, jf.B_KN, torch.float16, a_layout=jf.A_KM, splitk=sk)
+            e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+            e0.record()
+            for _ in range(20):
+                jf.igemm_block_fp(g, x, sg, sx, jf.B_KN, torch.float16, a_layout=jf.A_KM, splitk=sk)
+            e1.record()
+            torch.cuda.synchronize()
+            us = e0.elapsed_time(e1) * 1e3 / 20
+            r[key] = {"us": round(us, 1), "TOP/s": round(2.0 * T * cout * cin / us / 1e6, 1)}
+        out[f"{name}_{cout}x{cin}x{T}"] = r
+    return out
+
+
 def nonlinear_extras(jf, torch):
     """Achieved GB/s (algorithmic bytes / event time) of the memory-bound kernels at the GPT-2 XL sizes of BASELINE
     config 4 (LayerNorm on 8192x1600, GELU on 8192x6400), fp32 scales."""
@@ -269,6 +297,7 @@ def main():
     if not a.no_extras:
         out["calibration"] = calibration(jf, torch)
         out["memory_bound_kernels"] = nonlinear_extras(jf, torch)
+        out["deep_k_weight_gradients"] = deep_k_weight_gradients(jf, torch)
     if not a.no_cpu:
         out["cpu_baseline"] = cpu_baseline(ops, a.cpu_rows)
     print(json.dumps(out))

@@ -88,10 +88,21 @@ int jf_igemm_block_acc(const int8_t *A, const int8_t *B, int32_t *acc, int M, in
 /* C_fp[M,N] = sum_kb sa*sb*(A_kb*B_kb), fp32 accumulate in ascending kb, stored as out_dtype.
  * Replaces igemm_output_fp_no_quantize (include/igemm.h:14-25, igemm/igemm_BlockSquare32OutputFp.cu:340-382).
  * With a_layout = JF_A_KM the weight gradient dW = dY^T X is computed from dY [tokens, C_out] as it lies in memory:
- * the reference's callers materialise dY^T first (Linear/linear_bwd.py:21, Nonlinear/transpose.py:69-97). */
+ * the reference's callers materialise dY^T first (Linear/linear_bwd.py:21, Nonlinear/transpose.py:69-97).
+ *
+ * splitk: 1 = one accumulation chain over all of K per output (the reference's arithmetic, bit for bit).
+ * n > 1 = K is cut into up to n parts of whole multiples of 4 K blocks (at least 16 K blocks each); every part is
+ * accumulated as above into an fp32 partial result, and the partial results are added in ascending order before the
+ * conversion to out_dtype: the result differs from splitk = 1 only in the rounding of those last additions.  For
+ * weight gradients with few output tiles and a deep K (GPT-2 small: 768 x 768 outputs over 12288 tokens = 36 tiles
+ * for 256 CUs; the reference runs the same under-filled grid, igemm_BlockSquare32OutputFp.cu:346-352) it fills the
+ * GPU.  0 = the library picks n from the tile count.  jf_igemm_splitk_plan reports the parts actually used (so a
+ * checker can reproduce the arithmetic), jf_igemm_block_fp_workspace_bytes the scratch needed (0 for one part). */
+int jf_igemm_splitk_plan(int M, int N, int K, int splitk, int *splits, int *kb_per_split);
+size_t jf_igemm_block_fp_workspace_bytes(int M, int N, int K, int b_layout, int splitk);
 int jf_igemm_block_fp(const int8_t *A, const int8_t *B, const void *sa, const void *sb, void *C,
                       int M, int N, int K, int a_layout, int b_layout, int scale_dtype, int sa_layout, int sb_layout,
-                      int out_dtype, void *workspace, size_t workspace_bytes, jf_stream_t stream);
+                      int out_dtype, int splitk, void *workspace, size_t workspace_bytes, jf_stream_t stream);
 
 /* (C_s8[M,N], sc[M/32,N/32]) = per-32x32-block requantisation of the same accumulation.
  *   rounding JF_ROUND_NEAREST : q = clamp(rn(127*(acc+bias[n]) / (amax+biasmax)), +-127)

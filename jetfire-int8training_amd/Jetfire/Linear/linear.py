@@ -70,12 +70,14 @@ def int8_linear_forward(X8_3D, SX16_3D, W8, SW16, output_quantized, B):
     return o8.reshape(*lead, n_out), so.reshape(*s_lead, SW16.shape[0])
 
 
-def int8_linear_backward(X8_3D, SX16_3D, G8_3D, SG16_3D, G8T, W8, SW16, B, stochastic=True, dgrad_quantize=True):
+def int8_linear_backward(X8_3D, SX16_3D, G8_3D, SG16_3D, G8T, W8, SW16, B, stochastic=True, dgrad_quantize=True,
+                         wgrad_splitk=1):
     """dX = dY W (requantised with stochastic rounding) and dW = dY^T X (fp16).
     G8 [BS,T,N] with SG [BS,T/32,N/32]; G8T = G8 transposed to [N, BS*T], or None (then G8 itself is read, no copy);
     W8 [N,K], SW [N/32,K/32].
     Returns (GX8, GSX, GW) or (GX_fp, GW) when dgrad_quantize=False (reference: linear_bwd.py:4-29; like
-    there, the activation gradient is always rounded stochastically)."""
+    there, the activation gradient is always rounded stochastically).  wgrad_splitk (not in the reference): 1 = its
+    arithmetic; 0 = let the library cut K into ordered partial sums when dW has too few tiles to fill the GPU."""
     _check_block(B)
     g2, sg2 = _flat2(G8_3D).contiguous(), _flat2(SG16_3D).contiguous()
     x2, sx2 = _flat2(X8_3D).contiguous(), _flat2(SX16_3D).contiguous()
@@ -84,7 +86,7 @@ def int8_linear_backward(X8_3D, SX16_3D, G8_3D, SG16_3D, G8T, W8, SW16, B, stoch
     gx8, gsx = BQC.igemm_output_int_quantize_stochastic(g2, W8, _k_major(sg2), SW16, tokens, c_in, c_out)
     if G8T is None:
         G8T = g2.t()                                               # a view: the extension reads g2 as the [K, M] operand
-    gw = BQC.igemm_output_fp_no_quantize(G8T, x2, sg2, sx2, G8T.shape[0], c_in, G8T.shape[1])
+    gw = BQC.igemm_output_fp_no_quantize(G8T, x2, sg2, sx2, G8T.shape[0], c_in, G8T.shape[1], wgrad_splitk)
     if not dgrad_quantize:
         return _dequant_like(gx8, gsx, tuple(G8_3D.shape[:-1])), gw
     return (gx8.reshape(*G8_3D.shape[:-1], c_in), gsx.reshape(*SG16_3D.shape[:-1], SW16.shape[1]), gw)

@@ -8,7 +8,8 @@ float8_e4m3fn (same bytes), exactly as the reference does (qmodel.py:131,153,230
 
 Two per-call costs of the reference are gone: weights are quantised once per weight version (WeightCodes below), and no
 transposed gradient is materialised for the weight-gradient GEMMs (the reference calls int8_transpose /
-int8_quantize_transpose before every one, qmodel.py:156,237,250; here the GEMM reads the gradient in place).
+int8_quantize_transpose before every one, qmodel.py:156,237,250; here the GEMM reads the gradient in place).  Weight
+gradients with too few output tiles to fill the GPU are computed with the library's K split (ordered fp32 partial sums).
 
 Linear biases are not part of the data flow (the reference ignores them as well); LayerNorm has a weight only.
 """
@@ -107,7 +108,7 @@ class AttentionIn(torch.autograd.Function):
     def backward(ctx, fpg, g):
         qx, sx, qn, sn, qw, sw, ln_w, mean, rstd = ctx.saved_tensors
         qg, sg = int8_quantize(g.contiguous(), QB, stochastic=True)
-        qg, sg, gw = int8_linear_backward(qn, sn, qg, sg, None, qw, sw, QB, stochastic=True)
+        qg, sg, gw = int8_linear_backward(qn, sn, qg, sg, None, qw, sw, QB, stochastic=True, wgrad_splitk=0)
         qg, sg, g_ln = int8_layernorm_backward(qx, sx, qg, sg, ln_w, QB, mean, rstd, stochastic=True)
         res_g, qg, sg = int8_add_Ifp_Ig16_Ofp_Og(fpg.contiguous(), qg, sg, QB, stochastic=True)
         return res_g, _as_f8(qg), sg, gw, g_ln, None, None
@@ -129,7 +130,7 @@ class AttentionOut(torch.autograd.Function):
     def backward(ctx, fpg, qg, sg, _m, _r):
         qy, sy, qw, sw = ctx.saved_tensors
         qg = _as_s8(qg)
-        g, gw = int8_linear_backward(qy, sy, qg, sg, None, qw, sw, QB, stochastic=True, dgrad_quantize=False)
+        g, gw = int8_linear_backward(qy, sy, qg, sg, None, qw, sw, QB, stochastic=True, dgrad_quantize=False, wgrad_splitk=0)
         return fpg, g, gw
 
 
@@ -153,9 +154,9 @@ class MLPResidual(torch.autograd.Function):
     def backward(ctx, fpg, qg, sg, _m, _r):
         qx, sx, qn, sn, qh, sh, qa, sa, qw1, sw1, qw2, sw2, ln_w, mean, rstd = ctx.saved_tensors
         qg = _as_s8(qg)
-        qg, sg, gw2 = int8_linear_backward(qa, sa, qg, sg, None, qw2, sw2, QB, stochastic=True)
+        qg, sg, gw2 = int8_linear_backward(qa, sa, qg, sg, None, qw2, sw2, QB, stochastic=True, wgrad_splitk=0)
         qg, sg = int8_gelu_backward(qh, sh, qg, sg, QB, stochastic=True)
-        qg, sg, gw1 = int8_linear_backward(qn, sn, qg, sg, None, qw1, sw1, QB, stochastic=True)
+        qg, sg, gw1 = int8_linear_backward(qn, sn, qg, sg, None, qw1, sw1, QB, stochastic=True, wgrad_splitk=0)
         qg, sg, g_ln = int8_layernorm_backward(qx, sx, qg, sg, ln_w, QB, mean, rstd, stochastic=True)
         res_g, qg, sg = int8_add_Ifp_Ig16_Ofp_Og(fpg.contiguous(), qg, sg, QB, stochastic=True)
         return res_g, _as_f8(qg), sg, gw1, gw2, g_ln, None, None

@@ -120,9 +120,10 @@ struct Workspace {
     torch::Tensor t;
     void *ptr = nullptr;
     size_t bytes = 0;
-    Workspace(const torch::Tensor &like, int M, int N, int K, int layout)
+    Workspace(const torch::Tensor &like, int M, int N, int K, int layout) : Workspace(like, jf_igemm_workspace_bytes(M, N, K, layout)) {}
+    Workspace(const torch::Tensor &like, size_t nbytes)
     {
-        bytes = jf_igemm_workspace_bytes(M, N, K, layout);
+        bytes = nbytes;
         if (bytes) {
             t = torch::empty({(int64_t)bytes}, like.options().dtype(torch::kInt8));
             ptr = t.data_ptr();
@@ -235,8 +236,9 @@ torch::Tensor igemm_basic_int8_gemm(torch::Tensor X, torch::Tensor W, const int 
 }
 
 // include/igemm.h:14-25 : fp16 output, B [K,N]
+// splitk (not in the reference's signature; default 1 = its arithmetic): see jf_igemm_block_fp.
 torch::Tensor igemm_output_fp_no_quantize(torch::Tensor X, torch::Tensor W, torch::Tensor SX, torch::Tensor SW,
-                                          const int M, const int N, const int K)
+                                          const int M, const int N, const int K, const int splitk)
 {
     check_dims(M, N, K);
     const int a_layout = check_a_any_layout(X, M, K);
@@ -245,10 +247,11 @@ torch::Tensor igemm_output_fp_no_quantize(torch::Tensor X, torch::Tensor W, torc
     const int code = check_scales(SX, SW, X, M, N, K, sxl, swl);
     c10::DeviceGuard guard(X.device());
     torch::Tensor O = torch::empty({M, N}, X.options().dtype(torch::kFloat16));
-    Workspace ws(X, M, N, K, JF_B_KN);
+    TORCH_CHECK(splitk >= 0, "splitk must be >= 0");
+    Workspace ws(X, jf_igemm_block_fp_workspace_bytes(M, N, K, JF_B_KN, splitk));
     pybind11::gil_scoped_release nogil;
     check_rc(jf_igemm_block_fp((const int8_t *)X.data_ptr(), (const int8_t *)W.data_ptr(), SX.data_ptr(), SW.data_ptr(),
-                               O.data_ptr(), M, N, K, a_layout, JF_B_KN, code, sxl, swl, JF_FP_F16, ws.ptr, ws.bytes,
+                               O.data_ptr(), M, N, K, a_layout, JF_B_KN, code, sxl, swl, JF_FP_F16, splitk, ws.ptr, ws.bytes,
                                current_stream(X)),
              "igemm_output_fp_no_quantize");
     return O;
@@ -321,7 +324,9 @@ PYBIND11_MODULE(TORCH_EXTENSION_NAME, m)
           "dequantize + INT8 MFMA GEMM + round-to-nearest requantize (fused); B is [K,N]");
     m.def("igemm_output_int_quantize_fused", &igemm_output_int_quantize_fused, "not implemented (unused in the reference)");
     m.def("igemm_output_fp_no_quantize", &igemm_output_fp_no_quantize,
-          "dequantize + INT8 MFMA GEMM, fp16 output; B is [K,N]; backward weight gradient");
+          "dequantize + INT8 MFMA GEMM, fp16 output; B is [K,N]; backward weight gradient", pybind11::arg("X"),
+          pybind11::arg("W"), pybind11::arg("SX"), pybind11::arg("SW"), pybind11::arg("M"), pybind11::arg("N"),
+          pybind11::arg("K"), pybind11::arg("splitk") = 1);
     m.def("igemm_basic_int8_gemm", &igemm_basic_int8_gemm, "INT8 MFMA GEMM, INT32 output; B is [K,N]");
     m.def("hgemm_v1", &hgemm_v1, "fp16 GEMM (library)");
     // not in the reference: makes the stochastic entry point reproducible from Python

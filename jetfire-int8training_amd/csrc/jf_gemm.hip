@@ -50,19 +50,23 @@ struct GemmArgs {
     uint64_t seed, offset;
     int M, N, K, lda, ldb;
     int tiles_m, tiles_n;
+    int splits, kb_per_split;   // split-K (EPI_FP only): workgroup w works on K blocks [s*kb_per_split, ...) of tile w % tiles,
+                                // s = w / tiles, and stores fp32 partial sums at C + s*M*N
     int out_dtype;        // JF_FP_*        (EPI_FP)
     int rounding;         // JF_ROUND_*     (EPI_Q)
 };
 
-// Logical tile of this workgroup.  Workgroups are dealt round-robin to the 8 XCDs, each with a
-// private L2: give every XCD one contiguous run of tiles, and walk tiles in groups of 8 tile-rows so
-// that concurrently resident workgroups of an XCD share A and B panels.
-__device__ __forceinline__ void tile_of_workgroup(int tiles_m, int tiles_n, int &tm, int &tn)
+// Logical tile (and K split) of this workgroup.  Workgroups are dealt round-robin to the 8 XCDs, each with a
+// private L2: give every XCD one contiguous run of the launch's work, and walk tiles in groups of 8 tile-rows so
+// that concurrently resident workgroups of an XCD share A and B panels.  With K splits the order is split-major.
+__device__ __forceinline__ void tile_of_workgroup(int tiles_m, int tiles_n, bool has_splits, int &tm, int &tn, int &split)
 {
     const int nwg = gridDim.x, wg = blockIdx.x;
     const int xcd = wg & 7, idx = wg >> 3;
     const int per = nwg >> 3, rem = nwg & 7;
-    const int logical = xcd * per + (xcd < rem ? xcd : rem) + idx;
+    int logical = xcd * per + (xcd < rem ? xcd : rem) + idx;
+    split = has_splits ? logical / (tiles_m * tiles_n) : 0;
+    logical -= split * (tiles_m * tiles_n);
     constexpr int GROUP = 8;
     const int group_size = GROUP * tiles_n;
     const int g = logical / group_size;
@@ -92,8 +96,9 @@ constexpr int WBM = 2, WBN = 1;
 // BKN = 0: B is [N, ldb] (K-contiguous rows, like A).  BKN = 1: B is [K, ldb] (N-contiguous rows); its tile is staged
 // as it lies in memory and the K-contiguous MFMA operand is produced by the transposing LDS read of gfx950.
 template <int EPI, typename ST, int WGM, int WGN, int NSTAGE, int WGPC, int BKN, int AKM = 0>
-__global__ __launch_bounds__(64 * WGM * WGN, WGPC * WGM * WGN / 4) void igemm_nt_kernel(GemmArgs p)
+__global__ __launch_bounds__(64 * WGM * WGN, WGPC * WGM * WGN / 4) void igemm_nt_kernel(GemmArgs p_in)
 {
+    GemmArgs p = p_in;                                        // K-split launches narrow it to the split's K range below
     constexpr int NW = WGM * WGN;
     constexpr int BM = QB * WBM * WGM, BN = QB * WBN * WGN;
     constexpr int A_BYTES = BM * ROW_BYTES;                  // one stage of A
@@ -113,8 +118,18 @@ __global__ __launch_bounds__(64 * WGM * WGN, WGPC * WGM * WGN / 4) void igemm_nt
     const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
     const int wm = wave % WGM, wn = wave / WGM;
 
-    int tile_m, tile_n;
-    tile_of_workgroup(p.tiles_m, p.tiles_n, tile_m, tile_n);
+    int tile_m, tile_n, split;
+    tile_of_workgroup(p.tiles_m, p.tiles_n, EPI == EPI_FP && p.splits > 1, tile_m, tile_n, split);
+    int kb_base = 0;                                          // first K block of this workgroup (scale indices count from 0)
+    if (EPI == EPI_FP && p.splits > 1) {                      // uniform: the same problem on a K range, fp32 partial output
+        kb_base = split * p.kb_per_split;
+        const int kbn = (p.K / QB - kb_base) < p.kb_per_split ? (p.K / QB - kb_base) : p.kb_per_split;
+        p.A += AKM ? (size_t)kb_base * QB * (size_t)p.lda : (size_t)kb_base * QB;
+        p.B += BKN ? (size_t)kb_base * QB * (size_t)p.ldb : (size_t)kb_base * QB;
+        p.K = kbn * QB;
+        p.C = reinterpret_cast<float *>(p.C) + (size_t)split * (size_t)p.M * (size_t)p.N;
+        p.out_dtype = JF_FP_F32;
+    }
     const int m0 = tile_m * BM, n0 = tile_n * BN;
     const int SM = p.M / QB, SN = p.N / QB;
     const int nkb = p.K / QB;
@@ -175,7 +190,7 @@ __global__ __launch_bounds__(64 * WGM * WGN, WGPC * WGM * WGN / 4) void igemm_nt
     const int s_ks = s_is_a ? p.sa_ks : p.sb_ks, s_is = s_is_a ? p.sa_is : p.sb_is;   // element strides: K block, tile block
     const unsigned char *const s_base = reinterpret_cast<const unsigned char *>(s_is_a ? p.sa : p.sb);
     auto scale_addr = [&](int kbg) {
-        const unsigned e = (unsigned)(kbg * s_ks + s_idx * s_is);
+        const unsigned e = (unsigned)((kbg + kb_base) * s_ks + s_idx * s_is);
         return s_base + (sizeof(ST) == 4 ? e * 4u : (e >> 1) * 4u);
     };
     const unsigned char *s_ptr = scale_addr((lane >> 4) < nkb ? (lane >> 4) : nkb - 1);
@@ -281,6 +296,13 @@ __global__ __launch_bounds__(64 * WGM * WGN, WGPC * WGM * WGN / 4) void igemm_nt
     for (int i = 0; i < WBM; ++i) { mb[i] = m0 / QB + wm * WBM + i; mb[i] = mb[i] < SM ? mb[i] : SM - 1; }
 #pragma unroll
     for (int j = 0; j < WBN; ++j) { nb[j] = n0 / QB + wn * WBN + j; nb[j] = nb[j] < SN ? nb[j] : SN - 1; }
+
+    // element index of a scale = K block * K stride + these (only its parity matters, for binary16 scales)
+    int par_a[WBM], par_b[WBN];
+#pragma unroll
+    for (int i = 0; i < WBM; ++i) par_a[i] = __builtin_amdgcn_readfirstlane((kb_base * p.sa_ks + mb[i] * p.sa_is) & 1);
+#pragma unroll
+    for (int j = 0; j < WBN; ++j) par_b[j] = __builtin_amdgcn_readfirstlane((kb_base * p.sb_ks + nb[j] * p.sb_is) & 1);
 
     // ---- main loop ----------------------------------------------------------------------------
     // The whole ring is filled up front; afterwards the loads of stage s+NSTAGE are issued when the last K block
@@ -396,9 +418,9 @@ __global__ __launch_bounds__(64 * WGM * WGN, WGPC * WGM * WGN / 4) void igemm_nt
                 return (float)__builtin_bit_cast(half_t, h);
             };
 #pragma unroll
-            for (int i = 0; i < WBM; ++i) fa[i] = scale_of(sc_raw[CUR][i], kbg * p.sa_ks + mb[i] * p.sa_is);
+            for (int i = 0; i < WBM; ++i) fa[i] = scale_of(sc_raw[CUR][i], kbg * p.sa_ks + par_a[i]);
 #pragma unroll
-            for (int j = 0; j < WBN; ++j) fb[j] = scale_of(sc_raw[CUR][WBM + j], kbg * p.sb_ks + nb[j] * p.sb_is);
+            for (int j = 0; j < WBN; ++j) fb[j] = scale_of(sc_raw[CUR][WBM + j], kbg * p.sb_ks + par_b[j]);
             static_for<0, NBLK>([&](auto n_c) {
                 constexpr int n = decltype(n_c)::value, i = n / WBN, j = n % WBN;
                 // asm: as a builtin operand the constant is hoisted into 16 registers instead of being encoded inline.
@@ -536,7 +558,7 @@ __global__ __launch_bounds__(64 * WGM * WGN, WGPC * WGM * WGN / 4) void igemm_nt
                     }
                     const v16i z = {0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0};
                     const v16i d = __builtin_amdgcn_mfma_i32_32x32x32_i8(fa, fb, z, 0, 0, 0);
-                    const float sab = (float)sa_t[kb * p.sa_ks + mb[i] * p.sa_is] * (float)sb_t[kb * p.sb_ks + nb[j] * p.sb_is];
+                    const float sab = (float)sa_t[(kb + kb_base) * p.sa_ks + mb[i] * p.sa_is] * (float)sb_t[(kb + kb_base) * p.sb_ks + nb[j] * p.sb_is];
 #pragma unroll
                     for (int v = 0; v < 16; ++v) r[v] = __builtin_fmaf(sab, (float)d[v], r[v]);
                 }
@@ -721,8 +743,59 @@ static int launch_gemm_cfg(const GemmArgs &a, hipStream_t st)
     // more than 64 KiB of dynamic LDS has to be opted into, per function
     hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void *>(kern), hipFuncAttributeMaxDynamicSharedMemorySize, SMEM);
     if (e != hipSuccess) return (int)e;
-    hipLaunchKernelGGL(kern, dim3(p.tiles_m * p.tiles_n), dim3(NT), SMEM, st, p);
+    if (EPI != EPI_FP || p.splits < 1) p.splits = 1;
+    hipLaunchKernelGGL(kern, dim3(p.tiles_m * p.tiles_n * p.splits), dim3(NT), SMEM, st, p);
     return (int)hipGetLastError();
+}
+
+// out[i] = convert(part[0][i] + part[1][i] + ... + part[S-1][i]), added in ascending split order.
+__global__ __launch_bounds__(256) void splitk_reduce_kernel(const float *part, size_t n, int splits, void *out, int out_dtype)
+{
+    const size_t i = ((size_t)blockIdx.x * 256 + threadIdx.x) * 4;
+    if (i >= n) return;                                        // n is a multiple of 1024
+    v4f t = *reinterpret_cast<const v4f *>(part + i);
+    for (int s = 1; s < splits; ++s) {
+        const v4f u = *reinterpret_cast<const v4f *>(part + (size_t)s * n + i);
+        t.x = t.x + u.x; t.y = t.y + u.y; t.z = t.z + u.z; t.w = t.w + u.w;
+    }
+    if (out_dtype == JF_FP_F32) {
+        *reinterpret_cast<v4f *>(reinterpret_cast<float *>(out) + i) = t;
+    } else if (out_dtype == JF_FP_F16) {
+        half_t h[4] = {(half_t)t.x, (half_t)t.y, (half_t)t.z, (half_t)t.w};
+        *reinterpret_cast<v2i *>(reinterpret_cast<half_t *>(out) + i) = *reinterpret_cast<v2i *>(h);
+    } else {
+        __bf16 h[4] = {(__bf16)t.x, (__bf16)t.y, (__bf16)t.z, (__bf16)t.w};
+        *reinterpret_cast<v2i *>(reinterpret_cast<__bf16 *>(out) + i) = *reinterpret_cast<v2i *>(h);
+    }
+}
+
+static int cu_count()
+{
+    static const int n = [] {
+        int dev = 0, cus = 0;
+        if (hipGetDevice(&dev) != hipSuccess || hipDeviceGetAttribute(&cus, hipDeviceAttributeMultiprocessorCount, dev) != hipSuccess || cus <= 0)
+            cus = 256;
+        return cus;
+    }();
+    return n;
+}
+
+// K split of the fp-output GEMM.  request 1: none; request > 1: that many parts (fewer if K is short); request 0: as
+// many parts as it takes to give every CU two workgroups, when the tiles alone fill less than half of them.  Parts are
+// whole multiples of 4 K blocks (one LDS stage), at least 16 K blocks long.
+static void splitk_plan(int M, int N, int K, int request, int &splits, int &kb_per_split)
+{
+    const int nkb = K / QB;
+    int want = request;
+    if (request == 0) {
+        const int tiles = ((M + 127) / 128) * ((N + 127) / 128), slots = 2 * cu_count();
+        want = 2 * tiles <= slots ? slots / tiles : 1;
+        if (want > 16) want = 16;
+    }
+    if (want > nkb / 16) want = nkb / 16;
+    if (want < 1) want = 1;
+    kb_per_split = ((nkb + want - 1) / want + 3) / 4 * 4;
+    splits = (nkb + kb_per_split - 1) / kb_per_split;
 }
 
 // Tile configuration.  JF_GEMM_CFG selects it at build time (for experiments); the default is 128x128 tiles,
@@ -848,13 +921,33 @@ static bool scale_strides(int layout, int K, int blocks, int &ks, int &is)
     return false;
 }
 
+int jf_igemm_splitk_plan(int M, int N, int K, int splitk, int *splits, int *kb_per_split)
+{
+    if (!mult32(M) || !mult32(N) || !mult32(K)) return JF_ERR_SHAPE;
+    if (splitk < 0 || !splits || !kb_per_split) return splitk < 0 ? JF_ERR_ENUM : JF_ERR_NULL;
+    if (KN_NATIVE) splitk_plan(M, N, K, splitk, *splits, *kb_per_split);
+    else { *splits = 1; *kb_per_split = (K / QB + 3) / 4 * 4; }
+    return JF_OK;
+}
+
+size_t jf_igemm_block_fp_workspace_bytes(int M, int N, int K, int b_layout, int splitk)
+{
+    int splits = 1, kb_per = 0;
+    if (jf_igemm_splitk_plan(M, N, K, splitk, &splits, &kb_per) != JF_OK) return 0;
+    return jf_igemm_workspace_bytes(M, N, K, b_layout) + (splits > 1 ? (size_t)splits * (size_t)M * (size_t)N * sizeof(float) : 0);
+}
+
 int jf_igemm_block_fp(const int8_t *A, const int8_t *B, const void *sa, const void *sb, void *C,
                       int M, int N, int K, int a_layout, int b_layout, int scale_dtype, int sa_layout, int sb_layout,
-                      int out_dtype, void *workspace, size_t workspace_bytes, jf_stream_t stream)
+                      int out_dtype, int splitk, void *workspace, size_t workspace_bytes, jf_stream_t stream)
 {
     int rc = check_gemm_common(A, B, C, M, N, K, b_layout, workspace, workspace_bytes);
     if (rc) return rc;
     if (a_layout != JF_A_MK && a_layout != JF_A_KM) return JF_ERR_ENUM;
+    int splits = 1, kb_per = 0;
+    if ((rc = jf_igemm_splitk_plan(M, N, K, splitk, &splits, &kb_per))) return rc;
+    if (splits > 1 && (!workspace || !aligned16(workspace) || workspace_bytes < jf_igemm_block_fp_workspace_bytes(M, N, K, b_layout, splitk)))
+        return JF_ERR_WORKSPACE;
     if (!sa || !sb) return JF_ERR_NULL;
     if ((scale_dtype != JF_SCALE_F16 && scale_dtype != JF_SCALE_F32) ||
         (out_dtype != JF_FP_F16 && out_dtype != JF_FP_F32 && out_dtype != JF_FP_BF16)) return JF_ERR_ENUM;
@@ -868,7 +961,13 @@ int jf_igemm_block_fp(const int8_t *A, const int8_t *B, const void *sa, const vo
     if (!scale_strides(sa_layout, K, M / QB, a.sa_ks, a.sa_is) || !scale_strides(sb_layout, K, N / QB, a.sb_ks, a.sb_is))
         return JF_ERR_ENUM;
     a.out_dtype = out_dtype;
-    return scale_dtype == JF_SCALE_F16 ? launch_gemm<EPI_FP, half_t>(a, st, kn, a_km) : launch_gemm<EPI_FP, float>(a, st, kn, a_km);
+    a.splits = splits; a.kb_per_split = kb_per;
+    if (splits > 1) a.C = workspace;                          // fp32 partial sums [splits][M][N]
+    rc = scale_dtype == JF_SCALE_F16 ? launch_gemm<EPI_FP, half_t>(a, st, kn, a_km) : launch_gemm<EPI_FP, float>(a, st, kn, a_km);
+    if (rc || splits == 1) return rc;
+    const size_t n = (size_t)M * (size_t)N;
+    hipLaunchKernelGGL(splitk_reduce_kernel, dim3((unsigned)(n / 1024)), dim3(256), 0, st, (const float *)workspace, n, splits, C, out_dtype);
+    return (int)hipGetLastError();
 }
 
 int jf_igemm_block_q(const int8_t *A, const int8_t *B, const void *sa, const void *sb,

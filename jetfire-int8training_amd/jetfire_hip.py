@@ -26,6 +26,7 @@ GELU_ERF, GELU_TANH = 0, 1
 
 EXPORTS = [
     "jf_error_string", "jf_igemm_workspace_bytes", "jf_igemm_s32", "jf_igemm_block_acc", "jf_igemm_block_fp",
+    "jf_igemm_splitk_plan", "jf_igemm_block_fp_workspace_bytes",
     "jf_igemm_block_q", "jf_quantize", "jf_dequantize", "jf_transpose_s8", "jf_rowstats", "jf_layernorm_fwd",
     "jf_layernorm_bwd_workspace_bytes", "jf_layernorm_bwd", "jf_gelu_fwd", "jf_gelu_bwd", "jf_add", "jf_calibrate",
 ]
@@ -47,7 +48,10 @@ def lib():
         L.jf_igemm_workspace_bytes.restype = _sz
         L.jf_igemm_s32.argtypes = [_p, _p, _p, _i, _i, _i, _i, _p, _sz, _p]
         L.jf_igemm_block_acc.argtypes = [_p, _p, _p, _i, _i, _i, _i, _p, _sz, _p]
-        L.jf_igemm_block_fp.argtypes = [_p, _p, _p, _p, _p, _i, _i, _i, _i, _i, _i, _i, _i, _i, _p, _sz, _p]
+        L.jf_igemm_block_fp.argtypes = [_p, _p, _p, _p, _p, _i, _i, _i, _i, _i, _i, _i, _i, _i, _i, _p, _sz, _p]
+        L.jf_igemm_splitk_plan.argtypes = [_i, _i, _i, _i, C.POINTER(C.c_int), C.POINTER(C.c_int)]
+        L.jf_igemm_block_fp_workspace_bytes.argtypes = [_i, _i, _i, _i, _i]
+        L.jf_igemm_block_fp_workspace_bytes.restype = _sz
         L.jf_igemm_block_q.argtypes = [_p, _p, _p, _p, _p, _p, _p, _p, _i, _i, _i, _i, _i, _i, _i, _i, _u64, _u64, _p, _sz, _p]
         L.jf_quantize.argtypes = [_p, _i, _i, _i, _p, _p, _p, _i, _i, _u64, _u64, _f, _p]
         L.jf_dequantize.argtypes = [_p, _p, _i, _i, _i, _p, _p]
@@ -198,13 +202,24 @@ def igemm_block_acc(A, B, b_layout=B_KN):
     return out
 
 
-def igemm_block_fp(A, B, sa, sb, b_layout=B_KN, out_dtype=torch.float16, a_layout=A_MK):
-    """a_layout=A_KM: A is given as [K, M] (the un-transposed gradient of a weight-gradient GEMM)."""
+def splitk_plan(M, N, K, splitk):
+    """(parts, K blocks per part) the library uses for this problem and splitk request."""
+    parts, per = C.c_int(0), C.c_int(0)
+    check(lib().jf_igemm_splitk_plan(M, N, K, splitk, C.byref(parts), C.byref(per)))
+    return parts.value, per.value
+
+
+def igemm_block_fp(A, B, sa, sb, b_layout=B_KN, out_dtype=torch.float16, a_layout=A_MK, splitk=1):
+    """a_layout=A_KM: A is given as [K, M] (the un-transposed gradient of a weight-gradient GEMM).
+    splitk: 1 = one accumulation chain over K (reference arithmetic); n > 1 = up to n ordered partial chains;
+    0 = chosen by the library from the tile count."""
     M, N, K, ws, nb = _gemm_operands(A, B, b_layout, a_layout)
+    nb = lib().jf_igemm_block_fp_workspace_bytes(M, N, K, b_layout, splitk)
+    ws = torch.empty(nb, dtype=torch.int8, device=A.device) if nb else None
     code, la, lb = _gemm_scales(sa, sb, M, N, K)
     out = torch.empty((M, N), dtype=out_dtype, device=A.device)
     check(lib().jf_igemm_block_fp(_ptr(A), _ptr(B), _ptr(sa), _ptr(sb), _ptr(out), M, N, K, a_layout, b_layout, code, la,
-                                  lb, _FP_CODE[out_dtype], _ptr(ws), nb, _stream()))
+                                  lb, _FP_CODE[out_dtype], splitk, _ptr(ws), nb, _stream()))
     return out
 
 

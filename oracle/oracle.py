@@ -193,6 +193,25 @@ def igemm_block_f32(A, B, sa, sb, b_layout, fused=True):
     return out
 
 
+def igemm_block_f32_splitk(A, B, sa, sb, b_layout, parts, kb_per_part):
+    """The K-split variant of the fp-output GEMM (an addition of this library's C ABI, no counterpart in the reference):
+    part p accumulates K blocks [p*kb_per_part, (p+1)*kb_per_part) exactly as igemm_block_f32 does, and the partial
+    results are added in ascending order in fp32.  Pinned by construction: igemm_block_f32 on K slices + IEEE adds."""
+    A = _c(A, np.int8)
+    B = _c(B, np.int8)
+    sa = _c(sa, np.float32)
+    sb = _c(sb, np.float32)
+    M, N, K = _gemm_dims(A, B, b_layout)
+    out = None
+    for p in range(parts):
+        kb0, kb1 = p * kb_per_part, min((p + 1) * kb_per_part, K // QB)
+        ks = slice(kb0 * QB, kb1 * QB)
+        Bp = B[ks, :] if b_layout == 1 else B[:, ks]
+        part = igemm_block_f32(np.ascontiguousarray(A[:, ks]), np.ascontiguousarray(Bp), sa[kb0:kb1], sb[kb0:kb1], b_layout)
+        out = part if out is None else (out + part).astype(np.float32)
+    return out
+
+
 def requant(acc, bias=None, biasmax=0.0, stochastic=False, seed=0, offset=0, scale_dtype="f32"):
     acc = _c(acc, np.float32)
     M, N = acc.shape

@@ -190,6 +190,35 @@ def test_block_fp_a_given_as_km(jf, oracle, M, N, K, f16):
         jf.igemm_block_fp(dev(Akm), dev(np.ascontiguousarray(Bkn.T)), dsa, dsb, jf.B_NK, torch.float32, a_layout=jf.A_KM)
 
 
+@pytest.mark.parametrize("a_km", [False, True])
+@pytest.mark.parametrize("M,N,K,req", [(128, 256, 2048, 2), (160, 96, 3104, 4), (96, 160, 2560, 0), (64, 64, 12288, 0),
+                                           (128, 128, 512, 3), (32, 32, 992, 2), (256, 384, 544, 0)])
+def test_block_fp_split_k(jf, oracle, M, N, K, req, a_km):
+    """K cut into ordered partial chains: bit-exact against the oracle's composition with the same plan; request 1
+    stays the reference arithmetic; the two differ by fp32 rounding only."""
+    print(f"case fp splitk M={M} N={N} K={K} request={req} a_km={a_km}", flush=True)
+    A, Bkn, sa, sb = make_problem(M + N + K + req, M, N, K, f16=False)
+    parts, per = jf.splitk_plan(M, N, K, req)
+    assert parts >= 1 and per % 4 == 0 and (parts - 1) * per < K // QB <= parts * per
+    if req == 0:
+        assert parts > 1 or K // QB < 32 or 2 * ((M + 127) // 128) * ((N + 127) // 128) > 512
+    dA = dev(np.ascontiguousarray(A.T)) if a_km else dev(A)
+    kw = dict(a_layout=jf.A_KM if a_km else jf.A_MK)
+    dsa, dsb = dev(sa), dev(sb)
+    want = oracle.igemm_block_f32_splitk(A, Bkn, sa, sb, 1, parts, per)
+    one = oracle.igemm_block_f32(A, Bkn, sa, sb, 1)
+    got = jf.igemm_block_fp(dA, dev(Bkn), dsa, dsb, jf.B_KN, torch.float32, splitk=req, **kw)
+    same(got, want, f"fp32, {parts} parts of {per} K blocks")
+    same(jf.igemm_block_fp(dA, dev(Bkn), dsa, dsb, jf.B_KN, torch.float32, splitk=1, **kw), one, "one chain")
+    np.testing.assert_allclose(want, one, rtol=1e-5, atol=1e-5 * np.abs(one).max())
+    got16 = jf.igemm_block_fp(dA, dev(Bkn), dsa, dsb, jf.B_KN, torch.float16, splitk=req, **kw)
+    with np.errstate(over="ignore"):
+        same(got16, want.astype(np.float16), "fp16 output")
+    if not a_km:                                                  # B as [N,K] takes the same path
+        same(jf.igemm_block_fp(dA, dev(np.ascontiguousarray(Bkn.T)), dsa, dsb, jf.B_NK, torch.float32, splitk=req),
+             oracle.igemm_block_f32_splitk(A, np.ascontiguousarray(Bkn.T), sa, sb, 0, parts, per), "B as [N,K]")
+
+
 def test_block_q_bias(jf, oracle):
     """The forward kernel's bias / biasmax inputs (…BiasRowCol.cu:313,341,357)."""
     M, N, K = 128, 256, 96
