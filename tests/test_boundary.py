@@ -206,6 +206,40 @@ def test_linear_package_3d_shapes_and_values(oracle):
 
 
 @pytest.mark.gpu
+def test_weight_gradient_k_split_through_the_packages(oracle):
+    """The K split of the weight gradient (an extension: trailing argument / keyword, default = the reference's single
+    chain) through BlockQuantizeCUDA and Linear: bit-exact against the oracle's composition with the library's plan."""
+    from Linear import int8_linear_backward
+    from Nonlinear import int8_quantize
+    import BlockQuantizeCUDA as BQC
+    import jetfire_hip as jf
+    torch.manual_seed(11)
+    BS, T, Cin, Cout = 2, 1024, 96, 160
+    x = torch.randn(BS, T, Cin, device="cuda")
+    w = torch.randn(Cout, Cin, device="cuda") * 0.02
+    g = torch.randn(BS, T, Cout, device="cuda", dtype=torch.float16) * 1e-3
+    qx, sx = int8_quantize(x, 32)
+    qw, sw = int8_quantize(w, 32)
+    qg, sg = int8_quantize(g, 32, stochastic=True)
+    K = BS * T
+    A = np.ascontiguousarray(qg.reshape(K, Cout).cpu().numpy().T)
+    X = qx.reshape(K, Cin).cpu().numpy()
+    SG, SX = sg.reshape(-1, Cout // 32).float().cpu().numpy(), sx.reshape(-1, Cin // 32).float().cpu().numpy()
+    for req in (2, 0):
+        parts, per = jf.splitk_plan(Cout, Cin, K, req)
+        assert parts > 1
+        want = oracle.igemm_block_f32_splitk(A, X, SG, SX, 1, parts, per).astype(np.float16)
+        got = BQC.igemm_output_fp_no_quantize(qg.reshape(K, Cout).t(), qx.reshape(K, Cin), sg.reshape(-1, Cout // 32),
+                                              sx.reshape(-1, Cin // 32), Cout, Cin, K, req)
+        assert eq(got, want)
+    _, _, gw0 = int8_linear_backward(qx, sx, qg, sg, None, qw, sw, 32, wgrad_splitk=0)
+    assert eq(gw0, want)
+    _, _, gw1 = int8_linear_backward(qx, sx, qg, sg, None, qw, sw, 32)
+    assert eq(gw1, oracle.igemm_block_fp(A, X, SG, SX, 1, "f16"))
+    assert torch.allclose(gw0.float(), gw1.float(), rtol=2e-3, atol=1e-7)
+
+
+@pytest.mark.gpu
 def test_nonlinear_package_3d(oracle):
     from Nonlinear import (int8_add_Ifp_Ig16_Ofp_Og, int8_add_Ifp_Ig16_Ofp_Og_MeanVar, int8_dequantize,
                            int8_gelu_backward, int8_gelu_forward, int8_layernorm_backward, int8_layernorm_forward,
