@@ -565,6 +565,7 @@ using namespace jf;
 
 #define JF_LAUNCH(kern, grid, smem, st, ...)                         \
     do {                                                             \
+        if (!device_is_gfx950()) return JF_ERR_DEVICE;               \
         hipLaunchKernelGGL(kern, dim3(grid), dim3(NT), smem, st, __VA_ARGS__); \
         return (int)hipGetLastError();                               \
     } while (0)
@@ -659,6 +660,7 @@ int jf_layernorm_bwd(const int8_t *qx, const void *sx, const int8_t *qg, const v
     // LDS: two [32][C/16] partial-sum arrays, c1/c2, one column-sum patch per wave
     const size_t smem = ((size_t)2 * QB * (C / 16) + 2 * QB + (LNB_THREADS / WAVE) * COLSUM_PATCH) * sizeof(float);
     if (smem > 160 * 1024 - 512) return JF_ERR_SHAPE;          // rows of up to ~5700 columns
+    if (!device_is_gfx950()) return JF_ERR_DEVICE;
     hipStream_t st = (hipStream_t)stream;
     const bool want_dw = dgamma || dbeta;
     // workspace: [2R floats, unused by this implementation][strips x C partial dgamma][strips x C partial dbeta]

@@ -318,6 +318,24 @@ template <int APPROX> __device__ __forceinline__ void dgelu_pair(float x, float 
 
 // ---------------------------------------------------------------------------------------------
 // host-side argument checks shared by the entry points
+// The kernels exist as gfx950 code objects only: say so instead of failing at launch with "no binary for GPU".
+// (One property query per device and process; afterwards a table look-up.)
+static inline bool device_is_gfx950()
+{
+    static signed char known[64] = {};           // 0: not asked yet, 1: gfx950, -1: something else
+    int dev = 0;
+    if (hipGetDevice(&dev) != hipSuccess || dev < 0 || dev >= 64) return false;
+    if (known[dev] == 0) {
+        hipDeviceProp_t prop;
+        bool ok = hipGetDeviceProperties(&prop, dev) == hipSuccess;
+        if (ok) {
+            const char *a = prop.gcnArchName;
+            ok = a[0] == 'g' && a[1] == 'f' && a[2] == 'x' && a[3] == '9' && a[4] == '5' && a[5] == '0' && (a[6] == 0 || a[6] == ':');
+        }
+        known[dev] = ok ? 1 : -1;
+    }
+    return known[dev] == 1;
+}
 static inline bool mult32(int v) { return v > 0 && (v % QB) == 0; }
 static inline bool aligned16(const void *p) { return (reinterpret_cast<uintptr_t>(p) & 15u) == 0; }
 

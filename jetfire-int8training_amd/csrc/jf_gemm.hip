@@ -736,6 +736,7 @@ static int launch_gemm_cfg(const GemmArgs &a, hipStream_t st)
     constexpr int RING = NSTAGE * (BM + BN) * ROW_BYTES + WGM * WGN * NSTAGE * 256;   // operand ring + per-wave scale patches
     constexpr int PATCH = WGM * WGN * QB * EPI_LD * (int)sizeof(float) + (EPI == EPI_S32 ? 0 : BM * BN * (EPI == EPI_Q ? 1 : 2));   // + tile image
     constexpr int SMEM = RING > PATCH ? RING : PATCH;
+    if (!device_is_gfx950()) return JF_ERR_DEVICE;
     GemmArgs p = a;
     p.tiles_m = (p.M + BM - 1) / BM;
     p.tiles_n = (p.N + BN - 1) / BN;
@@ -998,6 +999,7 @@ int jf_transpose_s8(const int8_t *in, int R, int C, int8_t *out, jf_stream_t str
     if (!in || !out) return JF_ERR_NULL;
     if (R <= 0 || C <= 0 || (R % 16) || (C % 16)) return JF_ERR_SHAPE;
     if (!aligned16(in) || !aligned16(out)) return JF_ERR_ALIGN;
+    if (!device_is_gfx950()) return JF_ERR_DEVICE;
     return launch_transpose(in, R, C, out, (hipStream_t)stream);
 }
 

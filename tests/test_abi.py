@@ -38,4 +38,10 @@ def test_argument_errors_without_gpu(jf):
     assert L.jf_igemm_s32(p, p, p, 32, 32, 32, 7, None, 0, None) == -3          # unknown layout
     assert L.jf_igemm_s32(p + 1, p, p, 32, 32, 32, 0, None, 0, None) == -4      # misaligned
     assert L.jf_quantize(p, 9, 32, 32, p, p, None, 0, 0, 0, 0, 0.0, None) == -3
+    import torch
+    if not torch.cuda.is_available():
+        # valid arguments, but no gfx950 device to run on: refused by name, nothing is launched
+        assert L.jf_igemm_s32(p, p, p, 32, 32, 32, 0, None, 0, None) == -6
+        assert L.jf_quantize(p, 1, 32, 32, p, p, None, 0, 0, 0, 0, 0.0, None) == -6
+        assert b"gfx950" in L.jf_error_string(-6)
     assert L.jf_gelu_fwd(p, p, 32, 32, 0, 5, 0.0, p, p, None) == -3
