@@ -219,6 +219,43 @@ def test_block_fp_split_k(jf, oracle, M, N, K, req, a_km):
              oracle.igemm_block_f32_splitk(A, np.ascontiguousarray(Bkn.T), sa, sb, 0, parts, per), "B as [N,K]")
 
 
+def _random_cases(n, seed):
+    rng = np.random.default_rng(seed)
+    for _ in range(n):
+        yield (int(rng.integers(1, 13)) * 32, int(rng.integers(1, 13)) * 32, int(rng.integers(1, 41)) * 32,
+               int(rng.integers(0, 2)), bool(rng.integers(0, 2)), int(rng.integers(0, 4)), int(rng.integers(0, 1 << 30)))
+
+
+@pytest.mark.parametrize("M,N,K,layout,f16,scale_views,seed", list(_random_cases(32, 2024)))
+def test_random_shapes(jf, oracle, M, N, K, layout, f16, scale_views, seed):
+    """Random small problems (M, N up to 384, K up to 1280, all multiples of 32): every output kind, both B layouts, both
+    scale dtypes, K-major copies or row-major views of the scales, the [K,M] form of A where it applies."""
+    print(f"case random M={M} N={N} K={K} layout={layout} f16={f16} views={scale_views} seed={seed}", flush=True)
+    A, Bkn, sa, sb = make_problem(seed, M, N, K, f16)
+    B = b_of(Bkn, layout)
+    st = np.float16 if f16 else np.float32
+    sdt = "f16" if f16 else "f32"
+    dA, dB = dev(A), dev(B)
+    dsa = dev(np.ascontiguousarray(sa.astype(st).T)).t() if scale_views & 1 else dev(sa.astype(st))
+    dsb = dev(np.ascontiguousarray(sb.astype(st).T)).t() if scale_views & 2 else dev(sb.astype(st))
+    same(jf.igemm_s32(dA, dB, layout), oracle.igemm_s32(A, B, layout), "s32")
+    acc = oracle.igemm_block_f32(A, B, sa, sb, layout)
+    same(jf.igemm_block_fp(dA, dB, dsa, dsb, layout, torch.float32), acc, "fp32")
+    q, sc = jf.igemm_block_q(dA, dB, dsa, dsb, layout)
+    wq, wsc = oracle.requant(acc, scale_dtype=sdt)
+    same(q, wq, "det codes")
+    same(sc, wsc, "det scales")
+    q, sc = jf.igemm_block_q(dA, dB, dsa, dsb, layout, rounding=jf.ROUND_STOCHASTIC, seed=seed, offset=seed % 1000)
+    wq, wsc = oracle.requant(acc, stochastic=True, seed=seed, offset=seed % 1000, scale_dtype=sdt)
+    same(q, wq, "SR codes")
+    same(sc, wsc, "SR scales")
+    if layout == 1:
+        same(jf.igemm_block_fp(dev(np.ascontiguousarray(A.T)), dB, dsa, dsb, layout, torch.float32, a_layout=jf.A_KM), acc, "fp32, A as [K,M]")
+        parts, per = jf.splitk_plan(M, N, K, 0)
+        same(jf.igemm_block_fp(dA, dB, dsa, dsb, layout, torch.float32, splitk=0),
+             oracle.igemm_block_f32_splitk(A, B, sa, sb, layout, parts, per), f"fp32, {parts} parts")
+
+
 def test_block_q_bias(jf, oracle):
     """The forward kernel's bias / biasmax inputs (…BiasRowCol.cu:313,341,357)."""
     M, N, K = 128, 256, 96
