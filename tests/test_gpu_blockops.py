@@ -208,3 +208,18 @@ def test_full_size_nonlinear_properties(jf, oracle):
     assert torch.equal(q2, qy)
     # transpose twice is the identity
     assert torch.equal(jf.transpose_s8(jf.transpose_s8(qy)), qy)
+
+
+def _random_block_shapes(n, seed):
+    rng = np.random.default_rng(seed)
+    for _ in range(n):
+        yield int(rng.integers(1, 11)) * 32, int(rng.integers(1, 130)) * 32, bool(rng.integers(0, 2)), int(rng.integers(0, 2))
+
+
+@pytest.mark.parametrize("R,C,f16,approx", list(_random_block_shapes(12, 7)))
+def test_random_shapes(jf, oracle, R, C, f16, approx):
+    """The GELU and LayerNorm checks above on random tensor shapes (up to 320 x 4128: rows of more column blocks than a
+    workgroup has waves, block counts that are not multiples of the grid)."""
+    test_gelu_fwd_bwd(jf, oracle, R, C, approx, 5e-5 if approx == 0 else 0.0, f16)
+    test_rowstats_layernorm(jf, oracle, R, C, f16)
+    test_quantize(jf, oracle, R, C, "stochastic", f16)
