@@ -52,6 +52,30 @@ def test_one_block_matches_fp32_reference():
         assert cos(got[n], p.grad) > 0.97, n
 
 
+def test_xl_width_block_matches_fp32_reference():
+    """One block at the GPT-2 XL widths (1600 / 4800 / 6400, 25 heads) on 2048 tokens: every operator at its real
+    row length (LayerNorm rows of 50 blocks, GELU rows of 200), weight gradients through the K split."""
+    from recipe import QStack
+    torch.manual_seed(3)
+    B, T, C, H = 2, 1024, 1600, 25
+    model = QStack(1, C, H).cuda()
+    x = torch.randn(B, T, C, device="cuda", requires_grad=True)
+    w = torch.randn(B, T, C, device="cuda")
+    out = model(x)
+    (out * w).sum().backward()
+    got = {n: p.grad.clone() for n, p in model.named_parameters()}
+    gx = x.grad.clone()
+    for p in model.parameters():
+        p.grad = None
+    x2 = x.detach().clone().requires_grad_(True)
+    ref = ref_block(x2, model.blocks[0])
+    (ref * w).sum().backward()
+    assert torch.isfinite(out).all() and cos(out, ref) > 0.999
+    assert cos(gx, x2.grad) > 0.99
+    for n, p in model.named_parameters():
+        assert torch.isfinite(got[n]).all() and cos(got[n], p.grad) > 0.97, (n, cos(got[n], p.grad))
+
+
 def test_small_stack_trains():
     from recipe import QStack
     torch.manual_seed(1)
