@@ -118,6 +118,46 @@ def deep_k_weight_gradients(jf, torch):
     return out
 
 
+def recipe_block(torch):
+    """One GPT-2 XL transformer block (1600 wide, 25 heads) forward + backward on 8 x 1024 tokens: the INT8 data-flow
+    recipe (Jetfire/recipe.py: every linear layer, LayerNorm, GELU and residual add on INT8 block tensors, attention
+    itself in fp16 through torch) next to the same block in plain torch bf16."""
+    import torch.nn.functional as F
+    sys.path.insert(0, os.path.join(PKG, "Jetfire"))
+    from recipe import QStack
+    torch.manual_seed(0)
+    B, T, C, H = 8, 1024, 1600, 25
+    model = QStack(1, C, H).cuda()
+    blk = model.blocks[0]
+    x = torch.randn(B, T, C, device="cuda", requires_grad=True)
+    w = torch.randn(B, T, C, device="cuda")
+
+    def ref_block(xr, dt):
+        h = F.layer_norm(xr, (C,), blk.ln_1.to(dt), None, 1e-5)
+        qkv = h @ blk.w_qkv.to(dt).t()
+        q, k, v = (t.view(B, T, H, C // H).transpose(1, 2) for t in qkv.split(C, dim=2))
+        y = F.scaled_dot_product_attention(q, k, v, is_causal=True).transpose(1, 2).contiguous().view(B, T, C)
+        xr = xr + y @ blk.w_attn_proj.to(dt).t()
+        h = F.layer_norm(xr, (C,), blk.ln_2.to(dt), None, 1e-5)
+        return xr + F.gelu(h @ blk.w_fc.to(dt).t()) @ blk.w_mlp_proj.to(dt).t()
+
+    def t(fn, n=10):
+        for _ in range(3):
+            fn()
+        torch.cuda.synchronize()
+        e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+        e0.record()
+        for _ in range(n):
+            fn()
+        e1.record()
+        torch.cuda.synchronize()
+        return round(e0.elapsed_time(e1) / n, 3)
+
+    xr, wr = x.detach().to(torch.bfloat16).requires_grad_(True), w.to(torch.bfloat16)
+    return {"tokens": B * T, "int8_recipe_ms": t(lambda: model(x).backward(w)),
+            "torch_bf16_ms": t(lambda: ref_block(xr, torch.bfloat16).backward(wr))}
+
+
 def nonlinear_extras(jf, torch):
     """Achieved GB/s (algorithmic bytes / event time) of the memory-bound kernels at the GPT-2 XL sizes of BASELINE
     config 4 (LayerNorm on 8192x1600, GELU on 8192x6400), fp32 scales."""
@@ -298,6 +338,7 @@ def main():
         out["calibration"] = calibration(jf, torch)
         out["memory_bound_kernels"] = nonlinear_extras(jf, torch)
         out["deep_k_weight_gradients"] = deep_k_weight_gradients(jf, torch)
+        out["xl_block_forward_backward"] = recipe_block(torch)
     if not a.no_cpu:
         out["cpu_baseline"] = cpu_baseline(ops, a.cpu_rows)
     print(json.dumps(out))
