@@ -234,6 +234,17 @@ def calibration(jf, torch):
     t, n = jf.calibrate(1, 32)
     out["mfma_plus_32fmac_ns_per_simd"] = round(t * 1e9 * simds / n, 2)
     out["mfma_plus_32fmac_TOPs"] = round(n * 65536 / t / 1e12, 1)
+    a = torch.randn(TOKENS, 1600, device="cuda", dtype=torch.bfloat16)
+    b = torch.randn(6400, 1600, device="cuda", dtype=torch.bfloat16)
+    for _ in range(5):
+        a @ b.t()
+    e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+    e0.record()
+    for _ in range(20):
+        a @ b.t()
+    e1.record()
+    torch.cuda.synchronize()
+    out["torch_bf16_fc_forward_TFLOPs"] = round(2.0 * TOKENS * 6400 * 1600 * 20 / (e0.elapsed_time(e1) * 1e-3) / 1e12, 1)
     out["note"] = ("per SIMD, 4 waves resident; the scale-accumulate needs 32 VALU instructions per MFMA, and the two "
                    "pipes add up rather than overlap: the last line is the ceiling of any exact per-block kernel")
     return out
