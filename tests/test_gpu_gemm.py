@@ -256,6 +256,23 @@ def test_random_shapes(jf, oracle, M, N, K, layout, f16, scale_views, seed):
              oracle.igemm_block_f32_splitk(A, B, sa, sb, layout, parts, per), f"fp32, {parts} parts")
 
 
+@pytest.mark.parametrize("views", [0, 3])
+@pytest.mark.parametrize("a_km", [False, True])
+def test_block_fp_split_k_binary16_scales(jf, oracle, a_km, views):
+    """The K split with binary16 scales (fetched as 32-bit words, half selected by index parity) in both scale layouts."""
+    M, N, K, req = 96, 160, 4128, 3
+    A, Bkn, sa, sb = make_problem(77, M, N, K, f16=True)
+    parts, per = jf.splitk_plan(M, N, K, req)
+    assert parts == 3
+    dA = dev(np.ascontiguousarray(A.T)) if a_km else dev(A)
+    h = np.float16
+    dsa = dev(np.ascontiguousarray(sa.astype(h).T)).t() if views & 1 else dev(sa.astype(h))
+    dsb = dev(np.ascontiguousarray(sb.astype(h).T)).t() if views & 2 else dev(sb.astype(h))
+    want = oracle.igemm_block_f32_splitk(A, Bkn, sa, sb, 1, parts, per)
+    got = jf.igemm_block_fp(dA, dev(Bkn), dsa, dsb, jf.B_KN, torch.float32, splitk=req, a_layout=jf.A_KM if a_km else jf.A_MK)
+    same(got, want, "fp32")
+
+
 def test_block_q_bias(jf, oracle):
     """The forward kernel's bias / biasmax inputs (…BiasRowCol.cu:313,341,357)."""
     M, N, K = 128, 256, 96
