@@ -410,3 +410,39 @@ def test_full_size_small_wgrad_deep_k(jf, oracle):
         rows, rb = slice(r0, r0 + 32), slice(r0 // 32, r0 // 32 + 1)
         want = oracle.igemm_block_f32(GT[rows], X, np.ascontiguousarray(SG[:, rb]), SX, 1)
         same(dw[rows], want, f"wgrad rows {r0}")
+
+
+def test_gemm_entry_points_can_be_captured_in_a_graph(jf, oracle):
+    """The GEMM entry points only launch kernels (no allocation, no synchronisation, no memset), so a caller can record
+    them into a HIP graph: three replays, with eager work and synchronisations in between, all give the eager result."""
+    M, N, K = 256, 384, 2048
+    A, Bkn, sa, sb = make_problem(5, M, N, K, f16=False)
+    dA, dB, dsa, dsb = dev(A), dev(Bkn), dev(sa), dev(sb)
+    L = jf.lib()
+    nb = L.jf_igemm_block_fp_workspace_bytes(M, N, K, jf.B_KN, 4)
+    assert nb > 0
+    ws = torch.empty(nb, dtype=torch.int8, device="cuda")
+    q = torch.empty((M, N), dtype=torch.int8, device="cuda")
+    sc = torch.empty((M // QB, N // QB), dtype=torch.float32, device="cuda")
+    w = torch.empty((M, N), dtype=torch.float32, device="cuda")
+
+    def launch(stream):
+        jf.check(L.jf_igemm_block_q(dA.data_ptr(), dB.data_ptr(), dsa.data_ptr(), dsb.data_ptr(), None, None, q.data_ptr(),
+                                    sc.data_ptr(), M, N, K, jf.B_KN, 1, 0, 0, jf.ROUND_STOCHASTIC, 9, 4, None, 0, stream))
+        jf.check(L.jf_igemm_block_fp(dA.data_ptr(), dB.data_ptr(), dsa.data_ptr(), dsb.data_ptr(), w.data_ptr(), M, N, K,
+                                     jf.A_MK, jf.B_KN, 1, 0, 0, 1, 4, ws.data_ptr(), nb, stream))
+
+    launch(torch.cuda.current_stream().cuda_stream)
+    torch.cuda.synchronize()
+    eq, esc, ew = q.clone(), sc.clone(), w.clone()
+    parts, per = jf.splitk_plan(M, N, K, 4)
+    same(ew, oracle.igemm_block_f32_splitk(A, Bkn, sa, sb, 1, parts, per), "eager split-K")
+    graph = torch.cuda.CUDAGraph()
+    with torch.cuda.graph(graph):
+        launch(torch.cuda.current_stream().cuda_stream)
+    for _ in range(3):
+        q.zero_(); sc.zero_(); w.zero_(); ws.zero_()
+        torch.cuda.synchronize()
+        graph.replay()
+        torch.cuda.synchronize()
+        assert torch.equal(q, eq) and torch.equal(sc, esc) and torch.equal(w, ew)
