@@ -90,6 +90,29 @@ def dominant_kernel_roofline(jf, torch, ops, iters=20):
             "traffic": MEASURED_TRAFFIC_BYTES}
 
 
+def fused_fc_gelu(jf, torch, ops):
+    """The fc forward GEMM followed by the GELU kernel against the GEMM with the GELU in its epilogue (same bits)."""
+    o = ops[2]
+    sx, sw = o["sx"].t(), o["sw"].t()
+
+    def separate():
+        q, s = jf.igemm_block_q(o["qx"], o["qw"], sx, sw, jf.B_NK)
+        return jf.gelu_fwd(q, s)
+
+    out = {}
+    for key, fn in (("gemm_then_gelu_us", separate), ("fused_us", lambda: jf.igemm_block_q_gelu(o["qx"], o["qw"], sx, sw))):
+        for _ in range(3):
+            fn()
+        e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+        e0.record()
+        for _ in range(20):
+            fn()
+        e1.record()
+        torch.cuda.synchronize()
+        out[key] = round(e0.elapsed_time(e1) * 1e3 / 20, 1)
+    return out
+
+
 def deep_k_weight_gradients(jf, torch):
     """Weight gradients of BASELINE config 2 (GPT-2 small, 12288 tokens) and the smallest one of the XL set: few output
     tiles over a deep K.  One accumulation chain per output (the reference's arithmetic) against the library's K split
@@ -349,6 +372,7 @@ def main():
         out["calibration"] = calibration(jf, torch)
         out["memory_bound_kernels"] = nonlinear_extras(jf, torch)
         out["deep_k_weight_gradients"] = deep_k_weight_gradients(jf, torch)
+        out["fc_forward_with_gelu"] = fused_fc_gelu(jf, torch, ops)
         out["xl_block_forward_backward"] = recipe_block(torch)
     if not a.no_cpu:
         out["cpu_baseline"] = cpu_baseline(ops, a.cpu_rows)

@@ -117,6 +117,17 @@ int jf_igemm_block_q(const int8_t *A, const int8_t *B, const void *sa, const voi
                      uint64_t seed, uint64_t offset,
                      void *workspace, size_t workspace_bytes, jf_stream_t stream);
 
+/* The forward GEMM (A [M,K], B [N,K], round-to-nearest) with the GELU forward fused into its epilogue: (C, sc) is what
+ * jf_igemm_block_q writes, (C_gelu, sc_gelu) is what jf_gelu_fwd would make of it (bit for bit, including the scale
+ * as stored in scale_dtype), without the second pass over HBM.  Replaces the pair igemm_output_int_quantize_bias_rowcol
+ * (include/igemm.h:66-77) + int8_gelu_forward (Jetfire/Nonlinear/gelu_fwd.py:128-162) of the recipe's MLP
+ * (INT8_GPT2/qmodel.py:210-214), which needs both tensors: the first for the backward pass, the second as the input
+ * of the next layer. */
+int jf_igemm_block_q_gelu(const int8_t *A, const int8_t *B, const void *sa, const void *sb, const float *bias,
+                          const float *biasmax, int8_t *C, void *sc, int8_t *C_gelu, void *sc_gelu, int M, int N, int K,
+                          int scale_dtype, int sa_layout, int sb_layout, int gelu_approx, float gelu_amax_eps,
+                          jf_stream_t stream);
+
 /* Block quantise x[R,C] (x_dtype: JF_FP_*) -> (q, s); optionally also qT[C,R] = q transposed.
  * Replaces int8_quantize (Jetfire/Nonlinear/quantize.py:128-164) and, with qT != NULL,
  * int8_quantize_transpose (Jetfire/Nonlinear/quantize_transpose.py:131-171). */

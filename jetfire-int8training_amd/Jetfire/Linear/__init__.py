@@ -1,5 +1,5 @@
 """Per-block INT8 linear layer, forward and backward (same names and signatures as the reference's
-Jetfire/Linear package: linear_fwd.py:4, linear_bwd.py:4)."""
-from .linear import int8_linear_backward, int8_linear_forward
+Jetfire/Linear package: linear_fwd.py:4, linear_bwd.py:4), plus the forward with the GELU fused into its epilogue."""
+from .linear import int8_linear_backward, int8_linear_forward, int8_linear_forward_gelu
 
-__all__ = ["int8_linear_forward", "int8_linear_backward"]
+__all__ = ["int8_linear_forward", "int8_linear_backward", "int8_linear_forward_gelu"]

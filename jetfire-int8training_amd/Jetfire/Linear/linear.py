@@ -70,6 +70,23 @@ def int8_linear_forward(X8_3D, SX16_3D, W8, SW16, output_quantized, B):
     return o8.reshape(*lead, n_out), so.reshape(*s_lead, SW16.shape[0])
 
 
+def int8_linear_forward_gelu(X8_3D, SX16_3D, W8, SW16, B, approximate="none"):
+    """int8_linear_forward(..., output_quantized=True) followed by int8_gelu_forward, in one kernel (no counterpart in
+    the reference, whose MLP runs the two back to back, qmodel.py:210-214).  Returns (O8, SO, G8, SG): the linear
+    output (kept for the backward pass) and its GELU (the next layer's input), bit-identical to the two separate calls."""
+    _check_block(B)
+    if approximate not in ("none", "tanh"):
+        raise RuntimeError("approximate must be 'none' or 'tanh'")
+    lead, s_lead = tuple(X8_3D.shape[:-1]), tuple(SX16_3D.shape[:-1])
+    x2, sx2 = _flat2(X8_3D).contiguous(), _flat2(SX16_3D)
+    n_out = W8.shape[0]
+    o8, so, g8, sg = _jf.igemm_block_q_gelu(x2, W8.contiguous(), _k_major(sx2), _k_major(SW16),
+                                            _jf.GELU_TANH if approximate == "tanh" else _jf.GELU_ERF,
+                                            0.0 if approximate == "tanh" else 5e-5)   # as Nonlinear.int8_gelu_forward
+    shp, sshp = (*lead, n_out), (*s_lead, SW16.shape[0])
+    return o8.reshape(shp), so.reshape(sshp), g8.reshape(shp), sg.reshape(sshp)
+
+
 def int8_linear_backward(X8_3D, SX16_3D, G8_3D, SG16_3D, G8T, W8, SW16, B, stochastic=True, dgrad_quantize=True,
                          wgrad_splitk=1):
     """dX = dY W (requantised with stochastic rounding) and dW = dY^T X (fp16).

@@ -19,8 +19,8 @@ import torch
 import torch.nn as nn
 import torch.nn.functional as F
 
-from Linear import int8_linear_backward, int8_linear_forward
-from Nonlinear import (int8_add_Ifp_Ig16_Ofp_Og, int8_add_Ifp_Ig16_Ofp_Og_MeanVar, int8_gelu_backward, int8_gelu_forward,
+from Linear import int8_linear_backward, int8_linear_forward, int8_linear_forward_gelu
+from Nonlinear import (int8_add_Ifp_Ig16_Ofp_Og, int8_add_Ifp_Ig16_Ofp_Og_MeanVar, int8_gelu_backward,
                        int8_layernorm_backward, int8_layernorm_forward, int8_quantize)
 
 QB = 32
@@ -143,8 +143,7 @@ class MLPResidual(torch.autograd.Function):
         qw1, sw1 = weight_codes.get(w_fc)
         qw2, sw2 = weight_codes.get(w_proj)
         qn, sn, _ = int8_layernorm_forward(qx, sx, ln_w, mean, rstd, QB)
-        qh, sh = int8_linear_forward(qn, sn, qw1, sw1, True, QB)
-        qa, sa = int8_gelu_forward(qh, sh, QB)
+        qh, sh, qa, sa = int8_linear_forward_gelu(qn, sn, qw1, sw1, QB)      # fc and its GELU in one kernel
         qo, so = int8_linear_forward(qa, sa, qw2, sw2, True, QB)
         fp, q, s, mean2, rstd2 = int8_add_Ifp_Ig16_Ofp_Og_MeanVar(residual.contiguous(), qo, so, QB)
         ctx.save_for_backward(qx, sx, qn, sn, qh, sh, qa, sa, qw1, sw1, qw2, sw2, ln_w, mean, rstd)

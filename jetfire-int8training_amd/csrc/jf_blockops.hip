@@ -122,46 +122,6 @@ __global__ __launch_bounds__(NT) void dequantize_kernel(const int8_t *q, const S
     }
 }
 
-// GELU on a block tensor.  A block has ONE scale, so its 1024 inputs take at most 256 distinct values code*scale:
-// the wave evaluates the function once per code (4 codes per lane) into a 1 KiB LDS table and every element then
-// costs one LDS gather instead of ~40 vector instructions.  The table entry is computed from (float)code * scale,
-// the very expression a per-element evaluation would use, so the results are bit-identical to it.
-// PAIR(x, pos, neg) evaluates the function at +x and -x (x >= 0).  Lane l covers the magnitudes 2l+1 and 2l+2
-// (1 .. 128); entry index = the code's byte value, so -m sits at 256-m and index 128 is the code -128.  Entry 0
-// (the function at +0, the same for every block) is passed in.
-template <typename PAIR>
-__device__ __forceinline__ void fill_code_table(float *table, int lane, float scale, float f0, PAIR pair)
-{
-    const int m = 2 * lane + 1;
-    float p0, n0, p1, n1;
-    pair((float)m * scale, p0, n0);
-    pair((float)(m + 1) * scale, p1, n1);
-    table[m] = p0;
-    if (lane < 63) table[m + 1] = p1;                              // +128 is not a code
-    table[256 - m] = n0;
-    table[255 - m] = n1;
-    if (lane == 0) table[0] = f0;
-    __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
-    __builtin_amdgcn_wave_barrier();
-    __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
-}
-__device__ __forceinline__ void gather16(const float *table, v4i p, float x[16])
-{
-    const uint32_t w[4] = {(uint32_t)p.x, (uint32_t)p.y, (uint32_t)p.z, (uint32_t)p.w};
-#pragma unroll
-    for (int i = 0; i < 4; ++i) {
-        x[4 * i + 0] = table[w[i] & 0xFF];
-        x[4 * i + 1] = table[(w[i] >> 8) & 0xFF];
-        x[4 * i + 2] = table[(w[i] >> 16) & 0xFF];
-        x[4 * i + 3] = table[w[i] >> 24];
-    }
-}
-__device__ __forceinline__ void table_done()
-{
-    __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
-    __builtin_amdgcn_wave_barrier();                               // all gathers done before the next block's fill
-}
-
 // A wave that loads one block (1 KiB of codes), waits, computes and stores keeps far too few bytes in flight to
 // cover the memory latency, so the GELU kernels run the block loop with the codes and scales of the next PF blocks
 // already requested.
@@ -231,38 +191,8 @@ __global__ __launch_bounds__(NT) void gelu_fwd_kernel(const int8_t *q, const ST 
         const size_t e0 = (size_t)(w.rb * QB + (lane >> 1)) * C + w.cb * QB + (lane & 1) * 16;
         v4i c; float sc;
         in.next(c, sc);
-        fill_code_table(tab, lane, sc, f0, [](float v, float &a, float &b) { gelu_pair<APPROX>(v, a, b); });
-        // The outputs take at most 256 distinct values too, so the requantisation (exact division, rounding, clamp) is
-        // done on the table, 4 entries per lane, once the block's absmax is known; an element costs two gathers.
-        float x[16];
-        gather16(tab, c, x);
-        float m = 0.0f;
-#pragma unroll
-        for (int k = 0; k < 16; ++k) m = fmaxf(m, fabsf(x[k]));
-        const float amax = wave_max(m) + amax_eps;
-        float scale = 0.0f;
-        v4i codes = {0, 0, 0, 0};
-        if (amax > 0.0f) {                                         // uniform
-            scale = amax / 127.0f;
-            BlockDivisor d(scale);
-            const v4f t4 = *reinterpret_cast<const v4f *>(tab + 4 * lane);
-            const float t[4] = {t4.x, t4.y, t4.z, t4.w};
-            float y[4];
-            d.divn<4>(t, y);
-            v4i q4 = {clamp127(__builtin_rintf(y[0])), clamp127(__builtin_rintf(y[1])), clamp127(__builtin_rintf(y[2])),
-                      clamp127(__builtin_rintf(y[3]))};
-            *reinterpret_cast<v4i *>(qtab + 4 * lane) = q4;
-            __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
-            __builtin_amdgcn_wave_barrier();
-            __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
-            const uint32_t wd[4] = {(uint32_t)c.x, (uint32_t)c.y, (uint32_t)c.z, (uint32_t)c.w};
-            int o[4];
-#pragma unroll
-            for (int i = 0; i < 4; ++i)
-                o[i] = (int)pack4(qtab[wd[i] & 0xFF], qtab[(wd[i] >> 8) & 0xFF], qtab[(wd[i] >> 16) & 0xFF], qtab[wd[i] >> 24]);
-            codes = v4i{o[0], o[1], o[2], o[3]};
-        }
-        table_done();
+        float scale;
+        const v4i codes = gelu_fwd_block<APPROX>(c, sc, f0, amax_eps, tab, qtab, lane, &scale);
         *reinterpret_cast<v4i *>(qy + e0) = codes;
         if (lane == 0) store_scale(sy, w.rb * SC + w.cb, scale);
     }

@@ -35,7 +35,8 @@ constexpr int KB_STAGE = 4;                         // 32-deep K blocks per LDS 
 constexpr int ROW_BYTES = KB_STAGE * QB;            // 128: one LDS row = one 128-byte global segment
 constexpr int EPI_LD = 36;                          // floats per staged row (32 + pad, keeps 16B alignment)
 
-enum Epilogue { EPI_S32 = 0, EPI_FP = 1, EPI_Q = 2 };
+// EPI_QG: EPI_Q (deterministic) followed by the GELU forward of the block just requantised: two block tensors leave
+enum Epilogue { EPI_S32 = 0, EPI_FP = 1, EPI_Q = 2, EPI_QG = 3 };
 
 struct GemmArgs {
     const int8_t *A;      // [M, lda] (K-contiguous) or, for the AKM kernels, [K, lda] (M-contiguous rows)
@@ -54,6 +55,9 @@ struct GemmArgs {
                                 // s = w / tiles, and stores fp32 partial sums at C + s*M*N
     int out_dtype;        // JF_FP_*        (EPI_FP)
     int rounding;         // JF_ROUND_*     (EPI_Q)
+    void *C2, *sc2;       // s8 [M, N], [M/32, N/32]: GELU of the requantised result   (EPI_QG)
+    int gelu_approx;      // JF_GELU_*
+    float gelu_eps;       // added to the GELU output's block absmax (the reference: 5e-5, gelu_fwd.py:93)
 };
 
 // Logical tile (and K split) of this workgroup.  Workgroups are dealt round-robin to the 8 XCDs, each with a
@@ -584,8 +588,16 @@ __global__ __launch_bounds__(64 * WGM * WGN, WGPC * WGM * WGN / 4) void igemm_nt
     float *patch = reinterpret_cast<float *>(smem) + wave * (QB * EPI_LD);
     unsigned char *tile = smem + NW * (QB * EPI_LD) * sizeof(float);       // [BM][BN * out_bytes]
     const int rrow = lane >> 1, rcol = (lane & 1) * 16;
-    const float biasmax = (EPI == EPI_Q && p.biasmax) ? p.biasmax[0] : 0.0f;
-    const int out_bytes = EPI == EPI_Q ? 1 : (EPI == EPI_FP && p.out_dtype != JF_FP_F32 ? 2 : 4);   // uniform
+    constexpr bool QUANT = EPI == EPI_Q || EPI == EPI_QG;
+    const float biasmax = (QUANT && p.biasmax) ? p.biasmax[0] : 0.0f;
+    const int out_bytes = QUANT ? 1 : (EPI == EPI_FP && p.out_dtype != JF_FP_F32 ? 2 : 4);   // uniform
+    unsigned char *tile2 = tile + BM * BN;                    // EPI_QG: image of the second output
+    float gelu_f0 = 0.0f;                                     // gelu(+0), evaluated on the device like every table entry
+    if (EPI == EPI_QG) {
+        float zero = 0.0f;
+        asm volatile("" : "+v"(zero));
+        gelu_f0 = p.gelu_approx == JF_GELU_TANH ? gelu<JF_GELU_TANH>(zero) : gelu<JF_GELU_ERF>(zero);
+    }
 
 #pragma unroll
     for (int i = 0; i < WBM; ++i)
@@ -595,7 +607,7 @@ __global__ __launch_bounds__(64 * WGM * WGN, WGPC * WGM * WGN / 4) void igemm_nt
             const bool valid = bm < p.M && bn < p.N;          // wave-uniform
             if (!valid) continue;
             float amax = 0.0f;
-            if (EPI == EPI_Q) {
+            if (QUANT) {
                 float m = 0.0f;
 #pragma unroll
                 for (int v = 0; v < 16; ++v) m = fmaxf(m, fabsf(acc[i][j][v]));
@@ -677,6 +689,20 @@ __global__ __launch_bounds__(64 * WGM * WGN, WGPC * WGM * WGN / 4) void igemm_nt
                 }
                 *reinterpret_cast<v4i *>(tile + (size_t)trow * BN + tcol) = codes;
                 if (lane == 0) store_scale(reinterpret_cast<ST *>(p.sc), (bm / QB) * SN + bn / QB, scale);
+                if (EPI == EPI_QG) {
+                    // GELU of the block as a reader of the stored tensor would see it (codes x the scale rounded to ST),
+                    // with the wave's patch (free again) as the code tables
+                    const float stored = (float)(ST)scale;
+                    float *tab = patch;
+                    int *qtab = reinterpret_cast<int *>(patch + 256);
+                    float scale2;
+                    const v4i codes2 = p.gelu_approx == JF_GELU_TANH
+                        ? gelu_fwd_block<JF_GELU_TANH>(codes, stored, gelu_f0, p.gelu_eps, tab, qtab, lane, &scale2)
+                        : gelu_fwd_block<JF_GELU_ERF>(codes, stored, gelu_f0, p.gelu_eps, tab, qtab, lane, &scale2);
+                    *reinterpret_cast<v4i *>(tile2 + (size_t)trow * BN + tcol) = codes2;
+                    if (lane == 0) store_scale(reinterpret_cast<ST *>(p.sc2), (bm / QB) * SN + bn / QB, scale2);
+                    wave_sync();                              // the tables are the next block's patch
+                }
             }
         }
 
@@ -691,6 +717,9 @@ __global__ __launch_bounds__(64 * WGM * WGN, WGPC * WGM * WGN / 4) void igemm_nt
             if (gm < p.M && gn < p.N)
                 *reinterpret_cast<v4i *>(cbase + ((size_t)gm * p.N + gn) * out_bytes) =
                     *reinterpret_cast<const v4i *>(tile + (size_t)row * row_bytes + ch * 16);
+            if (EPI == EPI_QG && gm < p.M && gn < p.N)
+                *reinterpret_cast<v4i *>(reinterpret_cast<unsigned char *>(p.C2) + (size_t)gm * p.N + gn) =
+                    *reinterpret_cast<const v4i *>(tile2 + (size_t)row * row_bytes + ch * 16);
         }
     }
 }
@@ -734,7 +763,7 @@ static int launch_gemm_cfg(const GemmArgs &a, hipStream_t st)
 {
     constexpr int BM = QB * WBM * WGM, BN = QB * WBN * WGN, NT = 64 * WGM * WGN;
     constexpr int RING = NSTAGE * (BM + BN) * ROW_BYTES + WGM * WGN * NSTAGE * 256;   // operand ring + per-wave scale patches
-    constexpr int PATCH = WGM * WGN * QB * EPI_LD * (int)sizeof(float) + (EPI == EPI_S32 ? 0 : BM * BN * (EPI == EPI_Q ? 1 : 2));   // + tile image
+    constexpr int PATCH = WGM * WGN * QB * EPI_LD * (int)sizeof(float) + (EPI == EPI_S32 ? 0 : BM * BN * (EPI == EPI_Q ? 1 : 2));   // + tile image(s): bytes, 2-byte values, or two of bytes
     constexpr int SMEM = RING > PATCH ? RING : PATCH;
     if (!device_is_gfx950()) return JF_ERR_DEVICE;
     GemmArgs p = a;
@@ -811,17 +840,22 @@ constexpr bool KN_NATIVE = (JF_GEMM_CFG == 0);
 template <int EPI, typename ST> static int launch_gemm(const GemmArgs &a, hipStream_t st, bool b_kn, bool a_km = false)
 {
 #if JF_GEMM_CFG == 0
-    if (a_km) {
-        if constexpr (EPI == EPI_FP) {
-            if (b_kn) return launch_gemm_cfg<EPI, ST, 2, 4, 2, 2, 1, 1>(a, st);
+    if constexpr (EPI == EPI_QG) {                            // the forward form only: A [M,K], B [N,K]
+        if (a_km || b_kn) return JF_ERR_UNSUPPORTED;
+        return launch_gemm_cfg<EPI, ST, 2, 4, 2, 2, 0>(a, st);
+    } else {
+        if (a_km) {
+            if constexpr (EPI == EPI_FP) {
+                if (b_kn) return launch_gemm_cfg<EPI, ST, 2, 4, 2, 2, 1, 1>(a, st);
+            }
+            return JF_ERR_UNSUPPORTED;
         }
-        return JF_ERR_UNSUPPORTED;
+        return b_kn ? launch_gemm_cfg<EPI, ST, 2, 4, 2, 2, 1>(a, st) : launch_gemm_cfg<EPI, ST, 2, 4, 2, 2, 0>(a, st);
     }
-    return b_kn ? launch_gemm_cfg<EPI, ST, 2, 4, 2, 2, 1>(a, st) : launch_gemm_cfg<EPI, ST, 2, 4, 2, 2, 0>(a, st);
 #else
     // 256x128 or 128x256, whichever pads the problem less (1600 = 12.5 x 128 but 6.25 x 256); 16 waves, 3-deep ring
     (void)b_kn;
-    if (a_km) return JF_ERR_UNSUPPORTED;
+    if (a_km || EPI == EPI_QG) return JF_ERR_UNSUPPORTED;
     auto padded = [](long d, long t) { return (d + t - 1) / t * t; };
     const long tall = padded(a.M, 256) * padded(a.N, 128), wide = padded(a.M, 128) * padded(a.N, 256);
     return tall <= wide ? launch_gemm_cfg<EPI, ST, 4, 4, 3, 1, 0>(a, st) : launch_gemm_cfg<EPI, ST, 2, 8, 3, 1, 0>(a, st);
@@ -992,6 +1026,27 @@ int jf_igemm_block_q(const int8_t *A, const int8_t *B, const void *sa, const voi
     if (!scale_strides(sa_layout, K, M / QB, a.sa_ks, a.sa_is) || !scale_strides(sb_layout, K, N / QB, a.sb_ks, a.sb_is))
         return JF_ERR_ENUM;
     return scale_dtype == JF_SCALE_F16 ? launch_gemm<EPI_Q, half_t>(a, st, kn) : launch_gemm<EPI_Q, float>(a, st, kn);
+}
+
+int jf_igemm_block_q_gelu(const int8_t *A, const int8_t *B, const void *sa, const void *sb, const float *bias,
+                          const float *biasmax, int8_t *C, void *sc, int8_t *C_gelu, void *sc_gelu, int M, int N, int K,
+                          int scale_dtype, int sa_layout, int sb_layout, int gelu_approx, float gelu_amax_eps,
+                          jf_stream_t stream)
+{
+    int rc = check_gemm_common(A, B, C, M, N, K, JF_B_NK, nullptr, 0);
+    if (rc) return rc;
+    if (!sa || !sb || !sc || !C_gelu || !sc_gelu) return JF_ERR_NULL;
+    if ((scale_dtype != JF_SCALE_F16 && scale_dtype != JF_SCALE_F32) ||
+        (gelu_approx != JF_GELU_ERF && gelu_approx != JF_GELU_TANH)) return JF_ERR_ENUM;
+    if (!aligned16(C_gelu)) return JF_ERR_ALIGN;
+    GemmArgs a = {};
+    a.A = A; a.B = B; a.sa = sa; a.sb = sb; a.C = C; a.sc = sc; a.bias = bias; a.biasmax = biasmax;
+    a.C2 = C_gelu; a.sc2 = sc_gelu; a.gelu_approx = gelu_approx; a.gelu_eps = gelu_amax_eps;
+    a.M = M; a.N = N; a.K = K; a.lda = K; a.ldb = K; a.rounding = JF_ROUND_NEAREST;
+    if (!scale_strides(sa_layout, K, M / QB, a.sa_ks, a.sa_is) || !scale_strides(sb_layout, K, N / QB, a.sb_ks, a.sb_is))
+        return JF_ERR_ENUM;
+    hipStream_t st = (hipStream_t)stream;
+    return scale_dtype == JF_SCALE_F16 ? launch_gemm<EPI_QG, half_t>(a, st, false) : launch_gemm<EPI_QG, float>(a, st, false);
 }
 
 int jf_transpose_s8(const int8_t *in, int R, int C, int8_t *out, jf_stream_t stream)

@@ -26,7 +26,7 @@ GELU_ERF, GELU_TANH = 0, 1
 
 EXPORTS = [
     "jf_error_string", "jf_igemm_workspace_bytes", "jf_igemm_s32", "jf_igemm_block_acc", "jf_igemm_block_fp",
-    "jf_igemm_splitk_plan", "jf_igemm_block_fp_workspace_bytes",
+    "jf_igemm_splitk_plan", "jf_igemm_block_fp_workspace_bytes", "jf_igemm_block_q_gelu",
     "jf_igemm_block_q", "jf_quantize", "jf_dequantize", "jf_transpose_s8", "jf_rowstats", "jf_layernorm_fwd",
     "jf_layernorm_bwd_workspace_bytes", "jf_layernorm_bwd", "jf_gelu_fwd", "jf_gelu_bwd", "jf_add", "jf_calibrate",
 ]
@@ -49,6 +49,7 @@ def lib():
         L.jf_igemm_s32.argtypes = [_p, _p, _p, _i, _i, _i, _i, _p, _sz, _p]
         L.jf_igemm_block_acc.argtypes = [_p, _p, _p, _i, _i, _i, _i, _p, _sz, _p]
         L.jf_igemm_block_fp.argtypes = [_p, _p, _p, _p, _p, _i, _i, _i, _i, _i, _i, _i, _i, _i, _i, _p, _sz, _p]
+        L.jf_igemm_block_q_gelu.argtypes = [_p, _p, _p, _p, _p, _p, _p, _p, _p, _p, _i, _i, _i, _i, _i, _i, _i, _f, _p]
         L.jf_igemm_splitk_plan.argtypes = [_i, _i, _i, _i, C.POINTER(C.c_int), C.POINTER(C.c_int)]
         L.jf_igemm_block_fp_workspace_bytes.argtypes = [_i, _i, _i, _i, _i]
         L.jf_igemm_block_fp_workspace_bytes.restype = _sz
@@ -221,6 +222,25 @@ def igemm_block_fp(A, B, sa, sb, b_layout=B_KN, out_dtype=torch.float16, a_layou
     check(lib().jf_igemm_block_fp(_ptr(A), _ptr(B), _ptr(sa), _ptr(sb), _ptr(out), M, N, K, a_layout, b_layout, code, la,
                                   lb, _FP_CODE[out_dtype], splitk, _ptr(ws), nb, _stream()))
     return out
+
+
+def igemm_block_q_gelu(A, B, sa, sb, approx=GELU_ERF, amax_eps=5e-5, bias=None, biasmax=None):
+    """Forward GEMM (B as [N,K], round to nearest) with the GELU forward fused into its epilogue.
+    Returns (q, s, q_gelu, s_gelu): what igemm_block_q and then gelu_fwd would return."""
+    M, N, K, _, _ = _gemm_operands(A, B, B_NK)
+    code, la, lb = _gemm_scales(sa, sb, M, N, K)
+    if bias is not None:
+        _need(bias, torch.float32, "bias", 1)
+        if bias.numel() != N:
+            raise RuntimeError("bias must have N elements")
+    if biasmax is not None:
+        _need(biasmax, torch.float32, "biasmax", None)
+    q = torch.empty((M, N), dtype=torch.int8, device=A.device)
+    s = torch.empty((M // QB, N // QB), dtype=sa.dtype, device=A.device)
+    qg, sg = torch.empty_like(q), torch.empty_like(s)
+    check(lib().jf_igemm_block_q_gelu(_ptr(A), _ptr(B), _ptr(sa), _ptr(sb), _ptr(bias), _ptr(biasmax), _ptr(q), _ptr(s),
+                                      _ptr(qg), _ptr(sg), M, N, K, code, la, lb, approx, amax_eps, _stream()))
+    return q, s, qg, sg
 
 
 def igemm_block_q(A, B, sa, sb, b_layout=B_KN, bias=None, biasmax=None, rounding=ROUND_NEAREST, seed=None, offset=None):

@@ -176,6 +176,13 @@ def test_linear_package_3d_shapes_and_values(oracle):
     ref = x.reshape(-1, Cin) @ w.t()
     assert torch.nn.functional.cosine_similarity(ofp.reshape(-1).float(), ref.reshape(-1), dim=0) > 0.999
 
+    from Linear import int8_linear_forward_gelu
+    from Nonlinear import int8_gelu_forward
+    for approximate in ("none", "tanh"):
+        f8, fs, fg8, fgs = int8_linear_forward_gelu(qx, sx, qw, sw, 32, approximate)
+        g8, gs = int8_gelu_forward(o8, so, 32, approximate)
+        assert torch.equal(f8, o8) and torch.equal(fs, so) and torch.equal(fg8, g8) and torch.equal(fgs, gs)
+
     qg, sg, qgt = int8_quantize_transpose(g, 32, stochastic=True, transpose_output_2d=True)
     assert tuple(qgt.shape) == (Cout, BS * T)
     assert torch.equal(qgt, int8_transpose(qg, transpose_output_2d=True))

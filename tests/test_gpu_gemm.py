@@ -446,3 +446,31 @@ def test_gemm_entry_points_can_be_captured_in_a_graph(jf, oracle):
         graph.replay()
         torch.cuda.synchronize()
         assert torch.equal(q, eq) and torch.equal(sc, esc) and torch.equal(w, ew)
+
+
+@pytest.mark.parametrize("approx", [0, 1])
+@pytest.mark.parametrize("f16", [True, False])
+@pytest.mark.parametrize("M,N,K", [(128, 256, 96), (96, 160, 224), (256, 384, 544), (32, 32, 32)])
+def test_forward_gemm_with_fused_gelu(jf, oracle, M, N, K, f16, approx):
+    """The fused entry point returns, bit for bit, what the GEMM and then the GELU kernel return (both of which are
+    checked against the oracle elsewhere and here)."""
+    print(f"case q+gelu M={M} N={N} K={K} f16={f16} approx={approx}", flush=True)
+    A, Bkn, sa, sb = make_problem(M + N * 5 + K, M, N, K, f16)
+    sa = sa * np.float32(0.05)                                    # outputs of a few units: the interesting range of GELU
+    B = b_of(Bkn, 0)
+    st = np.float16 if f16 else np.float32
+    sa = sa.astype(st).astype(np.float32)
+    sdt = "f16" if f16 else "f32"
+    dA, dB, dsa, dsb = dev(A), dev(B), dev(sa.astype(st)), dev(sb.astype(st))
+    eps = 5e-5 if approx == 0 else 0.0
+    q, s, qg, sg = jf.igemm_block_q_gelu(dA, dB, dsa, dsb, approx, eps)
+    q0, s0 = jf.igemm_block_q(dA, dB, dsa, dsb, jf.B_NK)
+    qg0, sg0 = jf.gelu_fwd(q0, s0, approx, eps)
+    assert torch.equal(q, q0) and torch.equal(s, s0) and torch.equal(qg, qg0) and torch.equal(sg, sg0)
+    wq, ws = oracle.igemm_block_q(A, B, sa, sb, 0, scale_dtype=sdt)
+    wg, wgs = oracle.gelu_fwd(wq, ws.astype(np.float32), approx, eps, scale_dtype=sdt)
+    same(q, wq, "codes")
+    same(s, ws, "scales")
+    same(qg, wg, "gelu codes")
+    same(sg, wgs, "gelu scales")
+    assert qg.cpu().numpy().any()
