@@ -9,7 +9,8 @@
  *   - return value: 0 on success, a negative JF_ERR_* for a rejected argument, a positive
  *     hipError_t if the launch failed.  jf_error_string() names either.
  *   - a "block tensor" is (q: int8 [R,C] row-major, s: scale [R/32, C/32] row-major), x ~= q*s.
- *     All of R, C, M, N, K must be positive multiples of 32.  Data pointers must be 16-byte aligned.
+ *     All of R, C, M, N, K must be positive multiples of 32.  Data pointers must be 16-byte aligned, scale pointers
+ *     aligned to their element type (2 or 4 bytes); exactly the elements of a scale array are read, nothing beyond.
  *   - `scale_dtype` selects the element type of EVERY scale pointer of the call
  *     (JF_SCALE_F16 = IEEE binary16, what the reference stores; JF_SCALE_F32 = binary32).
  *   - GEMM scale operands are K-major (JF_SCALES_KMAJOR): sa[kb*(M/32)+mb], sb[kb*(N/32)+nb], or, per operand, the
@@ -70,9 +71,10 @@ typedef void *jf_stream_t;
 
 const char *jf_error_string(int code);
 
-/* Bytes of device scratch the GEMM entry points need for this problem.  Currently 0 for both layouts (a JF_B_KN
- * operand is staged as it lies in memory and transposed by the LDS read); callers still ask, and pass what they get,
- * so that a build that re-lays B out first (JF_ERR_WORKSPACE if the buffer is missing) stays a drop-in. */
+/* Bytes of device scratch the GEMM entry points need for this problem: 0 for both layouts (a JF_B_KN operand is
+ * staged as it lies in memory and transposed by the LDS read).  The workspace arguments of jf_igemm_s32,
+ * jf_igemm_block_acc and jf_igemm_block_q are kept for callers written against an implementation that re-lays B out
+ * first; they are ignored and may be NULL / 0. */
 size_t jf_igemm_workspace_bytes(int M, int N, int K, int b_layout);
 
 /* C_s32[M,N] = A[M,K] * B.   Replaces igemm_basic_int8_gemm (include/igemm.h:3-12,

@@ -25,6 +25,8 @@
 // into a private LDS patch.
 #include "jf_device.hpp"
 
+#include <atomic>
+#include <mutex>
 #include <type_traits>
 
 #pragma clang diagnostic ignored "-Winline-asm"     // M0 appears in clobber lists on purpose
@@ -33,6 +35,7 @@ namespace jf {
 
 constexpr int KB_STAGE = 4;                         // 32-deep K blocks per LDS stage (128 bytes of K per row)
 constexpr int ROW_BYTES = KB_STAGE * QB;            // 128: one LDS row = one 128-byte global segment
+constexpr int MAX_DEVICES = 64;                    // devices a process may use (per-device host state below)
 constexpr int EPI_LD = 36;                          // floats per staged row (32 + pad, keeps 16B alignment)
 
 // EPI_QG: EPI_Q (deterministic) followed by the GELU forward of the block just requantised: two block tensors leave
@@ -181,8 +184,7 @@ __global__ __launch_bounds__(64 * WGM * WGN, WGPC * WGM * WGN / 4) void igemm_nt
     // Scales of a stage: every wave fetches, again LDS-direct, the scales it needs itself into a private 256-byte
     // patch (lane l: K block l/16; word l%16 = the wave's WBM A-side scales, then its WBN B-side scales, the rest
     // padding), so that scale reads need no cross-wave synchronisation, every wave has the same number of loads in
-    // flight, and one LDS read per K block fetches all of them.  binary16 scales are fetched as the aligned 32-bit
-    // word that contains them.  The lane keeps a running pointer.
+    // flight, and one LDS read per K block fetches all of them.  The lane keeps a running pointer.
     constexpr int SCALE_WORDS = 64;
     constexpr int NSC = WBM + WBN;                            // scales per wave and K block
     static_assert(NSC <= 4, "one 16-byte LDS read per K block");
@@ -195,10 +197,10 @@ __global__ __launch_bounds__(64 * WGM * WGN, WGPC * WGM * WGN / 4) void igemm_nt
     const unsigned char *const s_base = reinterpret_cast<const unsigned char *>(s_is_a ? p.sa : p.sb);
     auto scale_addr = [&](int kbg) {
         const unsigned e = (unsigned)((kbg + kb_base) * s_ks + s_idx * s_is);
-        return s_base + (sizeof(ST) == 4 ? e * 4u : (e >> 1) * 4u);
+        return s_base + e * (unsigned)sizeof(ST);
     };
     const unsigned char *s_ptr = scale_addr((lane >> 4) < nkb ? (lane >> 4) : nkb - 1);
-    const unsigned s_step = (unsigned)(KB_STAGE * s_ks) * (unsigned)sizeof(ST);   // KB_STAGE*s_ks is even: exact for binary16
+    const unsigned s_step = (unsigned)(KB_STAGE * s_ks) * (unsigned)sizeof(ST);
 
     constexpr int A_LOADS = (BM / 8) / NW;                    // loads 0 .. A_LOADS-1 of a wave fetch A rows, the rest B rows
     static_assert((BM / 8) % NW == 0, "a load instruction fetches rows of one operand");
@@ -216,7 +218,12 @@ __global__ __launch_bounds__(64 * WGM * WGN, WGPC * WGM * WGN / 4) void igemm_nt
                 int kbg = kb0 + (lane >> 4);
                 src = scale_addr(kbg < nkb ? kbg : nkb - 1);
             }
-            asm volatile("s_mov_b32 m0, %1\n\ts_nop 0\n\tglobal_load_lds_dword %0, off" ::"v"(src), "s"(scale_lds) : "memory", "m0");
+            // a binary16 scale is fetched with the 16-bit form (zero-extended into the lane's LDS word): exactly the
+            // element's two bytes are read, whatever the parity of its index or the length of the array
+            if (sizeof(ST) == 4)
+                asm volatile("s_mov_b32 m0, %1\n\ts_nop 0\n\tglobal_load_lds_dword %0, off" ::"v"(src), "s"(scale_lds) : "memory", "m0");
+            else
+                asm volatile("s_mov_b32 m0, %1\n\ts_nop 0\n\tglobal_load_lds_ushort %0, off" ::"v"(src), "s"(scale_lds) : "memory", "m0");
             s_ptr += s_step;
         }
         unsigned la = loff_a, lb = loff_b;
@@ -300,13 +307,6 @@ __global__ __launch_bounds__(64 * WGM * WGN, WGPC * WGM * WGN / 4) void igemm_nt
     for (int i = 0; i < WBM; ++i) { mb[i] = m0 / QB + wm * WBM + i; mb[i] = mb[i] < SM ? mb[i] : SM - 1; }
 #pragma unroll
     for (int j = 0; j < WBN; ++j) { nb[j] = n0 / QB + wn * WBN + j; nb[j] = nb[j] < SN ? nb[j] : SN - 1; }
-
-    // element index of a scale = K block * K stride + these (only its parity matters, for binary16 scales)
-    int par_a[WBM], par_b[WBN];
-#pragma unroll
-    for (int i = 0; i < WBM; ++i) par_a[i] = __builtin_amdgcn_readfirstlane((kb_base * p.sa_ks + mb[i] * p.sa_is) & 1);
-#pragma unroll
-    for (int j = 0; j < WBN; ++j) par_b[j] = __builtin_amdgcn_readfirstlane((kb_base * p.sb_ks + nb[j] * p.sb_is) & 1);
 
     // ---- main loop ----------------------------------------------------------------------------
     // The whole ring is filled up front; afterwards the loads of stage s+NSTAGE are issued when the last K block
@@ -413,18 +413,15 @@ __global__ __launch_bounds__(64 * WGM * WGN, WGPC * WGM * WGN / 4) void igemm_nt
                     iacc[i][j] = __builtin_amdgcn_mfma_i32_32x32x32_i8(fa_reg[CUR][i], fb_reg[CUR][j], iacc[i][j], 0, 0, 0);
         } else {
             float fa[WBM], fb[WBN];
-            // binary16 scales arrive as the 32-bit word that holds them: the half to use is the parity of the
-            // scale's element index (wave-uniform)
-            auto scale_of = [&](float raw, int elem) -> float {
+            // a binary16 scale sits in the low half of its word
+            auto scale_of = [&](float raw) -> float {
                 if (sizeof(ST) == 4) return raw;
-                const uint32_t w = __float_as_uint(raw);
-                const uint16_t h = (elem & 1) ? (uint16_t)(w >> 16) : (uint16_t)w;
-                return (float)__builtin_bit_cast(half_t, h);
+                return (float)__builtin_bit_cast(half_t, (uint16_t)__float_as_uint(raw));
             };
 #pragma unroll
-            for (int i = 0; i < WBM; ++i) fa[i] = scale_of(sc_raw[CUR][i], kbg * p.sa_ks + par_a[i]);
+            for (int i = 0; i < WBM; ++i) fa[i] = scale_of(sc_raw[CUR][i]);
 #pragma unroll
-            for (int j = 0; j < WBN; ++j) fb[j] = scale_of(sc_raw[CUR][WBM + j], kbg * p.sb_ks + par_b[j]);
+            for (int j = 0; j < WBN; ++j) fb[j] = scale_of(sc_raw[CUR][WBM + j]);
             static_for<0, NBLK>([&](auto n_c) {
                 constexpr int n = decltype(n_c)::value, i = n / WBN, j = n % WBN;
                 // asm: as a builtin operand the constant is hoisted into 16 registers instead of being encoded inline.
@@ -770,9 +767,16 @@ static int launch_gemm_cfg(const GemmArgs &a, hipStream_t st)
     p.tiles_m = (p.M + BM - 1) / BM;
     p.tiles_n = (p.N + BN - 1) / BN;
     auto kern = igemm_nt_kernel<EPI, ST, WGM, WGN, NSTAGE, WGPC, BKN, AKM>;
-    // more than 64 KiB of dynamic LDS has to be opted into, per function
-    hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void *>(kern), hipFuncAttributeMaxDynamicSharedMemorySize, SMEM);
-    if (e != hipSuccess) return (int)e;
+    // more than 64 KiB of dynamic LDS has to be opted into, per function and device: once, not on every launch
+    // (the reference sets its attribute on every call, igemm_BlockSquare32OutputIntQuantizeBiasRowCol.cu:418)
+    static std::atomic<bool> opted_in[MAX_DEVICES] = {};
+    int dev = 0;
+    if (hipGetDevice(&dev) != hipSuccess || dev < 0 || dev >= MAX_DEVICES) return JF_ERR_DEVICE;
+    if (!opted_in[dev].load(std::memory_order_acquire)) {
+        hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void *>(kern), hipFuncAttributeMaxDynamicSharedMemorySize, SMEM);
+        if (e != hipSuccess) return (int)e;
+        opted_in[dev].store(true, std::memory_order_release);
+    }
     if (EPI != EPI_FP || p.splits < 1) p.splits = 1;
     hipLaunchKernelGGL(kern, dim3(p.tiles_m * p.tiles_n * p.splits), dim3(NT), SMEM, st, p);
     return (int)hipGetLastError();
@@ -828,18 +832,11 @@ static void splitk_plan(int M, int N, int K, int request, int &splits, int &kb_p
     splits = (nkb + kb_per_split - 1) / kb_per_split;
 }
 
-// Tile configuration.  JF_GEMM_CFG selects it at build time (for experiments); the default is 128x128 tiles,
-// 8 waves, a 2-deep ring and two workgroups per CU (the epilogue of one overlaps the main loop of the other).
-// The default configuration reads a [K,N] B operand in place; the experimental one transposes it into the
-// caller's workspace first.
-#ifndef JF_GEMM_CFG
-#define JF_GEMM_CFG 0
-#endif
-constexpr bool KN_NATIVE = (JF_GEMM_CFG == 0);
+// Tile configuration: 128x128 tiles, 8 waves, a 2-deep ring and two workgroups per CU (the epilogue of one overlaps
+// the main loop of the other).  A [K,N] B operand (and, for the weight gradient, a [K,M] A operand) is read in place.
 // a_km (A given as [K,M]) exists for the weight-gradient form only: fp output, B as [K,N].
 template <int EPI, typename ST> static int launch_gemm(const GemmArgs &a, hipStream_t st, bool b_kn, bool a_km = false)
 {
-#if JF_GEMM_CFG == 0
     if constexpr (EPI == EPI_QG) {                            // the forward form only: A [M,K], B [N,K]
         if (a_km || b_kn) return JF_ERR_UNSUPPORTED;
         return launch_gemm_cfg<EPI, ST, 2, 4, 2, 2, 0>(a, st);
@@ -852,41 +849,15 @@ template <int EPI, typename ST> static int launch_gemm(const GemmArgs &a, hipStr
         }
         return b_kn ? launch_gemm_cfg<EPI, ST, 2, 4, 2, 2, 1>(a, st) : launch_gemm_cfg<EPI, ST, 2, 4, 2, 2, 0>(a, st);
     }
-#else
-    // 256x128 or 128x256, whichever pads the problem less (1600 = 12.5 x 128 but 6.25 x 256); 16 waves, 3-deep ring
-    (void)b_kn;
-    if (a_km || EPI == EPI_QG) return JF_ERR_UNSUPPORTED;
-    auto padded = [](long d, long t) { return (d + t - 1) / t * t; };
-    const long tall = padded(a.M, 256) * padded(a.N, 128), wide = padded(a.M, 128) * padded(a.N, 256);
-    return tall <= wide ? launch_gemm_cfg<EPI, ST, 4, 4, 3, 1, 0>(a, st) : launch_gemm_cfg<EPI, ST, 2, 8, 3, 1, 0>(a, st);
-#endif
 }
 
-static int check_gemm_common(const void *A, const void *B, const void *C, int M, int N, int K, int b_layout,
-                             const void *ws, size_t ws_bytes)
+static int check_gemm_common(const void *A, const void *B, const void *C, int M, int N, int K, int b_layout)
 {
     if (!A || !B || !C) return JF_ERR_NULL;
     if (!mult32(M) || !mult32(N) || !mult32(K)) return JF_ERR_SHAPE;
     if (b_layout != JF_B_NK && b_layout != JF_B_KN) return JF_ERR_ENUM;
     if (!aligned16(A) || !aligned16(B) || !aligned16(C)) return JF_ERR_ALIGN;
-    if (b_layout == JF_B_KN && !KN_NATIVE) {
-        if (!ws || ws_bytes < (size_t)N * (size_t)K) return JF_ERR_WORKSPACE;
-        if (!aligned16(ws)) return JF_ERR_ALIGN;
-    }
     return JF_OK;
-}
-
-// Prepares the B operand: returns true if the kernel is to read it as [K,N] in place (leading dimension N);
-// otherwise B is [N,K] (the caller's buffer, or its transpose in the workspace) with leading dimension K.
-static bool prepare_b(const int8_t *&B, int &ldb, int N, int K, int b_layout, void *ws, hipStream_t st, int &rc)
-{
-    rc = JF_OK;
-    ldb = K;
-    if (b_layout == JF_B_NK) return false;
-    if (KN_NATIVE) { ldb = N; return true; }
-    rc = launch_transpose(B, K, N, reinterpret_cast<int8_t *>(ws), st);
-    B = reinterpret_cast<const int8_t *>(ws);
-    return false;
 }
 
 }  // namespace jf
@@ -912,38 +883,34 @@ const char *jf_error_string(int code)
 
 size_t jf_igemm_workspace_bytes(int M, int N, int K, int b_layout)
 {
-    (void)M;
-    return (b_layout == JF_B_KN && !KN_NATIVE) ? (size_t)N * (size_t)K : 0;
+    (void)M; (void)N; (void)K; (void)b_layout;                // both B layouts are read in place
+    return 0;
 }
 
 int jf_igemm_s32(const int8_t *A, const int8_t *B, int32_t *C, int M, int N, int K, int b_layout,
                  void *workspace, size_t workspace_bytes, jf_stream_t stream)
 {
-    int rc = check_gemm_common(A, B, C, M, N, K, b_layout, workspace, workspace_bytes);
+    (void)workspace; (void)workspace_bytes;
+    int rc = check_gemm_common(A, B, C, M, N, K, b_layout);
     if (rc) return rc;
-    hipStream_t st = (hipStream_t)stream;
-    int ldb;
-    const bool kn = prepare_b(B, ldb, N, K, b_layout, workspace, st, rc);
-    if (rc) return rc;
+    const bool kn = b_layout == JF_B_KN;
     GemmArgs a = {};
-    a.A = A; a.B = B; a.C = C; a.M = M; a.N = N; a.K = K; a.lda = K; a.ldb = ldb;
-    return launch_gemm<EPI_S32, float>(a, st, kn);
+    a.A = A; a.B = B; a.C = C; a.M = M; a.N = N; a.K = K; a.lda = K; a.ldb = kn ? N : K;
+    return launch_gemm<EPI_S32, float>(a, (hipStream_t)stream, kn);
 }
 
 int jf_igemm_block_acc(const int8_t *A, const int8_t *B, int32_t *acc, int M, int N, int K, int b_layout,
                        void *workspace, size_t workspace_bytes, jf_stream_t stream)
 {
-    int rc = check_gemm_common(A, B, acc, M, N, K, b_layout, workspace, workspace_bytes);
+    (void)workspace; (void)workspace_bytes;
+    int rc = check_gemm_common(A, B, acc, M, N, K, b_layout);
     if (rc) return rc;
-    hipStream_t st = (hipStream_t)stream;
-    int ldb;
-    const bool kn = prepare_b(B, ldb, N, K, b_layout, workspace, st, rc);
-    if (rc) return rc;
+    const bool kn = b_layout == JF_B_KN;
     for (int kb = 0; kb < K / QB; ++kb) {
         GemmArgs a = {};
         a.A = A + kb * QB; a.B = kn ? B + (size_t)kb * QB * N : B + kb * QB; a.C = acc + (size_t)kb * M * N;
-        a.M = M; a.N = N; a.K = QB; a.lda = K; a.ldb = ldb;
-        if ((rc = launch_gemm<EPI_S32, float>(a, st, kn))) return rc;
+        a.M = M; a.N = N; a.K = QB; a.lda = K; a.ldb = kn ? N : K;
+        if ((rc = launch_gemm<EPI_S32, float>(a, (hipStream_t)stream, kn))) return rc;
     }
     return JF_OK;
 }
@@ -956,53 +923,74 @@ static bool scale_strides(int layout, int K, int blocks, int &ks, int &is)
     return false;
 }
 
+// scale arrays need the natural alignment of their element type (binary16 scales are fetched one element at a time)
+static bool scale_ptr_ok(const void *p, int scale_dtype)
+{
+    return (reinterpret_cast<uintptr_t>(p) & (scale_dtype == JF_SCALE_F32 ? 3u : 1u)) == 0;
+}
+
 int jf_igemm_splitk_plan(int M, int N, int K, int splitk, int *splits, int *kb_per_split)
 {
     if (!mult32(M) || !mult32(N) || !mult32(K)) return JF_ERR_SHAPE;
     if (splitk < 0 || !splits || !kb_per_split) return splitk < 0 ? JF_ERR_ENUM : JF_ERR_NULL;
-    if (KN_NATIVE) splitk_plan(M, N, K, splitk, *splits, *kb_per_split);
-    else { *splits = 1; *kb_per_split = (K / QB + 3) / 4 * 4; }
+    splitk_plan(M, N, K, splitk, *splits, *kb_per_split);
     return JF_OK;
 }
 
 size_t jf_igemm_block_fp_workspace_bytes(int M, int N, int K, int b_layout, int splitk)
 {
+    (void)b_layout;
     int splits = 1, kb_per = 0;
     if (jf_igemm_splitk_plan(M, N, K, splitk, &splits, &kb_per) != JF_OK) return 0;
-    return jf_igemm_workspace_bytes(M, N, K, b_layout) + (splits > 1 ? (size_t)splits * (size_t)M * (size_t)N * sizeof(float) : 0);
+    return splits > 1 ? (size_t)splits * (size_t)M * (size_t)N * sizeof(float) : 0;
+}
+
+// The fp-output GEMM behind both of its entry points.  partials: fp32 [splits][M][N] scratch for the K split (only
+// touched when the plan has more than one part; every element of it that is read has been written by this call).
+static int block_fp_run(const int8_t *A, const int8_t *B, const void *sa, const void *sb, void *C, int M, int N, int K,
+                        int a_layout, int b_layout, int scale_dtype, int sa_layout, int sb_layout, int out_dtype,
+                        int splits, int kb_per, void *partials, hipStream_t st)
+{
+    GemmArgs a = {};
+    const bool a_km = a_layout == JF_A_KM, kn = b_layout == JF_B_KN;
+    a.A = A; a.B = B; a.sa = sa; a.sb = sb; a.C = C; a.M = M; a.N = N; a.K = K; a.lda = a_km ? M : K; a.ldb = kn ? N : K;
+    if (!scale_strides(sa_layout, K, M / QB, a.sa_ks, a.sa_is) || !scale_strides(sb_layout, K, N / QB, a.sb_ks, a.sb_is))
+        return JF_ERR_ENUM;
+    a.out_dtype = out_dtype;
+    a.splits = splits; a.kb_per_split = kb_per;
+    if (splits > 1) a.C = partials;
+    int rc = scale_dtype == JF_SCALE_F16 ? launch_gemm<EPI_FP, half_t>(a, st, kn, a_km) : launch_gemm<EPI_FP, float>(a, st, kn, a_km);
+    if (rc || splits == 1) return rc;
+    const size_t n = (size_t)M * (size_t)N;
+    hipLaunchKernelGGL(splitk_reduce_kernel, dim3((unsigned)(n / 1024)), dim3(256), 0, st, (const float *)partials, n, splits, C, out_dtype);
+    return (int)hipGetLastError();
+}
+
+static int block_fp_check(const int8_t *A, const int8_t *B, const void *sa, const void *sb, void *C, int M, int N, int K,
+                          int a_layout, int b_layout, int scale_dtype, int out_dtype)
+{
+    int rc = check_gemm_common(A, B, C, M, N, K, b_layout);
+    if (rc) return rc;
+    if (a_layout != JF_A_MK && a_layout != JF_A_KM) return JF_ERR_ENUM;
+    if (!sa || !sb) return JF_ERR_NULL;
+    if ((scale_dtype != JF_SCALE_F16 && scale_dtype != JF_SCALE_F32) ||
+        (out_dtype != JF_FP_F16 && out_dtype != JF_FP_F32 && out_dtype != JF_FP_BF16)) return JF_ERR_ENUM;
+    if (!scale_ptr_ok(sa, scale_dtype) || !scale_ptr_ok(sb, scale_dtype)) return JF_ERR_ALIGN;
+    return JF_OK;
 }
 
 int jf_igemm_block_fp(const int8_t *A, const int8_t *B, const void *sa, const void *sb, void *C,
                       int M, int N, int K, int a_layout, int b_layout, int scale_dtype, int sa_layout, int sb_layout,
                       int out_dtype, int splitk, void *workspace, size_t workspace_bytes, jf_stream_t stream)
 {
-    int rc = check_gemm_common(A, B, C, M, N, K, b_layout, workspace, workspace_bytes);
+    int rc = block_fp_check(A, B, sa, sb, C, M, N, K, a_layout, b_layout, scale_dtype, out_dtype);
     if (rc) return rc;
-    if (a_layout != JF_A_MK && a_layout != JF_A_KM) return JF_ERR_ENUM;
     int splits = 1, kb_per = 0;
     if ((rc = jf_igemm_splitk_plan(M, N, K, splitk, &splits, &kb_per))) return rc;
     if (splits > 1 && (!workspace || !aligned16(workspace) || workspace_bytes < jf_igemm_block_fp_workspace_bytes(M, N, K, b_layout, splitk)))
         return JF_ERR_WORKSPACE;
-    if (!sa || !sb) return JF_ERR_NULL;
-    if ((scale_dtype != JF_SCALE_F16 && scale_dtype != JF_SCALE_F32) ||
-        (out_dtype != JF_FP_F16 && out_dtype != JF_FP_F32 && out_dtype != JF_FP_BF16)) return JF_ERR_ENUM;
-    hipStream_t st = (hipStream_t)stream;
-    int ldb;
-    const bool kn = prepare_b(B, ldb, N, K, b_layout, workspace, st, rc);
-    if (rc) return rc;
-    GemmArgs a = {};
-    const bool a_km = a_layout == JF_A_KM;
-    a.A = A; a.B = B; a.sa = sa; a.sb = sb; a.C = C; a.M = M; a.N = N; a.K = K; a.lda = a_km ? M : K; a.ldb = ldb;
-    if (!scale_strides(sa_layout, K, M / QB, a.sa_ks, a.sa_is) || !scale_strides(sb_layout, K, N / QB, a.sb_ks, a.sb_is))
-        return JF_ERR_ENUM;
-    a.out_dtype = out_dtype;
-    a.splits = splits; a.kb_per_split = kb_per;
-    if (splits > 1) a.C = workspace;                          // fp32 partial sums [splits][M][N]
-    rc = scale_dtype == JF_SCALE_F16 ? launch_gemm<EPI_FP, half_t>(a, st, kn, a_km) : launch_gemm<EPI_FP, float>(a, st, kn, a_km);
-    if (rc || splits == 1) return rc;
-    const size_t n = (size_t)M * (size_t)N;
-    hipLaunchKernelGGL(splitk_reduce_kernel, dim3((unsigned)(n / 1024)), dim3(256), 0, st, (const float *)workspace, n, splits, C, out_dtype);
-    return (int)hipGetLastError();
+    return block_fp_run(A, B, sa, sb, C, M, N, K, a_layout, b_layout, scale_dtype, sa_layout, sb_layout, out_dtype, splits,
+                        kb_per, workspace, (hipStream_t)stream);
 }
 
 int jf_igemm_block_q(const int8_t *A, const int8_t *B, const void *sa, const void *sb,
@@ -1011,20 +999,20 @@ int jf_igemm_block_q(const int8_t *A, const int8_t *B, const void *sa, const voi
                      uint64_t seed, uint64_t offset,
                      void *workspace, size_t workspace_bytes, jf_stream_t stream)
 {
-    int rc = check_gemm_common(A, B, C, M, N, K, b_layout, workspace, workspace_bytes);
+    (void)workspace; (void)workspace_bytes;
+    int rc = check_gemm_common(A, B, C, M, N, K, b_layout);
     if (rc) return rc;
     if (!sa || !sb || !sc) return JF_ERR_NULL;
     if ((scale_dtype != JF_SCALE_F16 && scale_dtype != JF_SCALE_F32) ||
         (rounding != JF_ROUND_NEAREST && rounding != JF_ROUND_STOCHASTIC)) return JF_ERR_ENUM;
-    hipStream_t st = (hipStream_t)stream;
-    int ldb;
-    const bool kn = prepare_b(B, ldb, N, K, b_layout, workspace, st, rc);
-    if (rc) return rc;
+    if (!scale_ptr_ok(sa, scale_dtype) || !scale_ptr_ok(sb, scale_dtype)) return JF_ERR_ALIGN;
+    const bool kn = b_layout == JF_B_KN;
     GemmArgs a = {};
     a.A = A; a.B = B; a.sa = sa; a.sb = sb; a.C = C; a.sc = sc; a.bias = bias; a.biasmax = biasmax;
-    a.M = M; a.N = N; a.K = K; a.lda = K; a.ldb = ldb; a.rounding = rounding; a.seed = seed; a.offset = offset;
+    a.M = M; a.N = N; a.K = K; a.lda = K; a.ldb = kn ? N : K; a.rounding = rounding; a.seed = seed; a.offset = offset;
     if (!scale_strides(sa_layout, K, M / QB, a.sa_ks, a.sa_is) || !scale_strides(sb_layout, K, N / QB, a.sb_ks, a.sb_is))
         return JF_ERR_ENUM;
+    hipStream_t st = (hipStream_t)stream;
     return scale_dtype == JF_SCALE_F16 ? launch_gemm<EPI_Q, half_t>(a, st, kn) : launch_gemm<EPI_Q, float>(a, st, kn);
 }
 
@@ -1033,12 +1021,12 @@ int jf_igemm_block_q_gelu(const int8_t *A, const int8_t *B, const void *sa, cons
                           int scale_dtype, int sa_layout, int sb_layout, int gelu_approx, float gelu_amax_eps,
                           jf_stream_t stream)
 {
-    int rc = check_gemm_common(A, B, C, M, N, K, JF_B_NK, nullptr, 0);
+    int rc = check_gemm_common(A, B, C, M, N, K, JF_B_NK);
     if (rc) return rc;
     if (!sa || !sb || !sc || !C_gelu || !sc_gelu) return JF_ERR_NULL;
     if ((scale_dtype != JF_SCALE_F16 && scale_dtype != JF_SCALE_F32) ||
         (gelu_approx != JF_GELU_ERF && gelu_approx != JF_GELU_TANH)) return JF_ERR_ENUM;
-    if (!aligned16(C_gelu)) return JF_ERR_ALIGN;
+    if (!aligned16(C_gelu) || !scale_ptr_ok(sa, scale_dtype) || !scale_ptr_ok(sb, scale_dtype)) return JF_ERR_ALIGN;
     GemmArgs a = {};
     a.A = A; a.B = B; a.sa = sa; a.sb = sb; a.C = C; a.sc = sc; a.bias = bias; a.biasmax = biasmax;
     a.C2 = C_gelu; a.sc2 = sc_gelu; a.gelu_approx = gelu_approx; a.gelu_eps = gelu_amax_eps;

@@ -38,6 +38,11 @@ def test_argument_errors_without_gpu(jf):
     assert L.jf_igemm_s32(p, p, p, 32, 32, 32, 7, None, 0, None) == -3          # unknown layout
     assert L.jf_igemm_s32(p + 1, p, p, 32, 32, 32, 0, None, 0, None) == -4      # misaligned
     assert L.jf_quantize(p, 9, 32, 32, p, p, None, 0, 0, 0, 0, 0.0, None) == -3
+    # scale arrays: natural alignment of their element type (2 bytes for binary16, 4 for binary32)
+    q_args = (None, None, p, p, 32, 32, 32, 0)
+    assert L.jf_igemm_block_q(p, p, p + 2, p, *q_args, 1, 0, 0, 0, 0, 0, None, 0, None) == -4
+    assert L.jf_igemm_block_q(p, p, p + 1, p, *q_args, 0, 0, 0, 0, 0, 0, None, 0, None) == -4
+    assert L.jf_igemm_block_q(p, p, p + 2, p, *q_args, 0, 0, 0, 0, 0, 0, None, 0, None) in (0, -6)
     import torch
     if not torch.cuda.is_available():
         # valid arguments, but no gfx950 device to run on: refused by name, nothing is launched
