@@ -38,6 +38,7 @@ extern "C" {
 #define JF_ERR_WORKSPACE     -5   /* workspace missing or smaller than required      */
 #define JF_ERR_DEVICE        -6   /* the current device is not gfx950                */
 #define JF_ERR_UNSUPPORTED   -7   /* valid codes, but this combination of layouts is not implemented */
+#define JF_ERR_SCRATCH_LIMIT -8   /* jf_igemm_block_fp_noalloc: the K split needs more than JF_NOALLOC_SCRATCH_BYTES */
 
 /* A operand layout of jf_igemm_block_fp (every other GEMM entry point takes A as [M,K]) */
 #define JF_A_MK 0                 /* A is [M,K] row-major                                                          */
@@ -105,6 +106,19 @@ size_t jf_igemm_block_fp_workspace_bytes(int M, int N, int K, int b_layout, int 
 int jf_igemm_block_fp(const int8_t *A, const int8_t *B, const void *sa, const void *sb, void *C,
                       int M, int N, int K, int a_layout, int b_layout, int scale_dtype, int sa_layout, int sb_layout,
                       int out_dtype, int splitk, void *workspace, size_t workspace_bytes, jf_stream_t stream);
+
+/* jf_igemm_block_fp for callers that cannot allocate or pass device scratch: code under HIP graph capture, tight serving
+ * loops, harnesses that forbid hipMalloc.  No counterpart in the reference.  Same arguments, same arithmetic and the
+ * same bits as jf_igemm_block_fp with the same splitk request, minus the workspace: the fp32 partial results of the K
+ * split live in a buffer built into the library (JF_NOALLOC_SCRATCH_BYTES per GPU the library runs on, held until the
+ * process ends).  Calls nothing that allocates or frees.  A problem whose K split needs more scratch
+ * (parts * M * N * 4 bytes, see jf_igemm_splitk_plan) is refused with JF_ERR_SCRATCH_LIMIT; splitk = 1 never needs any.
+ * All calls on one GPU share that GPU's buffer: two calls that may overlap on one GPU (different streams, or threads
+ * without ordering between them) race on it and must be serialised by the caller. */
+#define JF_NOALLOC_SCRATCH_BYTES (64u << 20)
+int jf_igemm_block_fp_noalloc(const int8_t *A, const int8_t *B, const void *sa, const void *sb, void *C,
+                              int M, int N, int K, int a_layout, int b_layout, int scale_dtype, int sa_layout,
+                              int sb_layout, int out_dtype, int splitk, jf_stream_t stream);
 
 /* (C_s8[M,N], sc[M/32,N/32]) = per-32x32-block requantisation of the same accumulation.
  *   rounding JF_ROUND_NEAREST : q = clamp(rn(127*(acc+bias[n]) / (amax+biasmax)), +-127)

@@ -877,6 +877,7 @@ const char *jf_error_string(int code)
     case JF_ERR_WORKSPACE: return "jetfire_hip: workspace missing or too small";
     case JF_ERR_DEVICE: return "jetfire_hip: device is not gfx950";
     case JF_ERR_UNSUPPORTED: return "jetfire_hip: this combination of operand layouts is not implemented";
+    case JF_ERR_SCRATCH_LIMIT: return "jetfire_hip: the K split of this problem needs more than the built-in scratch buffer (JF_NOALLOC_SCRATCH_BYTES); use jf_igemm_block_fp with a workspace, or splitk = 1";
     default: return code > 0 ? hipGetErrorString((hipError_t)code) : "jetfire_hip: unknown error";
     }
 }
@@ -991,6 +992,52 @@ int jf_igemm_block_fp(const int8_t *A, const int8_t *B, const void *sa, const vo
         return JF_ERR_WORKSPACE;
     return block_fp_run(A, B, sa, sb, C, M, N, K, a_layout, b_layout, scale_dtype, sa_layout, sb_layout, out_dtype, splits,
                         kb_per, workspace, (hipStream_t)stream);
+}
+
+// ---- the allocation-free weight-gradient entry point ---------------------------------------------------------------
+// Scratch of the K split, for callers that cannot hand over a workspace: one array per device, resident until the
+// process ends.  In host code `noalloc_scratch` is only a handle; the device address is looked up once per device.
+}  // extern "C"
+static __device__ __align__(256) unsigned char noalloc_scratch[JF_NOALLOC_SCRATCH_BYTES];
+namespace {
+std::mutex noalloc_mu;
+void *noalloc_ptr[jf::MAX_DEVICES] = {};                       // device address of noalloc_scratch, per device
+// rc = 0 and *out = this device's copy of the array (looked up on the first call on the device, with it current)
+int noalloc_scratch_of_current_device(void **out)
+{
+    int dev = 0;
+    if (hipGetDevice(&dev) != hipSuccess || dev < 0 || dev >= jf::MAX_DEVICES) return JF_ERR_DEVICE;
+    std::lock_guard<std::mutex> g(noalloc_mu);
+    if (!noalloc_ptr[dev]) {
+        void *ptr = nullptr;
+        hipError_t e = hipGetSymbolAddress(&ptr, HIP_SYMBOL(noalloc_scratch));
+        if (e != hipSuccess) return (int)e;
+        if (!ptr) return JF_ERR_DEVICE;
+        noalloc_ptr[dev] = ptr;
+    }
+    *out = noalloc_ptr[dev];
+    return JF_OK;
+}
+}  // namespace
+extern "C" {
+
+int jf_igemm_block_fp_noalloc(const int8_t *A, const int8_t *B, const void *sa, const void *sb, void *C,
+                              int M, int N, int K, int a_layout, int b_layout, int scale_dtype, int sa_layout,
+                              int sb_layout, int out_dtype, int splitk, jf_stream_t stream)
+{
+    int rc = block_fp_check(A, B, sa, sb, C, M, N, K, a_layout, b_layout, scale_dtype, out_dtype);
+    if (rc) return rc;
+    int splits = 1, kb_per = 0;
+    if ((rc = jf_igemm_splitk_plan(M, N, K, splitk, &splits, &kb_per))) return rc;
+    void *partials = nullptr;
+    if (splits > 1) {
+        if ((size_t)splits * (size_t)M * (size_t)N * sizeof(float) > (size_t)JF_NOALLOC_SCRATCH_BYTES) return JF_ERR_SCRATCH_LIMIT;
+        if ((rc = noalloc_scratch_of_current_device(&partials))) return rc;
+    }
+    // nothing in the scratch has to start at zero: every part stores its whole [M][N] partial result before the
+    // reduction reads it, so what an earlier (larger) call left behind is never read
+    return block_fp_run(A, B, sa, sb, C, M, N, K, a_layout, b_layout, scale_dtype, sa_layout, sb_layout, out_dtype, splits,
+                        kb_per, partials, (hipStream_t)stream);
 }
 
 int jf_igemm_block_q(const int8_t *A, const int8_t *B, const void *sa, const void *sb,

@@ -26,7 +26,7 @@ GELU_ERF, GELU_TANH = 0, 1
 
 EXPORTS = [
     "jf_error_string", "jf_igemm_workspace_bytes", "jf_igemm_s32", "jf_igemm_block_acc", "jf_igemm_block_fp",
-    "jf_igemm_splitk_plan", "jf_igemm_block_fp_workspace_bytes", "jf_igemm_block_q_gelu",
+    "jf_igemm_splitk_plan", "jf_igemm_block_fp_workspace_bytes", "jf_igemm_block_q_gelu", "jf_igemm_block_fp_noalloc",
     "jf_igemm_block_q", "jf_quantize", "jf_dequantize", "jf_transpose_s8", "jf_rowstats", "jf_layernorm_fwd",
     "jf_layernorm_bwd_workspace_bytes", "jf_layernorm_bwd", "jf_gelu_fwd", "jf_gelu_bwd", "jf_add", "jf_calibrate",
 ]
@@ -49,6 +49,7 @@ def lib():
         L.jf_igemm_s32.argtypes = [_p, _p, _p, _i, _i, _i, _i, _p, _sz, _p]
         L.jf_igemm_block_acc.argtypes = [_p, _p, _p, _i, _i, _i, _i, _p, _sz, _p]
         L.jf_igemm_block_fp.argtypes = [_p, _p, _p, _p, _p, _i, _i, _i, _i, _i, _i, _i, _i, _i, _i, _p, _sz, _p]
+        L.jf_igemm_block_fp_noalloc.argtypes = [_p, _p, _p, _p, _p, _i, _i, _i, _i, _i, _i, _i, _i, _i, _i, _p]
         L.jf_igemm_block_q_gelu.argtypes = [_p, _p, _p, _p, _p, _p, _p, _p, _p, _p, _i, _i, _i, _i, _i, _i, _i, _f, _p]
         L.jf_igemm_splitk_plan.argtypes = [_i, _i, _i, _i, C.POINTER(C.c_int), C.POINTER(C.c_int)]
         L.jf_igemm_block_fp_workspace_bytes.argtypes = [_i, _i, _i, _i, _i]
@@ -221,6 +222,23 @@ def igemm_block_fp(A, B, sa, sb, b_layout=B_KN, out_dtype=torch.float16, a_layou
     out = torch.empty((M, N), dtype=out_dtype, device=A.device)
     check(lib().jf_igemm_block_fp(_ptr(A), _ptr(B), _ptr(sa), _ptr(sb), _ptr(out), M, N, K, a_layout, b_layout, code, la,
                                   lb, _FP_CODE[out_dtype], splitk, _ptr(ws), nb, _stream()))
+    return out
+
+
+NOALLOC_SCRATCH_BYTES = 64 << 20
+
+
+def igemm_block_fp_noalloc(A, B, sa, sb, out, b_layout=B_KN, a_layout=A_MK, splitk=1):
+    """igemm_block_fp into a caller-supplied `out` ([M,N] float16 / float32 / bfloat16) through the entry point that
+    neither takes nor allocates scratch (the K split uses the library's built-in buffer); this wrapper allocates
+    nothing either.  Refuses K splits that need more than NOALLOC_SCRATCH_BYTES."""
+    M, N, K, _, _ = _gemm_operands(A, B, b_layout, a_layout)
+    code, la, lb = _gemm_scales(sa, sb, M, N, K)
+    _need(out, None, "out")
+    if tuple(out.shape) != (M, N) or out.dtype not in _FP_CODE or out.device != A.device:
+        raise RuntimeError(f"out: expected a float [M,N]={M, N} tensor on {A.device}")
+    check(lib().jf_igemm_block_fp_noalloc(_ptr(A), _ptr(B), _ptr(sa), _ptr(sb), _ptr(out), M, N, K, a_layout, b_layout,
+                                          code, la, lb, _FP_CODE[out.dtype], splitk, _stream()))
     return out
 
 

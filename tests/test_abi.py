@@ -50,3 +50,7 @@ def test_argument_errors_without_gpu(jf):
         assert L.jf_quantize(p, 1, 32, 32, p, p, None, 0, 0, 0, 0, 0.0, None) == -6
         assert b"gfx950" in L.jf_error_string(-6)
     assert L.jf_gelu_fwd(p, p, 32, 32, 0, 5, 0.0, p, p, None) == -3
+    # the allocation-free weight-gradient entry point refuses a K split that does not fit its built-in scratch buffer
+    # (16 parts of 1600 x 1600 fp32 = 164 MB) before it touches the device
+    assert L.jf_igemm_block_fp_noalloc(p, p, p, p, p, 1600, 1600, 8192, 0, 1, 1, 0, 0, 1, 16, None) == -8
+    assert b"scratch" in L.jf_error_string(-8)
