@@ -12,7 +12,6 @@
 #include <c10/core/DeviceGuard.h>
 #include <c10/hip/HIPStream.h>
 
-#include <atomic>
 #include <mutex>
 #include <tuple>
 
@@ -131,53 +130,48 @@ struct Workspace {
     }
 };
 
-// (seed, offset) of the next stochastic kernel: the seed follows torch.manual_seed (default GPU generator),
-// the offset counts Philox calls handed out by this process.  (Reference: rand(), …Stochastic.cu:416.)
-struct PhiloxState {
-    std::mutex mu;
-    uint64_t seed = 0, offset = 0;
-    bool have = false;
-};
-PhiloxState &philox_state()
+// (seed, offset) of the next stochastic kernel.  There is ONE source of Philox counters per device for everything in
+// this library that rounds stochastically (these GEMMs and the Nonlinear operators, which reach it from Python): the
+// device's default torch generator.  An op reserves the counters it may consume (one per 8 output elements) by advancing
+// the generator's offset under the generator's mutex, so consecutive ops draw from disjoint ranges, torch.manual_seed
+// (also with the seed it already has) rewinds everything, and torch's own random kernels never see a counter twice.
+// The generator refuses this during stream capture: a captured graph would replay the same noise, so code that is
+// captured passes explicit (seed, offset) through the C ABI instead.  (Reference: rand(), ...Stochastic.cu:416.)
+at::Generator default_generator(int device_index)
 {
-    static PhiloxState s;
-    return s;
+    return at::detail::getCUDAHooks().getDefaultGenerator(device_index);
 }
 
-uint64_t generator_seed(int device_index)
+uint64_t reserve_calls(int64_t numel)
 {
-    at::Generator gen = at::detail::getCUDAHooks().getDefaultGenerator(device_index);
-    std::lock_guard<std::mutex> g(gen.mutex());
-    return gen.current_seed();
+    const uint64_t calls = (uint64_t)(numel + 7) / 8;
+    return (calls + 3) / 4 * 4;                                // the generator keeps its offset a multiple of 4
 }
 
 std::pair<uint64_t, uint64_t> next_philox(const torch::Tensor &t, int64_t numel)
 {
-    const uint64_t seed = generator_seed(t.device().index());
-    PhiloxState &ps = philox_state();
-    std::lock_guard<std::mutex> g(ps.mu);
-    if (!ps.have || seed != ps.seed) { ps.seed = seed; ps.offset = 0; ps.have = true; }
-    const uint64_t off = ps.offset;
-    ps.offset += (uint64_t)(numel + 7) / 8;
+    at::Generator gen = default_generator(t.device().index());
+    std::lock_guard<std::mutex> g(gen.mutex());
+    const uint64_t seed = gen.current_seed(), off = gen.get_offset();
+    gen.set_offset(off + reserve_calls(numel));
     return {seed, off};
 }
 
 // For reproducible tests: the (seed, offset) the next stochastic call on `device_index` will use, and a way
-// to place the offset.
+// to place the offset (a multiple of 4).
 std::tuple<uint64_t, uint64_t> philox_peek(int device_index)
 {
-    const uint64_t seed = generator_seed(device_index);
-    PhiloxState &ps = philox_state();
-    std::lock_guard<std::mutex> g(ps.mu);
-    return std::make_tuple(seed, (ps.have && seed == ps.seed) ? ps.offset : (uint64_t)0);
+    at::Generator gen = default_generator(device_index);
+    std::lock_guard<std::mutex> g(gen.mutex());
+    return std::make_tuple(gen.current_seed(), gen.get_offset());
 }
 
 void philox_set_offset(int device_index, uint64_t offset)
 {
-    const uint64_t seed = generator_seed(device_index);
-    PhiloxState &ps = philox_state();
-    std::lock_guard<std::mutex> g(ps.mu);
-    ps.seed = seed; ps.offset = offset; ps.have = true;
+    TORCH_CHECK(offset % 4 == 0, "the Philox offset must be a multiple of 4, got ", offset);
+    at::Generator gen = default_generator(device_index);
+    std::lock_guard<std::mutex> g(gen.mutex());
+    gen.set_offset(offset);
 }
 
 std::tuple<torch::Tensor, torch::Tensor> block_q(const torch::Tensor &X, const torch::Tensor &W, const torch::Tensor *bias,

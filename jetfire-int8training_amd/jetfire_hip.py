@@ -119,28 +119,34 @@ def _mult32(*dims):
 
 # ------------------------------------------------------------------------------------------------ RNG
 class _Philox:
-    """(seed, offset) for the stochastic-rounding kernels.  The seed follows torch.manual_seed; the
-    offset advances by the number of Philox calls an op may consume, so a program is reproducible."""
+    """(seed, offset) for the stochastic-rounding kernels: reserved from the device's default torch generator (the one
+    source of Philox counters for every stochastic op of this library, the GEMM extension included), one counter per 8
+    output elements.  Consecutive ops therefore draw disjoint counter ranges and torch.manual_seed (also with an
+    unchanged seed) rewinds them.  The generator refuses this during stream capture: captured code passes explicit
+    seed / offset arguments."""
 
-    def __init__(self):
-        self.seed = None
-        self.offset = 0
+    @staticmethod
+    def _gen(device):
+        idx = device.index if device.index is not None else torch.cuda.current_device()
+        return torch.cuda.default_generators[idx]
 
-    def next(self, numel):
-        s = torch.initial_seed() & 0xFFFFFFFFFFFFFFFF
-        if s != self.seed:
-            self.seed, self.offset = s, 0
-        off = self.offset
-        self.offset += (numel + 7) // 8
-        return self.seed, off
+    def peek(self, device):
+        g = self._gen(device)
+        return g.initial_seed() & 0xFFFFFFFFFFFFFFFF, g.get_offset()
+
+    def next(self, numel, device):
+        g = self._gen(device)
+        seed, off = g.initial_seed() & 0xFFFFFFFFFFFFFFFF, g.get_offset()
+        g.set_offset(off + ((numel + 7) // 8 + 3) // 4 * 4)
+        return seed, off
 
 
 philox = _Philox()
 
 
-def _rng(rounding, numel, seed, offset):
+def _rng(rounding, numel, seed, offset, device):
     if rounding in (ROUND_STOCHASTIC, ROUND_STOCHASTIC_TRUNC) and seed is None:
-        return philox.next(numel)
+        return philox.next(numel, device)
     return (seed or 0), (offset or 0)
 
 
@@ -272,7 +278,7 @@ def igemm_block_q(A, B, sa, sb, b_layout=B_KN, bias=None, biasmax=None, rounding
         _need(biasmax, torch.float32, "biasmax", None)
     if rounding not in (ROUND_NEAREST, ROUND_STOCHASTIC):
         raise RuntimeError("rounding must be ROUND_NEAREST or ROUND_STOCHASTIC")
-    seed, offset = _rng(rounding, M * N, seed, offset)
+    seed, offset = _rng(rounding, M * N, seed, offset, A.device)
     out = torch.empty((M, N), dtype=torch.int8, device=A.device)
     sc = torch.empty((M // QB, N // QB), dtype=sa.dtype, device=A.device)
     check(lib().jf_igemm_block_q(_ptr(A), _ptr(B), _ptr(sa), _ptr(sb), _ptr(bias), _ptr(biasmax), _ptr(out), _ptr(sc),
@@ -287,7 +293,7 @@ def quantize(x, rounding=ROUND_NEAREST, scale_dtype=torch.float16, transpose=Fal
         raise RuntimeError(f"x: unsupported dtype {x.dtype}")
     R, Cc = x.shape
     _mult32(R, Cc)
-    seed, offset = _rng(rounding, R * Cc, seed, offset)
+    seed, offset = _rng(rounding, R * Cc, seed, offset, x.device)
     q = torch.empty((R, Cc), dtype=torch.int8, device=x.device)
     s = torch.empty((R // QB, Cc // QB), dtype=scale_dtype, device=x.device)
     qT = torch.empty((Cc, R), dtype=torch.int8, device=x.device) if transpose else None
@@ -362,7 +368,7 @@ def layernorm_bwd(qx, sx, qg, sg, gamma, mean, rstd, rounding=ROUND_NEAREST, wan
     _vec(gamma, Cc, "gamma")
     _vec(mean, R, "mean")
     _vec(rstd, R, "rstd")
-    seed, offset = _rng(rounding, R * Cc, seed, offset)
+    seed, offset = _rng(rounding, R * Cc, seed, offset, qx.device)
     nbytes = lib().jf_layernorm_bwd_workspace_bytes(R, Cc)
     ws = torch.empty(nbytes, dtype=torch.int8, device=qx.device)
     qdx = torch.empty_like(qx)
@@ -388,7 +394,7 @@ def gelu_bwd(qx, sx, qg, sg, approx=GELU_ERF, rounding=ROUND_NEAREST, seed=None,
     R2, C2, code2 = _block_tensor(qg, sg, "g")
     if (R2, C2, code2) != (R, Cc, code):
         raise RuntimeError("x and g must have the same shape and scale dtype")
-    seed, offset = _rng(rounding, R * Cc, seed, offset)
+    seed, offset = _rng(rounding, R * Cc, seed, offset, qx.device)
     qy = torch.empty_like(qx)
     sy = torch.empty_like(sx)
     check(lib().jf_gelu_bwd(_ptr(qx), _ptr(sx), _ptr(qg), _ptr(sg), R, Cc, code, approx, rounding, seed, offset,
@@ -401,7 +407,7 @@ def add(x1, q2, s2, rounding=ROUND_TRUNC, with_stats=False, seed=None, offset=No
     _need(x1, None, "x1")
     if x1.dtype not in _FP_CODE or tuple(x1.shape) != (R, Cc):
         raise RuntimeError("x1 must be a float tensor of the same shape as x2")
-    seed, offset = _rng(rounding, R * Cc, seed, offset)
+    seed, offset = _rng(rounding, R * Cc, seed, offset, x1.device)
     y1 = torch.empty((R, Cc), dtype=torch.float32, device=x1.device)
     q = torch.empty_like(q2)
     s = torch.empty_like(s2)

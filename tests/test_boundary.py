@@ -286,3 +286,57 @@ def test_nonlinear_package_3d(oracle):
     assert tuple(t2.shape) == (C, BS * T)
     t3 = int8_transpose(qx)
     assert t3.dim() == 3 and t3.shape[0] == BS and t3.shape[-1] == BS * T     # 3-D when not asked for 2-D
+
+
+@pytest.mark.gpu
+def test_stochastic_ops_share_one_counter_source(oracle):
+    """The Nonlinear operators (ctypes binding) and the GEMM extension reserve their Philox counters from the same place,
+    the device's torch generator: consecutive stochastic ops of a backward pass get disjoint counter ranges, and
+    torch.manual_seed rewinds them, also when called with the seed that is already set."""
+    from Linear import int8_linear_backward
+    from Nonlinear import int8_gelu_backward, int8_quantize
+    import BlockQuantizeCUDA as BQC
+    import jetfire_hip as jf
+    BS, T, Cin, Cout = 1, 256, 96, 160
+    gsrc = torch.Generator().manual_seed(5)
+    x = torch.randn(BS, T, Cin, generator=gsrc).cuda()
+    w = (torch.randn(Cout, Cin, generator=gsrc) * 0.02).cuda()
+    g = (torch.randn(BS, T, Cout, generator=gsrc) * 1e-3).cuda()
+    qx, sx = int8_quantize(x, 32)
+    qw, sw = int8_quantize(w, 32)
+
+    def backward():
+        spans = []
+        seed, off = BQC.philox_peek(0)
+        qg, sg = int8_quantize(g, 32, stochastic=True)             # Nonlinear: counters [off, off + T*Cout/8)
+        spans.append((off, T * Cout // 8))
+        assert jf.philox.peek(qg.device) == BQC.philox_peek(0)     # both bindings look at the same state
+        seed2, off2 = BQC.philox_peek(0)
+        gx8, gsx, gw = int8_linear_backward(qx, sx, qg, sg, None, qw, sw, 32)   # extension: the dgrad GEMM
+        spans.append((off2, T * Cin // 8))
+        seed3, off3 = BQC.philox_peek(0)
+        d8, ds = int8_gelu_backward(gx8, gsx, gx8, gsx, 32, stochastic=True)    # Nonlinear again
+        spans.append((off3, T * Cin // 8))
+        assert seed == seed2 == seed3
+        return spans, (qg, sg, gx8, gsx, d8, ds), (seed, off, off2)
+
+    torch.manual_seed(77)
+    spans, first, (seed, off, off2) = backward()
+    assert seed == 77 and off == 0
+    for (a, n), (b, _) in zip(spans, spans[1:]):
+        assert b >= a + n, f"counter ranges overlap: {spans}"
+    # each op used exactly the counters it reserved: the oracle reproduces it from (seed, offset)
+    wq, ws = oracle.quantize(g.reshape(-1, Cout).cpu().numpy(), stochastic=True, seed=seed, offset=off, scale_dtype="f16")
+    assert np.array_equal(first[0].reshape(-1, Cout).cpu().numpy(), wq)
+    sg2 = first[1].reshape(-1, Cout // 32).float().cpu().numpy()
+    wq, ws = oracle.igemm_block_q(first[0].reshape(-1, Cout).cpu().numpy(), qw.cpu().numpy(), np.ascontiguousarray(sg2.T),
+                                  sw.float().cpu().numpy(), 1, stochastic=True, seed=seed, offset=off2, scale_dtype="f16")
+    assert np.array_equal(first[2].reshape(-1, Cin).cpu().numpy(), wq)
+    second_spans, second, _ = backward()                          # no re-seed: fresh counters, different noise
+    assert second_spans[0][0] >= spans[-1][0] + spans[-1][1]
+    assert not torch.equal(second[0], first[0])
+    torch.manual_seed(77)                                          # same seed again: the stream rewinds
+    again_spans, again, _ = backward()
+    assert again_spans == spans
+    for a, b in zip(first, again):
+        assert torch.equal(a, b)
