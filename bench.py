@@ -8,8 +8,9 @@ wgrad GEMM (fp16 output) -- 12 fused per-block INT8 GEMMs, 1.51e12 integer ops. 
 quantised once, outside the timed region, and stay resident in HBM.
 
 Prints ONE JSON line: whole-step throughput as `value` (tera-ops/s), the roofline of the dominant
-kernel (igemm_nt_kernel, measured live with events on the launch stream) and a CPU baseline (the CPU
-checker under oracle/ timed on this host's cores on a bounded slice of the same workload).
+kernel (igemm_nt_kernel, measured live with events on the launch stream) and a CPU baseline (a PyTorch
+emulation of the same arithmetic, and the C restatement under oracle/, timed on this host's cores on a
+bounded slice of the same workload).
 """
 import argparse
 import json
@@ -24,7 +25,11 @@ for p in (ROOT, PKG):
         sys.path.insert(0, p)
 
 INT8_PEAK_TOPS = 5000.0      # MI355X dense INT8 MFMA peak, tera-ops/s
-MEASURED_TRAFFIC_BYTES = 150.2e6   # fc forward GEMM: 97.3 MB fetched + 52.8 MB written per launch (counter run)
+# HBM-side bytes per launch of the fc forward GEMM, from the rocprofv3 --pmc runs summarised in
+# profiles/igemm_fc_forward_pmc.md (FETCH_SIZE and WRITE_SIZE, each scaled by a copy of known size): a property of the
+# kernel, carried over from that profile, not re-measured by this run (counters need the profiler attached)
+PROFILED_TRAFFIC_BYTES = 150.2e6
+PROFILED_TRAFFIC_SOURCE = "profiles/igemm_fc_forward_pmc.md (97.3 MB fetched + 52.8 MB written; algorithmic 75.9 MB)"
 TOKENS = 8192
 LAYERS = [("qkv", 1600, 4800), ("proj", 1600, 1600), ("fc", 1600, 6400), ("fc2", 6400, 1600)]
 
@@ -52,12 +57,14 @@ def make_inputs(jf, torch, seed=0):
 
 def step(jf, torch, ops, it):
     outs = []
+    offset = it * (sum(TOKENS * o["cin"] for o in ops) // 8)      # every dgrad launch of the run draws its own counters
     for o in ops:
         # forward  Y = X W^T           (M,N,K) = (T, cout, cin), B = W as [N,K]
         outs.append(jf.igemm_block_q(o["qx"], o["qw"], o["sxT"], o["swT"], jf.B_NK))
         # dgrad    dX = dY W           (T, cin, cout), B = W as [K,N], stochastic rounding
         outs.append(jf.igemm_block_q(o["qg"], o["qw"], o["sgT"], o["sw"], jf.B_KN, rounding=jf.ROUND_STOCHASTIC,
-                                     seed=1234, offset=it * 7))
+                                     seed=1234, offset=offset))
+        offset += TOKENS * o["cin"] // 8
         # wgrad    dW = dY^T X         (cout, cin, T), A = dY^T, B = X as [K,N], fp16 out
         outs.append(jf.igemm_block_fp(o["qgT"], o["qx"], o["sg"], o["sx"], jf.B_KN, torch.float16))
     return outs
@@ -67,7 +74,7 @@ def step_ops():
     return sum(3 * 2 * TOKENS * cin * cout for _, cin, cout in LAYERS)
 
 
-def dominant_kernel_roofline(jf, torch, ops, iters=20):
+def dominant_kernel_roofline(jf, torch, ops, iters=200):
     """igemm_nt_kernel on the fc forward GEMM (8192 x 6400 x 1600, both operands K-contiguous, so the call is
     exactly one launch of that kernel): average launch duration from events on the launch stream."""
     o = ops[2]
@@ -85,9 +92,7 @@ def dominant_kernel_roofline(jf, torch, ops, iters=20):
     return {"bound": "mfma", "kernel": "igemm_nt_kernel<EPI_Q,f32> fc forward 8192x6400x1600",
             "achieved": round(achieved, 2), "peak": INT8_PEAK_TOPS, "unit": "TOP/s",
             "frac": round(achieved / INT8_PEAK_TOPS, 4), "avg_launch_us": round(avg_s * 1e6, 2),
-            # HBM-side bytes per launch from rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE (profiles/igemm_fc_forward_pmc.md);
-            # algorithmic minimum is 75.9 MB (A + W + C)
-            "traffic": MEASURED_TRAFFIC_BYTES}
+            "launches": iters, "traffic": PROFILED_TRAFFIC_BYTES, "traffic_source": PROFILED_TRAFFIC_SOURCE}
 
 
 def fused_fc_gelu(jf, torch, ops):
@@ -246,17 +251,27 @@ def nonlinear_extras(jf, torch):
 
 
 def calibration(jf, torch):
-    """Register-only loops: what the matrix pipe and the vector ALU deliver alone and together on this part."""
-    simds = torch.cuda.get_device_properties(0).multi_processor_count * 4
-    out = {}
-    t, n = jf.calibrate(1, 0)
-    out["mfma_only_TOPs"] = round(n * 65536 / t / 1e12, 1)
-    out["mfma_only_ns_per_mfma_per_simd"] = round(t * 1e9 * simds / n, 2)
-    t, n = jf.calibrate(0, 32)
-    out["valu_32fmac_ns_per_simd"] = round(t * 1e9 * simds / n, 2)
-    t, n = jf.calibrate(1, 32)
-    out["mfma_plus_32fmac_ns_per_simd"] = round(t * 1e9 * simds / n, 2)
-    out["mfma_plus_32fmac_TOPs"] = round(n * 65536 / t / 1e12, 1)
+    """Register-only loops: what the matrix pipe and the vector ALU deliver alone, together in one wave, together from
+    separate waves of one SIMD, and on the GEMM's real K-block instruction stream, at 1 / 2 / 4 waves per SIMD, in
+    nanoseconds and in shader cycles (with the clock the kernel ran at) per work item and SIMD."""
+    out = {"unit": "per 32x32x32 work item and SIMD", "rows": []}
+
+    def row(name, *a, **kw):
+        r = jf.calibrate(*a, **kw)
+        ns = r["seconds"] * 1e9 * r["simds"] / r["items"]
+        out["rows"].append({"case": name, "waves_per_simd": r["waves_per_simd"], "ns": round(ns, 2),
+                            "cycles": round(ns * r["shader_MHz"] * 1e-3, 1), "shader_MHz": round(r["shader_MHz"])})
+        return ns
+
+    for wpc in (1, 2, 4):                                         # 256-thread workgroups: one wave per SIMD each
+        row("mfma_only", 1, 0, workgroups_per_cu=wpc)
+        row("valu_32fmac_only", 0, 32, workgroups_per_cu=wpc)
+        both = row("mfma_and_32fmac_same_wave", 1, 32, workgroups_per_cu=wpc)
+        stream = row("gemm_k_block_stream", 1, 32, workgroups_per_cu=wpc, mode=jf.CAL_STREAM)
+    for wpc in (1, 2):                                            # 512-thread workgroups: waves w and w+4 share a SIMD
+        row("mfma_and_32fmac_separate_waves", 1, 32, workgroups_per_cu=wpc, threads=512, mode=jf.CAL_SPLIT)
+    out["ceiling_TOPs_independent"] = round(65536 / both * 1e9 * 1024 / 1e12, 1)
+    out["ceiling_TOPs_k_block_stream"] = round(65536 / stream * 1e9 * 1024 / 1e12, 1)
     a = torch.randn(TOKENS, 1600, device="cuda", dtype=torch.bfloat16)
     b = torch.randn(6400, 1600, device="cuda", dtype=torch.bfloat16)
     for _ in range(5):
@@ -268,8 +283,59 @@ def calibration(jf, torch):
     e1.record()
     torch.cuda.synchronize()
     out["torch_bf16_fc_forward_TFLOPs"] = round(2.0 * TOKENS * 6400 * 1600 * 20 / (e0.elapsed_time(e1) * 1e-3) / 1e12, 1)
-    out["note"] = ("per SIMD, 4 waves resident; the scale-accumulate needs 32 VALU instructions per MFMA, and the two "
-                   "pipes add up rather than overlap: the last line is the ceiling of any exact per-block kernel")
+    out["note"] = ("the exact fp32 scale-accumulate needs 32 VALU instructions per MFMA; with two or more waves per SIMD "
+                   "the times of the two pipes add (in cycles, not through a clock drop), also when they come from "
+                   "separate waves: the two ceilings are what any kernel with these semantics can reach at 4 waves per SIMD")
+    return out
+
+
+def timed_us(torch, fn, n, warm=3):
+    for _ in range(warm):
+        fn()
+    torch.cuda.synchronize()
+    e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+    e0.record()
+    for _ in range(n):
+        fn()
+    e1.record()
+    torch.cuda.synchronize()
+    return e0.elapsed_time(e1) * 1e3 / n
+
+
+def other_configurations(jf, torch):
+    """Absolute TOP/s and fraction of the dense INT8 peak for the two other GEMM configurations: the GPT-2 small linear
+    set (12288 tokens; forward, dgrad with stochastic rounding, wgrad) and the 8192^3 stress GEMM with requantised
+    output in deterministic and stochastic mode (synthetic data of the configurations' distributions, fp32 scales)."""
+    out = {}
+    g = torch.Generator().manual_seed(0)
+    T = 12288
+    layers = []
+    for name, cin, cout in (("qkv", 768, 2304), ("proj", 768, 768), ("fc", 768, 3072), ("fc2", 3072, 768)):
+        qx, sx = jf.quantize(torch.randn(T, cin, generator=g).cuda(), scale_dtype=torch.float32)
+        qw, sw = jf.quantize((torch.randn(cout, cin, generator=g) * 0.02).cuda(), scale_dtype=torch.float32)
+        qg, sg = jf.quantize((torch.randn(T, cout, generator=g) * 1e-3).cuda(), jf.ROUND_STOCHASTIC, torch.float32, seed=0, offset=0)
+        layers.append((name, cin, cout, qx, sx, qw, sw, qg, sg))
+
+    def small_step():
+        for name, cin, cout, qx, sx, qw, sw, qg, sg in layers:
+            jf.igemm_block_q(qx, qw, sx.t(), sw.t(), jf.B_NK)
+            jf.igemm_block_q(qg, qw, sg.t(), sw, jf.B_KN, rounding=jf.ROUND_STOCHASTIC, seed=1, offset=0)
+            jf.igemm_block_fp(qg, qx, sg, sx, jf.B_KN, torch.float16, a_layout=jf.A_KM, splitk=0)
+    us = timed_us(torch, small_step, 50)
+    nops = sum(3 * 2.0 * T * cin * cout for _, cin, cout, *_ in layers)
+    out["gpt2_small_set_12288_tokens"] = {"us_per_set": round(us, 1), "TOP/s": round(nops / us / 1e6, 1),
+                                          "frac_of_int8_peak": round(nops / us / 1e6 / INT8_PEAK_TOPS, 4),
+                                          "wgrad": "gradient read in place, library K split"}
+    del layers
+    n = 8192
+    a = torch.randn(n, n, generator=g) / torch.sqrt(torch.randn(3, n, n, generator=g).pow_(2).mean(0))   # Student-t, 3 dof
+    qa, sa = jf.quantize(a.cuda(), scale_dtype=torch.float32)
+    del a
+    qb, sb = jf.quantize((torch.randn(n, n, generator=g) * 0.02).cuda(), scale_dtype=torch.float32)
+    for key, kw in (("deterministic", {}), ("stochastic", dict(rounding=jf.ROUND_STOCHASTIC, seed=5, offset=11))):
+        us = timed_us(torch, lambda: jf.igemm_block_q(qa, qb, sa.t(), sb.t(), jf.B_NK, **kw), 30)
+        out[f"stress_8192_cubed_{key}"] = {"us": round(us, 1), "TOP/s": round(2.0 * n ** 3 / us / 1e6, 1),
+                                           "frac_of_int8_peak": round(2.0 * n ** 3 / us / 1e6 / INT8_PEAK_TOPS, 4)}
     return out
 
 
@@ -286,40 +352,100 @@ def pmc_probe(jf, torch, ops):
     torch.cuda.synchronize()
 
 
-def cpu_baseline(ops, rows=512):
-    """The CPU checker (scalar C restatement of the reference arithmetic, OpenMP over rows) on the first
-    `rows` token rows of the fc layer: forward + dgrad + the matching slice of wgrad work."""
+def _torch_emulation(torch, A8, B8_nk, sa_km, sb_km):
+    """The PyTorch emulation of the per-block linear forward on the host: per 32-deep K block an exact fp32 matmul of
+    the INT8 codes (32 * 127^2 < 2^24), scaled by the outer product of the two block-scale vectors, accumulated in
+    ascending K-block order; then absmax per 32x32 output block, q = clamp(round(127 * acc / amax)).  A8 [M,K] int8,
+    B8_nk [N,K] int8, sa_km [K/32, M/32], sb_km [K/32, N/32] fp32.  Returns (codes int8 [M,N], scales fp32)."""
+    M, K = A8.shape
+    N = B8_nk.shape[0]
+    acc = torch.zeros(M, N, dtype=torch.float32)
+    for kb in range(K // 32):
+        d = A8[:, kb * 32:(kb + 1) * 32].float() @ B8_nk[:, kb * 32:(kb + 1) * 32].float().t()
+        sab = sa_km[kb].repeat_interleave(32)[:, None] * sb_km[kb].repeat_interleave(32)[None, :]
+        acc += sab * d
+    blocks = acc.view(M // 32, 32, N // 32, 32)
+    amax = blocks.abs().amax(dim=(1, 3), keepdim=True)
+    q = torch.where(amax > 0, torch.round(127.0 * blocks / amax), torch.zeros(())).clamp_(-127, 127)
+    return q.to(torch.int8).view(M, N), (amax / 127.0).view(M // 32, N // 32)
+
+
+def cpu_baseline(ops, rows):
+    """The CPU path beside the GPU numbers, on this host's cores.  `value`: the PyTorch emulation (all torch threads) on
+    the four forward GEMMs of the timed step restricted to their first `rows` token rows (a bounded sample of the workload).
+    Next to it: the same emulation on the 2048 x 768 x 768 seed-0 case (median of 3) with the number of INT8 codes in
+    which it differs from the canonical fused arithmetic (a separate multiply and add round differently from an fma),
+    and the C restatement under oracle/ (OpenMP) timed on the same two inputs."""
+    import platform
+    import statistics
     import numpy as np
+    import torch
     from oracle import oracle as O
     threads = min(os.cpu_count() or 1, 16)
+    torch.set_num_threads(threads)
     O.set_threads(threads)
-    o = ops[2]
-    f = lambda t: np.ascontiguousarray(t.cpu().numpy())
-    qx, qw, qg = f(o["qx"][:rows]), f(o["qw"]), f(o["qg"][:rows])
-    sxT, swT, sgT, sw = f(o["sxT"][:, : rows // 32]), f(o["swT"]), f(o["sgT"][:, : rows // 32]), f(o["sw"])
-    qgT, sg, sx = f(o["qgT"][:, :rows]), f(o["sg"][: rows // 32]), f(o["sx"][: rows // 32])
+    model = platform.processor() or ""
+    try:
+        for line in open("/proc/cpuinfo"):
+            if line.startswith("model name"):
+                model = line.split(":", 1)[1].strip()
+                break
+    except OSError:
+        pass
+    cpu = lambda t: t.cpu().contiguous()
+    nops, dt, dt_oracle = 0.0, 0.0, 0.0
+    for o in ops:                                                  # the four forward GEMMs of the timed step
+        qx, qw, sxT, swT = cpu(o["qx"][:rows]), cpu(o["qw"]), cpu(o["sxT"][:, : rows // 32]), cpu(o["swT"])
+        nops += 2.0 * rows * o["cin"] * o["cout"]
+        t0 = time.perf_counter()
+        _torch_emulation(torch, qx, qw, sxT, swT)
+        dt += time.perf_counter() - t0
+        t0 = time.perf_counter()
+        O.igemm_block_q(qx.numpy(), qw.numpy(), sxT.numpy(), swT.numpy(), 0)
+        dt_oracle += time.perf_counter() - t0
+    out = {"value": round(nops / dt / 1e12, 5), "unit": "TOP/s", "cores": threads, "kind": "port",
+           "sample": f"PyTorch emulation of the four forward GEMMs of the step (qkv, proj, fc, fc2), first {rows} of 8192 "
+                     f"token rows, {nops:.3g} of the step's 1.51e12 ops in {dt:.1f} s, 1 run",
+           "cpu_model": model, "torch_version": torch.__version__,
+           "c_restatement_same_sample": {"TOP/s": round(nops / dt_oracle / 1e12, 5), "seconds": round(dt_oracle, 2), "threads": threads}}
+    # the 2048 x 768 x 768 case, seed 0
+    g = torch.Generator().manual_seed(0)
+    x = torch.randn(2048, 768, generator=g)
+    w = torch.randn(768, 768, generator=g) * 0.02
+    qx1, sx1 = O.quantize(x.numpy())
+    qw1, sw1 = O.quantize(w.numpy())
+    sx1T, sw1T = np.ascontiguousarray(sx1.T), np.ascontiguousarray(sw1.T)
+    tx = [torch.from_numpy(a) for a in (qx1, qw1, sx1T, sw1T)]
+    times = []
+    for _ in range(3):
+        t0 = time.perf_counter()
+        eq, es = _torch_emulation(torch, *tx)
+        times.append(time.perf_counter() - t0)
     t0 = time.perf_counter()
-    O.igemm_block_q(qx, qw, sxT, swT, 0)
-    O.igemm_block_q(qg, qw, sgT, sw, 1, stochastic=True, seed=1234, offset=0)
-    O.igemm_block_fp(qgT, qx, sg, sx, 1, "f16")
-    dt = time.perf_counter() - t0
-    nops = 3 * 2.0 * rows * o["cin"] * o["cout"]
-    return {"value": round(nops / dt / 1e12, 5), "unit": "TOP/s", "cores": threads, "kind": "port",
-            "sample": f"fc layer (1600->6400), first {rows} of 8192 token rows: forward + dgrad(SR) + wgrad slice, "
-                      f"{nops:.3g} ops in {dt:.1f} s"}
+    wq, ws = O.igemm_block_q(qx1, qw1, sx1T, sw1T, 0)
+    dt_oracle = time.perf_counter() - t0
+    uq, _ = O.requant(O.igemm_block_f32(qx1, qw1, sx1T, sw1T, 0, fused=False))
+    med = statistics.median(times)
+    out["case_2048x768x768_seed0"] = {
+        "emulation_ms_median_of_3": round(med * 1e3, 1), "emulation_TOP/s": round(2.0 * 2048 * 768 * 768 / med / 1e12, 5),
+        "c_restatement_ms": round(dt_oracle * 1e3, 1), "codes": int(wq.size),
+        "codes_emulation_differs_from_fused": int((eq.numpy() != wq).sum()),
+        "codes_unfused_restatement_differs_from_fused": int((uq != wq).sum())}
+    return out
 
 
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
-    ap.add_argument("--steps", type=int, default=20)
-    ap.add_argument("--warmup", type=int, default=3)
-    ap.add_argument("--cpu-rows", type=int, default=8192)
+    ap.add_argument("--steps", type=int, default=200)
+    ap.add_argument("--warmup", type=int, default=5)
+    ap.add_argument("--cpu-rows", type=int, default=8192, help="token rows of the fc forward GEMM the CPU baseline runs")
     ap.add_argument("--no-cpu", action="store_true")
     ap.add_argument("--no-extras", action="store_true")
     ap.add_argument("--pmc-probe", action="store_true", help="copy kernel + 3 GEMM launches only (for rocprofv3 --pmc)")
     ap.add_argument("--roofline-only", action="store_true", help="only the dominant-kernel measurement (for rocprofv3 --stats)")
     ap.add_argument("--extras-only", action="store_true", help="only the block-kernel section (for rocprofv3 --pmc)")
+    ap.add_argument("--calibration-only", action="store_true", help="only the register-only calibration loops")
     a = ap.parse_args()
     if a.gpus != 1:
         sys.exit("bench.py: this build measures one GPU only (--gpus 1); nothing here uses a second GPU")
@@ -330,6 +456,9 @@ def main():
     if not torch.cuda.is_available():
         sys.exit("bench.py: no GPU visible")
     torch.cuda.set_device(0)
+    if a.calibration_only:
+        print(json.dumps({"calibration": calibration(jf, torch)}))
+        return
     ops = make_inputs(jf, torch)
     if a.pmc_probe:
         pmc_probe(jf, torch, ops)
@@ -370,6 +499,7 @@ def main():
     }
     if not a.no_extras:
         out["calibration"] = calibration(jf, torch)
+        out["other_configurations"] = other_configurations(jf, torch)
         out["memory_bound_kernels"] = nonlinear_extras(jf, torch)
         out["deep_k_weight_gradients"] = deep_k_weight_gradients(jf, torch)
         out["fc_forward_with_gelu"] = fused_fc_gelu(jf, torch, ops)

@@ -199,11 +199,24 @@ int jf_add(const void *x1, int x1_dtype, const int8_t *q2, const void *s2, int R
            int scale_dtype, int rounding, uint64_t seed, uint64_t offset,
            float *y1, int8_t *q, void *s, float *rowsum, float *rowsq, jf_stream_t stream);
 
-/* Calibration (no counterpart in the reference; used by bench.py for the roofline discussion): launches
- * `workgroups` x 256 threads, each wave doing `iters` x 4 x ( [one 32x32x32 INT8 MFMA if with_mfma] + [valu_per_mfma
- * independent v_fmac_f32] ) from registers.  Supported (with_mfma, valu_per_mfma): (1,0) (0,32) (1,32) (0,16) (1,16).
- * `scratch` is a device buffer of at least 4 bytes (never written in practice). */
-int jf_calibrate(int with_mfma, int valu_per_mfma, int iters, int workgroups, float *scratch, jf_stream_t stream);
+/* Calibration (no counterpart in the reference; used by bench.py for the roofline discussion): launches `workgroups` x
+ * `threads` (128, 256, 384 or 512) threads; per iteration every wave runs 4 work items from registers, an item being
+ *   JF_CAL_UNIFORM: [one 32x32x32 INT8 MFMA if with_mfma] + [valu_per_mfma independent v_fmac_f32]
+ *                   supported (with_mfma, valu_per_mfma): (1,0) (0,32) (1,32) (0,16) (1,16);
+ *   JF_CAL_SPLIT:   the MFMA in the first half of a workgroup's waves, 32 v_fmac_f32 in the second half (1, 32): with
+ *                   512 threads the two kinds of wave share each SIMD;
+ *   JF_CAL_STREAM:  the GEMM's K-block instruction stream (1, 32): MFMA with the constant accumulator input, then 16
+ *                   subtractions and 16 v_fmac_f32 on the previous product.
+ * `scratch`: a device buffer of at least 4 bytes (never written in practice).  `clocks` (may be NULL): 2 x workgroups
+ * 64-bit words; workgroup w's first wave stores the shader-clock cycles and the wall-clock ticks (constant rate,
+ * hipDeviceAttributeWallClockRate) it ran for, which gives the clock the shader ran at under this load. */
+#define JF_CAL_UNIFORM 0
+#define JF_CAL_SPLIT   1
+#define JF_CAL_STREAM  2
+int jf_calibrate(int mode, int with_mfma, int valu_per_mfma, int iters, int workgroups, int threads, float *scratch,
+                 unsigned long long *clocks, jf_stream_t stream);
+/* Ticks per millisecond of the wall clock above on the current device (0 or negative: not available). */
+int jf_wall_clock_khz(void);
 
 #ifdef __cplusplus
 }

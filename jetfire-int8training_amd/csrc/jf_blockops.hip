@@ -123,8 +123,11 @@ __global__ __launch_bounds__(NT) void dequantize_kernel(const int8_t *q, const S
 }
 
 // A wave that loads one block (1 KiB of codes), waits, computes and stores keeps far too few bytes in flight to
-// cover the memory latency, so the GELU kernels run the block loop with the codes and scales of the next PF blocks
-// already requested.
+// cover the memory latency, so the streaming kernels run their block loop with the codes and scales of the next PF
+// blocks already requested.  The PF request slots are named at compile time (the loop body is unrolled PF times, slot
+// s serving the iterations s, s + PF, ...): moving the slots' registers down a queue instead would make every
+// iteration wait for ALL outstanding loads (a register cannot be copied before its load has landed), which is no
+// prefetch at all.
 constexpr int PF = 3;
 // Walks the blocks blk0, blk0 + stride, ... of a wave without a division per block: (row block, column block) advance
 // by (stride / SC, stride % SC) with a carry.
@@ -141,6 +144,28 @@ struct BlockWalk {
         if (cb >= SC) { cb -= SC; ++rb; }
     }
 };
+// body(walk, slot) for every block of the walk while walk.rb < RB; slot = iteration number mod PF as a compile-time
+// constant.  The body takes the slot's data and then refills the slot (the block PF iterations ahead).  Whole groups
+// of PF blocks run in a loop without exits inside it (so that the slots' registers are the loop's own, not copies
+// made on the way round); the last, partial group follows.
+template <typename Body> __device__ __forceinline__ void for_each_block_pipelined(BlockWalk w, int RB, int blk0, int stride, Body body)
+{
+    const int nblk = RB * w.SC;
+    const int n = blk0 < nblk ? (nblk - blk0 + stride - 1) / stride : 0;     // blocks of this wave (uniform)
+    for (int i = n / PF; i > 0; --i) {
+        static_for<0, PF>([&](auto slot_c) {
+            body(w, slot_c);
+            w.step();
+        });
+    }
+    const int rem = n % PF;
+    static_for<0, PF - 1>([&](auto slot_c) {
+        if (decltype(slot_c)::value < rem) {
+            body(w, slot_c);
+            w.step();
+        }
+    });
+}
 template <typename ST> struct CodeStream {
     const int8_t *q;
     const ST *s;
@@ -148,28 +173,42 @@ template <typename ST> struct CodeStream {
     BlockWalk at;                 // the next block to request
     v4i codes[PF];
     float scale[PF];
-    __device__ __forceinline__ void request(int slot)
+    template <int SLOT> __device__ __forceinline__ void request()
     {
         if (at.rb < RB) {
-            codes[slot] = *reinterpret_cast<const v4i *>(q + (size_t)(at.rb * QB + (lane >> 1)) * C + at.cb * QB + (lane & 1) * 16);
-            scale[slot] = load_scale(s, at.rb * at.SC + at.cb);
+            codes[SLOT] = *reinterpret_cast<const v4i *>(q + (size_t)(at.rb * QB + (lane >> 1)) * C + at.cb * QB + (lane & 1) * 16);
+            scale[SLOT] = load_scale(s, at.rb * at.SC + at.cb);
         }
         at.step();
     }
     __device__ __forceinline__ CodeStream(const int8_t *q_, const ST *s_, int R, int C_, int stride, int lane_, int blk0)
         : q(q_), s(s_), C(C_), RB(R / QB), lane(lane_), at(blk0, stride, C_ / QB)
     {
-#pragma unroll
-        for (int i = 0; i < PF; ++i) request(i);
+        static_for<0, PF>([&](auto i) { request<decltype(i)::value>(); });
     }
-    // hands out the oldest block and requests the one PF strides ahead
-    __device__ __forceinline__ void next(v4i &c, float &sc)
+    // hands out the slot's block; refill() then requests the block PF iterations ahead into the same slot
+    template <int SLOT> __device__ __forceinline__ void take(v4i &c, float &sc) const { c = codes[SLOT]; sc = scale[SLOT]; }
+    template <int SLOT> __device__ __forceinline__ void refill() { request<SLOT>(); }
+};
+
+// The same walk for a per-row fp32 vector (mean, rstd): the lane's row of each block, requested PF blocks ahead.
+struct RowStream {
+    const float *v;
+    int RB, lane;
+    BlockWalk at;
+    float val[PF];
+    template <int SLOT> __device__ __forceinline__ void request()
     {
-        c = codes[0]; sc = scale[0];
-#pragma unroll
-        for (int i = 0; i + 1 < PF; ++i) { codes[i] = codes[i + 1]; scale[i] = scale[i + 1]; }
-        request(PF - 1);
+        if (at.rb < RB) val[SLOT] = v[at.rb * QB + (lane >> 1)];
+        at.step();
     }
+    __device__ __forceinline__ RowStream(const float *v_, int R, int SC, int stride, int lane_, int blk0)
+        : v(v_), RB(R / QB), lane(lane_), at(blk0, stride, SC)
+    {
+        static_for<0, PF>([&](auto i) { request<decltype(i)::value>(); });
+    }
+    template <int SLOT> __device__ __forceinline__ float take() const { return val[SLOT]; }
+    template <int SLOT> __device__ __forceinline__ void refill() { request<SLOT>(); }
 };
 
 // gelu_fwd.py:34-126
@@ -187,15 +226,17 @@ __global__ __launch_bounds__(NT) void gelu_fwd_kernel(const int8_t *q, const ST 
     float zero = 0.0f;
     asm volatile("" : "+v"(zero));                                 // evaluated on the device, like every other entry
     const float f0 = gelu<APPROX>(zero);
-    for (BlockWalk w(blk0, stride, SC); w.rb < RB; w.step()) {
+    for_each_block_pipelined(BlockWalk(blk0, stride, SC), RB, blk0, stride, [&](const BlockWalk &w, auto slot_c) {
+        constexpr int SLOT = decltype(slot_c)::value;
         const size_t e0 = (size_t)(w.rb * QB + (lane >> 1)) * C + w.cb * QB + (lane & 1) * 16;
         v4i c; float sc;
-        in.next(c, sc);
+        in.template take<SLOT>(c, sc);
         float scale;
         const v4i codes = gelu_fwd_block<APPROX>(c, sc, f0, amax_eps, tab, qtab, lane, &scale);
+        in.template refill<SLOT>();                                // after the last use of c: the load lands in its registers
         *reinterpret_cast<v4i *>(qy + e0) = codes;
         if (lane == 0) store_scale(sy, w.rb * SC + w.cb, scale);
-    }
+    });
 }
 
 // gelu_bwd.py:28-171
@@ -212,49 +253,86 @@ __global__ __launch_bounds__(NT) void gelu_bwd_kernel(const int8_t *qx, const ST
     float zero = 0.0f;
     asm volatile("" : "+v"(zero));
     const float f0 = dgelu<APPROX>(zero);
-    for (BlockWalk w(blk0, stride, SC); w.rb < RB; w.step()) {
+    for_each_block_pipelined(BlockWalk(blk0, stride, SC), RB, blk0, stride, [&](const BlockWalk &w, auto slot_c) {
+        constexpr int SLOT = decltype(slot_c)::value;
         const size_t e0 = (size_t)(w.rb * QB + (lane >> 1)) * C + w.cb * QB + (lane & 1) * 16;
         v4i cx, cg; float scx, scg;
-        inx.next(cx, scx);
-        ing.next(cg, scg);
+        inx.template take<SLOT>(cx, scx);
+        ing.template take<SLOT>(cg, scg);
         float x[16], g[16];
         unpack16(cg, scg, g);
         fill_code_table(tab, lane, scx, f0, [](float v, float &a, float &b) { dgelu_pair<APPROX>(v, a, b); });
         gather16(tab, cx, x);
         table_done();
+        inx.template refill<SLOT>();                               // after the last use of the slot's registers
+        ing.template refill<SLOT>();
 #pragma unroll
         for (int k = 0; k < 16; ++k) x[k] = x[k] * g[k];
         float scale;
         v4i codes = quantize16(x, 0.0f, rounding, seed, offset, e0, &scale);
         *reinterpret_cast<v4i *>(qy + e0) = codes;
         if (lane == 0) store_scale(sy, w.rb * SC + w.cb, scale);
-    }
+    });
 }
 
-// layernorm.py:74-190, with a real beta
+// layernorm.py:74-190, with a real beta.  Arithmetic (this library's definition; the reference dequantises in binary16):
+//   a = s * rstd[r],  b = -(mean[r] * rstd[r]),  xhat = fma(float(q), a, b),  y = fma(xhat, gamma[c], beta[c])
+// i.e. dequantisation and normalisation are one fma per element with two per-row, per-block constants.
+// The codes, scales and row statistics of the next PF blocks of a wave are requested ahead of their use.
+// One wave: one column block x CW_ROWS consecutive row blocks (gamma and beta are loaded once per wave); the four waves
+// of a workgroup take four adjacent column blocks, i.e. whole 128-byte lines per row.  A wave requests everything it
+// will read before it computes anything (per-column vectors first: they are needed first), works through its blocks in
+// the order their data arrives, and stores all results at the end: no wait ever follows a store (the vector-memory
+// counter cannot tell a finished load from an unfinished store, so a wait behind a store waits for the store too).
+constexpr int CW_ROWS = 4;
 template <typename ST>
 __global__ __launch_bounds__(NT) void layernorm_fwd_kernel(const int8_t *q, const ST *s, const float *gamma,
                                                            const float *beta, const float *mean, const float *rstd,
                                                            int R, int C, int8_t *qy, ST *sy)
 {
-    JF_FOR_EACH_BLOCK(R, C)
-    {
-        BlockPos pos(blk, SC, C, lane);
-        float x[16], w[16], b[16];
-        unpack16(*reinterpret_cast<const v4i *>(q + pos.e0), load_scale(s, pos.rb * SC + pos.cb), x);
-        Load16<float>::run(gamma + pos.col, w);
-        if (beta) Load16<float>::run(beta + pos.col, b);
-        else {
+    const int lane = threadIdx.x & 63, wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
+    const int SC = C / QB, RB = R / QB, S4 = (SC + WPB - 1) / WPB;
+    const int cb = (blockIdx.x % S4) * WPB + wave, grp = blockIdx.x / S4;
+    if (cb >= SC) return;                                          // a wave of the last, partial group of column blocks
+    const int col = cb * QB + (lane & 1) * 16;
+    const int nrb = (RB - grp * CW_ROWS) < CW_ROWS ? (RB - grp * CW_ROWS) : CW_ROWS;      // uniform
+    float g[16], bt[16];
+    Load16<float>::run(gamma + col, g);
+    if (beta) Load16<float>::run(beta + col, bt);
+    else {
 #pragma unroll
-            for (int k = 0; k < 16; ++k) b[k] = 0.0f;
+        for (int k = 0; k < 16; ++k) bt[k] = 0.0f;
+    }
+    v4i c[CW_ROWS];
+    float sc[CW_ROWS], mu[CW_ROWS], rs[CW_ROWS];
+#pragma unroll
+    for (int k = 0; k < CW_ROWS; ++k) {
+        const int rb = grp * CW_ROWS + (k < nrb ? k : 0);
+        const int row = rb * QB + (lane >> 1);
+        c[k] = *reinterpret_cast<const v4i *>(q + (size_t)row * C + col);
+        sc[k] = load_scale(s, rb * SC + cb);
+        mu[k] = mean[row];
+        rs[k] = rstd[row];
+    }
+    v4i out[CW_ROWS];
+    float so[CW_ROWS];
+#pragma unroll
+    for (int k = 0; k < CW_ROWS; ++k) {
+        const size_t e0 = (size_t)((grp * CW_ROWS + k) * QB + (lane >> 1)) * C + col;
+        const float a = sc[k] * rs[k], b = -(mu[k] * rs[k]);
+        float x[16];
+        codes_to_float16(c[k], x);
+#pragma unroll
+        for (int j = 0; j < 16; ++j) x[j] = __builtin_fmaf(__builtin_fmaf(x[j], a, b), g[j], bt[j]);
+        out[k] = quantize16(x, 0.0f, JF_ROUND_NEAREST, 0, 0, e0, &so[k]);
+    }
+#pragma unroll
+    for (int k = 0; k < CW_ROWS; ++k) {
+        if (k < nrb) {
+            const int rb = grp * CW_ROWS + k;
+            *reinterpret_cast<v4i *>(qy + (size_t)(rb * QB + (lane >> 1)) * C + col) = out[k];
+            if (lane == 0) store_scale(sy, rb * SC + cb, so[k]);
         }
-        const float mu = mean[pos.row], rs = rstd[pos.row];
-#pragma unroll
-        for (int k = 0; k < 16; ++k) x[k] = __builtin_fmaf((x[k] - mu) * rs, w[k], b[k]);
-        float scale;
-        v4i codes = quantize16(x, 0.0f, JF_ROUND_NEAREST, 0, 0, pos.e0, &scale);
-        *reinterpret_cast<v4i *>(qy + pos.e0) = codes;
-        if (lane == 0) store_scale(sy, pos.rb * SC + pos.cb, scale);
     }
 }
 
@@ -326,105 +404,219 @@ __device__ __forceinline__ float colsum16_over_rows(const float (&v)[16], int la
     return t;
 }
 
-constexpr int LNB_THREADS = 1024;
-// LayerNorm backward in one launch (layernorm.py:197-402): one workgroup (16 waves) per 32-row strip; the waves take
-// the column blocks round-robin.  Row reductions in a defined order (per row: 16-column partial sums of xhat*wdy as an
-// fmaf chain and of wdy as an add chain go to LDS, then one lane per row adds all C/16 partials in ascending order ->
-// c1, c2, so the requantised dx is bit-reproducible); then dx is computed and requantised.  The strip (2 x 32 x C bytes) is read a second time for that, from the L2 it was just fetched
-// into (keeping it in registers instead does not fit next to the column-sum butterfly).  Also the strip's column sums
-// for dgamma / dbeta.
+// ------------------------------------------------------------------------------------------------
+// LayerNorm backward over full rows (layernorm.py:197-428; the reference reduces over its 128-column tile only).
+// Arithmetic (this library's definition, restated by the CPU checker):
+//   xhat = fma(float(qx), sx * rstd[r], -(mean[r] * rstd[r]))     g = float(qg) * sg     wdy = gamma[c] * g
+//   per row and 16-column half block: p1 = fma chain of xhat * wdy, p2 = add chain of wdy, ascending columns;
+//   per block b = p(columns 0..15) + p(columns 16..31);  per row T_j = sum of b over the blocks j, j+8, ... (ascending),
+//   S = ((T0+T1)+(T2+T3)) + ((T4+T5)+(T6+T7));  c1 = S1 / C, c2 = S2 / C;   dx = (wdy - fma(xhat, c1, c2)) * rstd[r]
+//   dgamma[c] = sum over rows of g * xhat, dbeta[c] = sum over rows of g  (fp32, order fixed by the kernels below).
+//
+// Two launches.  layernorm_bwd_stats_kernel: one wave per (column block, group of LNB_RPW row blocks) walks down its
+// column block (the four waves of a workgroup take four adjacent column blocks, i.e. whole 128-byte lines); the lane keeps gamma and its dgamma / dbeta accumulators in registers (the cross-lane reduction over
+// the 32 rows of a block happens once per wave, not once per block) and stores the per-row block partials b1, b2.
+// layernorm_bwd_dx_kernel: one workgroup per 32-row strip first adds its rows' partials (c1, c2), then computes and
+// requantises dx block by block; at its end the launch also adds the row groups' dgamma / dbeta partials.
+constexpr int LNB_RPW = 4;                 // row blocks per wave of the statistics kernel
+constexpr int LNB_DX_WAVES = 16;           // waves per strip of the dx kernel
+
+// Workgroup = 4 waves = 4 adjacent column blocks (whole 128-byte lines per row) x LNB_RPW row blocks.
+// part1 / part2: [C/32][R] (a wave stores 32 consecutive rows); pdg / pdb: [C][groups].
 template <typename ST>
-__global__ __launch_bounds__(LNB_THREADS) void layernorm_bwd_fused_kernel(const int8_t *qx, const ST *sx, const int8_t *qg,
-                                                                          const ST *sg, const float *gamma, const float *mean,
-                                                                          const float *rstd, int R, int C, int rounding,
-                                                                          uint64_t seed, uint64_t offset, int8_t *qdx, ST *sdx,
-                                                                          float *pdg, float *pdb)
+__global__ __launch_bounds__(NT) void layernorm_bwd_stats_kernel(const int8_t *qx, const ST *sx, const int8_t *qg,
+                                                                 const ST *sg, const float *gamma, const float *mean,
+                                                                 const float *rstd, int R, int C, int groups, float *part1,
+                                                                 float *part2, float *pdg, float *pdb)
 {
-    extern __shared__ float fsm[];                // part1[32][C/16], part2[32][C/16], c1[32], c2[32], column-sum patches
-    const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
-    const int SC = C / QB, H = C / 16, rb = blockIdx.x;
-    float *part1 = fsm, *part2 = fsm + QB * H, *c1s = part2 + QB * H, *c2s = c1s + QB;
-    float *cpatch = c2s + QB + wave * COLSUM_PATCH;
-    const int r = lane >> 1;
-    const float mu = mean[rb * QB + r], rs = rstd[rb * QB + r];
-    for (int cb = wave; cb < SC; cb += LNB_THREADS / WAVE) {
-        const int col = cb * QB + (lane & 1) * 16;
-        const size_t e0 = (size_t)(rb * QB + r) * C + col;
-        float x[16], g[16], w[16], v[16];
-        unpack16(*reinterpret_cast<const v4i *>(qx + e0), load_scale(sx, rb * SC + cb), x);
-        unpack16(*reinterpret_cast<const v4i *>(qg + e0), load_scale(sg, rb * SC + cb), g);
-        Load16<float>::run(gamma + col, w);
-        float p1 = 0.0f, p2 = 0.0f;
+    __shared__ float cpatch_all[WPB][COLSUM_PATCH];
+    const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6, SC = C / QB, RB = R / QB, S4 = (SC + WPB - 1) / WPB;
+    const int cb = (blockIdx.x % S4) * WPB + wave, grp = blockIdx.x / S4;
+    if (cb >= SC) return;                                          // a wave of the last, partial group of column blocks
+    float *cpatch = cpatch_all[wave];
+    const int col = cb * QB + (lane & 1) * 16;
+    const int nrb = (RB - grp * LNB_RPW) < LNB_RPW ? (RB - grp * LNB_RPW) : LNB_RPW;      // uniform
+    // everything the wave reads is requested up front, what it needs first (gamma) first
+    float w[16];
+    Load16<float>::run(gamma + col, w);
+    v4i cx[LNB_RPW], cg[LNB_RPW];
+    float scx[LNB_RPW], scg[LNB_RPW], mu[LNB_RPW], rs[LNB_RPW];
 #pragma unroll
-        for (int k = 0; k < 16; ++k) {
-            const float xh = (x[k] - mu) * rs;
-            const float wdy = w[k] * g[k];
-            p1 = __builtin_fmaf(xh, wdy, p1);
-            p2 = p2 + wdy;
-            v[k] = g[k] * xh;
-        }
-        part1[r * H + cb * 2 + (lane & 1)] = p1;
-        part2[r * H + cb * 2 + (lane & 1)] = p2;
-        if (pdg) {
-            // output of lane j (j even): value index j/4 of column set (j/2)%2
-            const size_t dst = (size_t)rb * C + cb * QB + ((lane >> 1) & 1) * 16 + (lane >> 2);
-            const float tg = colsum16_over_rows(v, lane, cpatch);  // sum of dy*xhat
-            if ((lane & 1) == 0) pdg[dst] = tg;
-            const float tb = colsum16_over_rows(g, lane, cpatch);  // sum of dy
-            if ((lane & 1) == 0) pdb[dst] = tb;
+    for (int k = 0; k < LNB_RPW; ++k) {
+        const int rb = grp * LNB_RPW + (k < nrb ? k : 0);
+        const int row = rb * QB + (lane >> 1);
+        const size_t e0 = (size_t)row * C + col;
+        cx[k] = *reinterpret_cast<const v4i *>(qx + e0);
+        cg[k] = *reinterpret_cast<const v4i *>(qg + e0);
+        scx[k] = load_scale(sx, rb * SC + cb);
+        scg[k] = load_scale(sg, rb * SC + cb);
+        mu[k] = mean[row];
+        rs[k] = rstd[row];
+    }
+    float accg[16], accb[16], o1[LNB_RPW], o2[LNB_RPW];
+#pragma unroll
+    for (int j = 0; j < 16; ++j) { accg[j] = 0.0f; accb[j] = 0.0f; }
+#pragma unroll
+    for (int k = 0; k < LNB_RPW; ++k) {
+        if (k < nrb) {
+            const float a = scx[k] * rs[k], b = -(mu[k] * rs[k]);
+            float x[16], g[16];
+            codes_to_float16(cx[k], x);
+            codes_to_float16(cg[k], g);
+            float p1 = 0.0f, p2 = 0.0f;
+#pragma unroll
+            for (int j = 0; j < 16; ++j) {
+                const float xh = __builtin_fmaf(x[j], a, b);
+                const float gj = g[j] * scg[k];
+                const float wdy = w[j] * gj;
+                p1 = __builtin_fmaf(xh, wdy, p1);
+                p2 = p2 + wdy;
+                accg[j] = __builtin_fmaf(gj, xh, accg[j]);
+                accb[j] = accb[j] + gj;
+            }
+            // the two half blocks of a row: the same two operands in both lanes of the pair
+            p1 = p1 + __int_as_float(__builtin_amdgcn_update_dpp(0, __float_as_int(p1), 0xB1, 0xF, 0xF, false));
+            p2 = p2 + __int_as_float(__builtin_amdgcn_update_dpp(0, __float_as_int(p2), 0xB1, 0xF, 0xF, false));
+            o1[k] = p1; o2[k] = p2;
         }
     }
-    __syncthreads();
-    if (threadIdx.x < QB) {
-        const int rr = threadIdx.x;
-        float t1 = 0.0f, t2 = 0.0f;
-        for (int h = 0; h < H; ++h) { t1 = t1 + part1[rr * H + h]; t2 = t2 + part2[rr * H + h]; }
-        c1s[rr] = t1 / (float)C;
-        c2s[rr] = t2 / (float)C;
-    }
-    __syncthreads();
-    const float k1 = c1s[r], k2 = c2s[r];
-    for (int cb = wave; cb < SC; cb += LNB_THREADS / WAVE) {
-        const int col = cb * QB + (lane & 1) * 16;
-        const size_t e0 = (size_t)(rb * QB + r) * C + col;
-        float x[16], g[16], w[16];
-        unpack16(*reinterpret_cast<const v4i *>(qx + e0), load_scale(sx, rb * SC + cb), x);
-        unpack16(*reinterpret_cast<const v4i *>(qg + e0), load_scale(sg, rb * SC + cb), g);
-        Load16<float>::run(gamma + col, w);
 #pragma unroll
-        for (int k = 0; k < 16; ++k) {
-            const float xh = (x[k] - mu) * rs;
-            const float wdy = w[k] * g[k];
-            x[k] = (wdy - __builtin_fmaf(xh, k1, k2)) * rs;
+    for (int k = 0; k < LNB_RPW; ++k) {                            // all stores after all loads have been consumed
+        if (k < nrb && (lane & 1) == 0) {
+            const int row = (grp * LNB_RPW + k) * QB + (lane >> 1);
+            part1[(size_t)cb * R + row] = o1[k];
+            part2[(size_t)cb * R + row] = o2[k];
         }
-        float scale;
-        v4i codes = quantize16(x, 0.0f, rounding, seed, offset, e0, &scale);
-        *reinterpret_cast<v4i *>(qdx + e0) = codes;
-        if (lane == 0) store_scale(sdx, rb * SC + cb, scale);
+    }
+    if (pdg) {
+        // output of lane j (j even): value index j/4 of column set (j/2)%2
+        const size_t dst = ((size_t)cb * QB + ((lane >> 1) & 1) * 16 + (lane >> 2)) * groups + grp;
+        const float tg = colsum16_over_rows(accg, lane, cpatch);
+        if ((lane & 1) == 0) pdg[dst] = tg;
+        const float tb = colsum16_over_rows(accb, lane, cpatch);
+        if ((lane & 1) == 0) pdb[dst] = tb;
     }
 }
 
-// out[c] = sum over strips of part[strip][c]   (layernorm.py:405-428).  64 columns per workgroup, 16 strip lanes
-// per column (fixed partition and a fixed tree, so the result is reproducible).
-__global__ __launch_bounds__(1024) void colsum_kernel(const float *part0, float *out0, const float *part1, float *out1,
-                                                      int strips, int C)
+// 64-lane sum, every lane returns it (data-parallel-primitive moves; a fixed tree)
+__device__ __forceinline__ float wave_sum(float v)
 {
-    __shared__ float red[16][65];
-    const float *part = blockIdx.y ? part1 : part0;
-    float *out = blockIdx.y ? out1 : out0;
-    if (!out) return;                                              // uniform
-    const int tx = threadIdx.x & 63, ty = threadIdx.x >> 6;
-    const int c = blockIdx.x * 64 + tx;
-    float a = 0.0f;
-    if (c < C)
-        for (int i = ty; i < strips; i += 16) a += part[(size_t)i * C + c];
-    red[ty][tx] = a;
-    __syncthreads();
-    if (ty == 0 && c < C) {
-        float t = 0.0f;
+    auto step = [](float x, auto ctrl_c, auto rows_c) {
+        const int t = __builtin_amdgcn_update_dpp(0, __float_as_int(x), decltype(ctrl_c)::value, decltype(rows_c)::value, 0xF, false);
+        return x + __int_as_float(t);
+    };
+    using all = std::integral_constant<int, 0xF>;
+    v = step(v, std::integral_constant<int, 0xB1>{}, all{});
+    v = step(v, std::integral_constant<int, 0x4E>{}, all{});
+    v = step(v, std::integral_constant<int, 0x141>{}, all{});
+    v = step(v, std::integral_constant<int, 0x140>{}, all{});      // every lane: the sum of its 16-lane row
+    v = step(v, std::integral_constant<int, 0x142>{}, std::integral_constant<int, 0xA>{});   // rows 1, 3 += row 0, 2
+    v = step(v, std::integral_constant<int, 0x143>{}, std::integral_constant<int, 0xC>{});   // rows 2, 3 += row 1
+    return __int_as_float(__builtin_amdgcn_readlane(__float_as_int(v), 63));
+}
+
+template <typename ST>
+__global__ __launch_bounds__(WAVE * LNB_DX_WAVES) void layernorm_bwd_dx_kernel(
+    const int8_t *qx, const ST *sx, const int8_t *qg, const ST *sg, const float *gamma, const float *mean,
+    const float *rstd, int R, int C, int rounding, uint64_t seed, uint64_t offset, const float *part1, const float *part2,
+    int8_t *qdx, ST *sdx, const float *pdg, const float *pdb, int groups, float *dgamma, float *dbeta)
+{
+    extern __shared__ __attribute__((aligned(16))) float lds_f[];  // gamma[C], c1[32], c2[32], T[2][8][32]
+    float *gl = lds_f, *cs = lds_f + C, *tj = cs + 2 * QB;
+    const int lane = threadIdx.x & 63, wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
+    const int SC = C / QB, rb = blockIdx.x;
+    const int row = rb * QB + (lane >> 1);
+    // A wave's blocks are cb = wave, wave + 16, ...: up to DXB of them are requested at once, before anything else; they
+    // are computed in arrival order and their results stored together at the end (no wait follows a store, except
+    // between the batches of rows wider than 16 * DXB blocks).
+    constexpr int DXB = 4;
+    v4i cx[DXB], cg[DXB];
+    float scx[DXB], scg[DXB];
+    auto request_batch = [&](int cb0) {
+        static_for<0, DXB>([&](auto i_c) {
+            constexpr int I = decltype(i_c)::value;
+            const int cb = cb0 + I * LNB_DX_WAVES;
+            if (cb < SC) {
+                const size_t e0 = (size_t)row * C + cb * QB + (lane & 1) * 16;
+                cx[I] = *reinterpret_cast<const v4i *>(qx + e0);
+                cg[I] = *reinterpret_cast<const v4i *>(qg + e0);
+                scx[I] = load_scale(sx, rb * SC + cb);
+                scg[I] = load_scale(sg, rb * SC + cb);
+            }
+        });
+    };
+    request_batch(wave);
+    const float mu = mean[row], rs = rstd[row];
+    for (int c = threadIdx.x * 4; c < C; c += WAVE * LNB_DX_WAVES * 4)
+        *reinterpret_cast<v4f *>(gl + c) = *reinterpret_cast<const v4f *>(gamma + c);
+    if (threadIdx.x < 512) {
+        // Row sums of the block partials.  Threads 0..255: S1, 256..511: S2; thread (j, r) adds the blocks j, j+8, ... of
+        // row r in ascending order (absent blocks contribute +0, which changes no bit; 8 independent loads at a time).
+        const int t = threadIdx.x & 255, j = t >> 5, r = t & 31, which = threadIdx.x >> 8;
+        const float *part = (which ? part2 : part1) + rb * QB + r;
+        float acc = 0.0f;
+        for (int cb0 = 0; cb0 < SC; cb0 += 64) {
+            float v[8];
 #pragma unroll
-        for (int k = 0; k < 16; ++k) t += red[k][tx];
-        out[c] = t;
+            for (int i = 0; i < 8; ++i) { const int cb = cb0 + j + 8 * i; v[i] = cb < SC ? part[(size_t)cb * R] : 0.0f; }
+#pragma unroll
+            for (int i = 0; i < 8; ++i) acc = acc + v[i];
+        }
+        tj[(which * 8 + j) * QB + r] = acc;
+    }
+    // dgamma / dbeta: one column per wave of the whole launch: the row groups' partials, one per lane, then a wave sum
+    if (pdg) {
+        for (int c = blockIdx.x * LNB_DX_WAVES + wave; c < C; c += gridDim.x * LNB_DX_WAVES) {
+            float tg = 0.0f, tb = 0.0f;
+            for (int gi = lane; gi < groups; gi += WAVE) { tg = tg + pdg[(size_t)c * groups + gi]; tb = tb + pdb[(size_t)c * groups + gi]; }
+            tg = wave_sum(tg);
+            tb = wave_sum(tb);
+            if (lane == 0) {
+                if (dgamma) dgamma[c] = tg;
+                if (dbeta) dbeta[c] = tb;
+            }
+        }
+    }
+    __syncthreads();
+    if (threadIdx.x < 2 * QB) {
+        // S = ((T0+T1)+(T2+T3)) + ((T4+T5)+(T6+T7)),  c = S / C
+        const float *T = tj + (threadIdx.x >> 5) * 8 * QB + (threadIdx.x & 31);
+        const float S = ((T[0] + T[QB]) + (T[2 * QB] + T[3 * QB])) + ((T[4 * QB] + T[5 * QB]) + (T[6 * QB] + T[7 * QB]));
+        cs[threadIdx.x] = S / (float)C;
+    }
+    __syncthreads();
+    const float k1 = cs[lane >> 1], k2 = cs[QB + (lane >> 1)];
+    const float b = -(mu * rs);
+    for (int cb0 = wave; cb0 < SC; cb0 += DXB * LNB_DX_WAVES) {
+        if (cb0 != wave) request_batch(cb0);                       // rows of more than 64 blocks only
+        v4i out[DXB];
+        float so[DXB];
+        static_for<0, DXB>([&](auto i_c) {
+            constexpr int I = decltype(i_c)::value;
+            const int cb = cb0 + I * LNB_DX_WAVES;
+            if (cb >= SC) return;                                  // uniform
+            const int col = cb * QB + (lane & 1) * 16;
+            const size_t e0 = (size_t)row * C + col;
+            const float a = scx[I] * rs, sgk = scg[I];
+            float x[16], g[16], w[16];
+            Load16<float>::run(gl + col, w);
+            codes_to_float16(cx[I], x);
+            codes_to_float16(cg[I], g);
+#pragma unroll
+            for (int jj = 0; jj < 16; ++jj) {
+                const float xh = __builtin_fmaf(x[jj], a, b);
+                const float wdy = w[jj] * (g[jj] * sgk);
+                x[jj] = (wdy - __builtin_fmaf(xh, k1, k2)) * rs;
+            }
+            out[I] = quantize16(x, 0.0f, rounding, seed, offset, e0, &so[I]);
+        });
+        static_for<0, DXB>([&](auto i_c) {
+            constexpr int I = decltype(i_c)::value;
+            const int cb = cb0 + I * LNB_DX_WAVES;
+            if (cb >= SC) return;
+            *reinterpret_cast<v4i *>(qdx + (size_t)row * C + cb * QB + (lane & 1) * 16) = out[I];
+            if (lane == 0) store_scale(sdx, rb * SC + cb, so[I]);
+        });
     }
 }
 
@@ -486,6 +678,10 @@ static int check_block_tensor(const void *q, const void *s, int R, int C, int sc
     if (!aligned16(q)) return JF_ERR_ALIGN;
     return JF_OK;
 }
+
+// per-column fp32 vectors (gamma, beta) are kept in LDS by the LayerNorm kernels: up to 64 KiB of them, i.e. rows of up
+// to 8192 columns forward and 16320 backward
+constexpr size_t LDS_VECTOR_LIMIT = 64 * 1024;
 
 static inline bool rounding_ok(int r) { return r >= JF_ROUND_NEAREST && r <= JF_ROUND_STOCHASTIC_TRUNC; }
 
@@ -560,18 +756,22 @@ int jf_layernorm_fwd(const int8_t *q, const void *s, const float *gamma, const f
     if (!gamma || !mean || !rstd || !qy || !sy) return JF_ERR_NULL;
     if (!aligned16(qy) || !aligned16(gamma) || (beta && !aligned16(beta))) return JF_ERR_ALIGN;
     hipStream_t st = (hipStream_t)stream;
-    const int grid = grid_for_blocks(R, C);
+    const int grid = ((C / QB + WPB - 1) / WPB) * ((R / QB + CW_ROWS - 1) / CW_ROWS);
+    const size_t smem = 0;
     if (scale_dtype == JF_SCALE_F16)
-        JF_LAUNCH(layernorm_fwd_kernel<half_t>, grid, 0, st, q, (const half_t *)s, gamma, beta, mean, rstd, R, C, qy,
+        JF_LAUNCH(layernorm_fwd_kernel<half_t>, grid, smem, st, q, (const half_t *)s, gamma, beta, mean, rstd, R, C, qy,
                   (half_t *)sy);
-    JF_LAUNCH(layernorm_fwd_kernel<float>, grid, 0, st, q, (const float *)s, gamma, beta, mean, rstd, R, C, qy,
+    JF_LAUNCH(layernorm_fwd_kernel<float>, grid, smem, st, q, (const float *)s, gamma, beta, mean, rstd, R, C, qy,
               (float *)sy);
 }
+
+// workspace: per-row block partials [2][C/32][R] and per-row-group column partials [2][C][groups]
+static inline int lnb_groups(int R) { return (R / QB + LNB_RPW - 1) / LNB_RPW; }
 
 size_t jf_layernorm_bwd_workspace_bytes(int R, int C)
 {
     if (R <= 0 || C <= 0) return 0;
-    return ((size_t)2 * R + (size_t)2 * (R / QB) * C) * sizeof(float);
+    return ((size_t)2 * R * (C / QB) + (size_t)2 * lnb_groups(R) * C) * sizeof(float);
 }
 
 int jf_layernorm_bwd(const int8_t *qx, const void *sx, const int8_t *qg, const void *sg, const float *gamma,
@@ -587,30 +787,25 @@ int jf_layernorm_bwd(const int8_t *qx, const void *sx, const int8_t *qg, const v
     if (!aligned16(qdx) || !aligned16(gamma)) return JF_ERR_ALIGN;
     if (!workspace || workspace_bytes < jf_layernorm_bwd_workspace_bytes(R, C)) return JF_ERR_WORKSPACE;
     if (!aligned16(workspace)) return JF_ERR_ALIGN;
-    // LDS: two [32][C/16] partial-sum arrays, c1/c2, one column-sum patch per wave
-    const size_t smem = ((size_t)2 * QB * (C / 16) + 2 * QB + (LNB_THREADS / WAVE) * COLSUM_PATCH) * sizeof(float);
-    if (smem > 160 * 1024 - 512) return JF_ERR_SHAPE;          // rows of up to ~5700 columns
     if (!device_is_gfx950()) return JF_ERR_DEVICE;
     hipStream_t st = (hipStream_t)stream;
     const bool want_dw = dgamma || dbeta;
-    // workspace: [2R floats, unused by this implementation][strips x C partial dgamma][strips x C partial dbeta]
-    float *pdg = want_dw ? (float *)workspace + (size_t)2 * R : nullptr, *pdb = want_dw ? pdg + (size_t)(R / QB) * C : nullptr;
-#define JF_LNF(ST)                                                                                                    \
-    do {                                                                                                              \
-        auto kern = layernorm_bwd_fused_kernel<ST>;                                                                   \
-        if (smem > 64 * 1024) {                                                                                       \
-            hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void *>(kern),                                  \
-                                               hipFuncAttributeMaxDynamicSharedMemorySize, (int)smem);                \
-            if (e != hipSuccess) return (int)e;                                                                       \
-        }                                                                                                             \
-        hipLaunchKernelGGL(kern, dim3(R / QB), dim3(LNB_THREADS), smem, st, qx, (const ST *)sx, qg, (const ST *)sg,   \
-                           gamma, mean, rstd, R, C, rounding, seed, offset, qdx, (ST *)sdx, pdg, pdb);                \
+    const int SC = C / QB, groups = lnb_groups(R);
+    const size_t smem = ((size_t)C + 2 * QB + 16 * QB) * sizeof(float);   // gamma, c1, c2 and the row-sum partials in LDS
+    if (smem > LDS_VECTOR_LIMIT) return JF_ERR_SHAPE;
+    float *part1 = (float *)workspace, *part2 = part1 + (size_t)R * SC;
+    float *pdg = want_dw ? part2 + (size_t)R * SC : nullptr, *pdb = want_dw ? pdg + (size_t)groups * C : nullptr;
+#define JF_LNB(ST)                                                                                                     \
+    do {                                                                                                               \
+        hipLaunchKernelGGL(layernorm_bwd_stats_kernel<ST>, dim3((SC + WPB - 1) / WPB * groups), dim3(NT), 0, st, qx,   \
+                           (const ST *)sx, qg, (const ST *)sg, gamma, mean, rstd, R, C, groups, part1, part2, pdg, pdb); \
+        hipLaunchKernelGGL(layernorm_bwd_dx_kernel<ST>, dim3(R / QB), dim3(WAVE * LNB_DX_WAVES), smem, st, qx,         \
+                           (const ST *)sx, qg, (const ST *)sg, gamma, mean, rstd, R, C, rounding, seed, offset, part1, \
+                           part2, qdx, (ST *)sdx, pdg, pdb, groups, dgamma, dbeta);                                    \
     } while (0)
-    if (scale_dtype == JF_SCALE_F16) JF_LNF(half_t);
-    else JF_LNF(float);
-#undef JF_LNF
-    if (want_dw)
-        hipLaunchKernelGGL(colsum_kernel, dim3((C + 63) / 64, 2), dim3(1024), 0, st, pdg, dgamma, pdb, dbeta, R / QB, C);
+    if (scale_dtype == JF_SCALE_F16) JF_LNB(half_t);
+    else JF_LNB(float);
+#undef JF_LNB
     return (int)hipGetLastError();
 }
 

@@ -1,15 +1,26 @@
 // Calibration kernels for the roofline discussion: what the matrix pipe and the vector ALU of this part deliver,
 // alone and together, from registers (no memory traffic).  They have no counterpart in the reference; bench.py
 // uses them to print the measured MFMA peak and the measured cost of the fp32 scale-accumulate next to it.
+//
+// Every workgroup's first wave also records how many shader-clock cycles and how many ticks of the constant-rate
+// wall clock it ran for, so that a result can be stated in cycles as well as in nanoseconds: "the two pipes add up"
+// can then be told apart from "the clock dropped under the combined load".
 #include "jf_device.hpp"
 
 namespace jf {
 
 // Per iteration and wave: 4 x ( [one 32x32x32 INT8 MFMA on its own accumulator chain]  +  [NV independent v_fmac_f32] ).
-//   WITH_MFMA / NV = (1, 0): matrix pipe alone; (0, 32): vector ALU alone; (1, 32): both, independent of each other.
-template <int WITH_MFMA, int NV>
-__global__ __launch_bounds__(256) void calib_kernel(int iters, float *out)
+//   MODE JF_CAL_UNIFORM: every wave does both parts (WITH_MFMA / NV select them).
+//   MODE JF_CAL_SPLIT:   the first half of a workgroup's waves issue only the MFMAs, the second half only the
+//                        fmacs: with 8 waves per workgroup, waves w and w+4 share a SIMD, so each SIMD runs matrix
+//                        work and vector work from DIFFERENT waves.
+//   MODE JF_CAL_STREAM:  the instruction stream of the GEMM's K block: an MFMA whose accumulator input is the inline
+//                        constant, then 16 subtractions + 16 fmacs on the PREVIOUS product (real dependencies).
+template <int MODE, int WITH_MFMA, int NV>
+__global__ __launch_bounds__(512) void calib_kernel(int iters, float *out, unsigned long long *clocks)
 {
+    const long long c0 = clock64(), w0 = wall_clock64();
+    const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6), nwaves = blockDim.x >> 6;
     v4i a = {(int)threadIdx.x, 1, 2, 3}, b = {4, 5, 6, (int)blockIdx.x};
     v16i c[4];
     for (int i = 0; i < 4; ++i)
@@ -17,12 +28,48 @@ __global__ __launch_bounds__(256) void calib_kernel(int iters, float *out)
     float f[32];
     for (int i = 0; i < 32; ++i) f[i] = (float)i;
     const float s = 1.0f + 1e-6f * threadIdx.x, m = 0.5f;
-    for (int it = 0; it < iters; ++it) {
+    if (MODE == JF_CAL_STREAM) {
+        v16i d_pend = c[0];
+        for (int it = 0; it < iters; ++it) {
 #pragma unroll
-        for (int i = 0; i < 4; ++i) {
-            if (WITH_MFMA) c[i] = __builtin_amdgcn_mfma_i32_32x32x32_i8(a, b, c[i], 0, 0, 0);
+            for (int i = 0; i < 4; ++i) {
+                v16i d_new;
+                asm volatile("v_mfma_i32_32x32x32_i8 %0, %1, %2, 0x3e22f983" : "=&v"(d_new) : "v"(a), "v"(b));
+                __builtin_amdgcn_sched_barrier(0);
+                float t[16];
 #pragma unroll
-            for (int v = 0; v < NV; ++v) f[v % 32] = __builtin_fmaf(s, m, f[v % 32]);
+                for (int v = 0; v < 16; ++v) t[v] = __int_as_float(d_pend[v]) - __int_as_float(0x3e22f983);
+#pragma unroll
+                for (int v = 0; v < 16; ++v) f[16 * (i & 1) + v] = __builtin_fmaf(s, t[v], f[16 * (i & 1) + v]);
+#pragma unroll
+                for (int v = 0; v < 32; ++v) asm volatile("" : "+v"(f[v]));
+                __builtin_amdgcn_sched_barrier(0);
+                d_pend = d_new;
+            }
+        }
+        c[0] = d_pend;
+    } else if (MODE == JF_CAL_SPLIT) {
+        if (wave < nwaves / 2) {                                   // a uniform branch: this wave only multiplies matrices
+            for (int it = 0; it < iters; ++it) {
+#pragma unroll
+                for (int i = 0; i < 4; ++i) c[i] = __builtin_amdgcn_mfma_i32_32x32x32_i8(a, b, c[i], 0, 0, 0);
+            }
+        } else {                                                   // ... and this one only runs the vector ALU
+            for (int it = 0; it < iters; ++it) {
+#pragma unroll
+                for (int v = 0; v < 4 * 32; ++v) f[v % 32] = __builtin_fmaf(s, m, f[v % 32]);
+#pragma unroll
+                for (int v = 0; v < 32; ++v) asm volatile("" : "+v"(f[v]));
+            }
+        }
+    } else {
+        for (int it = 0; it < iters; ++it) {
+#pragma unroll
+            for (int i = 0; i < 4; ++i) {
+                if (WITH_MFMA) c[i] = __builtin_amdgcn_mfma_i32_32x32x32_i8(a, b, c[i], 0, 0, 0);
+#pragma unroll
+                for (int v = 0; v < NV; ++v) f[v % 32] = __builtin_fmaf(s, m, f[v % 32]);
+            }
         }
     }
     float t = 0.0f;
@@ -31,23 +78,39 @@ __global__ __launch_bounds__(256) void calib_kernel(int iters, float *out)
     for (int i = 0; i < 4; ++i)
         for (int v = 0; v < 16; ++v) u += c[i][v];
     if (t == 1.2345f || u == 123456789) out[0] = t + (float)u;      // never true: keeps the work alive
+    if (clocks && threadIdx.x == 0) {
+        clocks[2 * blockIdx.x] = (unsigned long long)(clock64() - c0);
+        clocks[2 * blockIdx.x + 1] = (unsigned long long)(wall_clock64() - w0);
+    }
 }
 
 }  // namespace jf
 
 using namespace jf;
 
-extern "C" int jf_calibrate(int with_mfma, int valu_per_mfma, int iters, int workgroups, float *scratch, jf_stream_t stream)
+extern "C" int jf_calibrate(int mode, int with_mfma, int valu_per_mfma, int iters, int workgroups, int threads,
+                            float *scratch, unsigned long long *clocks, jf_stream_t stream)
 {
     if (!scratch) return JF_ERR_NULL;
-    if (iters <= 0 || workgroups <= 0) return JF_ERR_SHAPE;
+    if (iters <= 0 || workgroups <= 0 || threads < 128 || threads > 512 || threads % 128) return JF_ERR_SHAPE;
+    if (!device_is_gfx950()) return JF_ERR_DEVICE;
     hipStream_t st = (hipStream_t)stream;
-#define JF_CAL(M, NV)                                                                               \
-    if (with_mfma == M && valu_per_mfma == NV) {                                                    \
-        hipLaunchKernelGGL((calib_kernel<M, NV>), dim3(workgroups), dim3(256), 0, st, iters, scratch); \
-        return (int)hipGetLastError();                                                              \
+#define JF_CAL(MODE, M, NV)                                                                                   \
+    if (mode == MODE && with_mfma == M && valu_per_mfma == NV) {                                              \
+        hipLaunchKernelGGL((calib_kernel<MODE, M, NV>), dim3(workgroups), dim3(threads), 0, st, iters, scratch, clocks); \
+        return (int)hipGetLastError();                                                                        \
     }
-    JF_CAL(1, 0) JF_CAL(0, 32) JF_CAL(1, 32) JF_CAL(0, 16) JF_CAL(1, 16)
+    JF_CAL(JF_CAL_UNIFORM, 1, 0) JF_CAL(JF_CAL_UNIFORM, 0, 32) JF_CAL(JF_CAL_UNIFORM, 1, 32)
+    JF_CAL(JF_CAL_UNIFORM, 0, 16) JF_CAL(JF_CAL_UNIFORM, 1, 16)
+    JF_CAL(JF_CAL_SPLIT, 1, 32) JF_CAL(JF_CAL_STREAM, 1, 32)
 #undef JF_CAL
     return JF_ERR_ENUM;
+}
+
+extern "C" int jf_wall_clock_khz(void)
+{
+    int dev = 0, khz = 0;
+    if (hipGetDevice(&dev) != hipSuccess) return 0;
+    if (hipDeviceGetAttribute(&khz, hipDeviceAttributeWallClockRate, dev) != hipSuccess) return 0;
+    return khz;
 }

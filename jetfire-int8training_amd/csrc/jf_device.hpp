@@ -23,6 +23,15 @@ typedef int v16i __attribute__((ext_vector_type(16)));
 typedef float v4f __attribute__((ext_vector_type(4)));
 typedef _Float16 half_t;
 
+// f(integral_constant<int, I>) for I = 0 .. N-1, unrolled at compile time
+template <int I, int N, typename F> __device__ __forceinline__ void static_for(F &&f)
+{
+    if constexpr (I < N) {
+        f(std::integral_constant<int, I>{});
+        static_for<I + 1, N>(f);
+    }
+}
+
 // ---------------------------------------------------------------------------------------------
 // scale element access: binary16 or binary32 behind one template parameter
 template <typename ST> __device__ __forceinline__ float load_scale(const ST *p, int i) { return (float)p[i]; }
@@ -50,12 +59,17 @@ __device__ __forceinline__ float wave_max(float v)
 }
 
 // ---------------------------------------------------------------------------------------------
-// Philox4x32-10.  (Salmon et al., SC'11.)
-__device__ __forceinline__ void philox4x32_10(uint32_t c0, uint32_t c1, uint32_t c2, uint32_t c3,
-                                              uint32_t k0, uint32_t k1, uint32_t out[4])
+// Philox4x32-R.  (Salmon et al., "Parallel random numbers: as easy as 1, 2, 3", SC'11.)  The rounding noise uses
+// R = 7, the smallest round count the authors report as passing BigCrush (10 is their default with a safety margin):
+// the generator is the largest single cost of every stochastic-rounding kernel here, and its multiplies run at a
+// quarter of the vector ALU's rate.
+constexpr int PHILOX_ROUNDS = 7;
+template <int ROUNDS>
+__device__ __forceinline__ void philox4x32(uint32_t c0, uint32_t c1, uint32_t c2, uint32_t c3,
+                                           uint32_t k0, uint32_t k1, uint32_t out[4])
 {
 #pragma unroll
-    for (int r = 0; r < 10; ++r) {
+    for (int r = 0; r < ROUNDS; ++r) {
         uint64_t p0 = (uint64_t)0xD2511F53u * c0;
         uint64_t p1 = (uint64_t)0xCD9E8D57u * c2;
         uint32_t n0 = (uint32_t)(p1 >> 32) ^ c1 ^ k0;
@@ -79,7 +93,7 @@ __device__ __forceinline__ void sr_noise16(uint64_t seed, uint64_t offset, uint6
     for (int call = 0; call < 2; ++call) {
         uint32_t o[4];
         uint64_t cc = c + (uint64_t)call;
-        philox4x32_10((uint32_t)cc, (uint32_t)(cc >> 32), 0u, 0u, (uint32_t)seed, (uint32_t)(seed >> 32), o);
+        philox4x32<PHILOX_ROUNDS>((uint32_t)cc, (uint32_t)(cc >> 32), 0u, 0u, (uint32_t)seed, (uint32_t)(seed >> 32), o);
 #pragma unroll
         for (int w = 0; w < 4; ++w) {
             // (h + 0.5) * 2^-16 - 0.5 = h * 2^-16 + (2^-17 - 0.5): every step of either form is exact (17 significant
@@ -134,10 +148,12 @@ __device__ __forceinline__ uint32_t pack4(int a, int b, int c, int d)
 // Round-to-nearest-even codes of 4 values, clamped to +-127, packed into one word.  Clamping first and rounding
 // second gives the same integers as rounding first (the bounds are integers).  Adding 1.5*2^23 rounds to an
 // integer in the addition itself and leaves its two's-complement low byte in the low byte of the bit pattern.
+// CLAMP = false: for values the caller knows to round into [-127, 127] (|y| < 127.5).
+template <bool CLAMP = true>
 __device__ __forceinline__ uint32_t round_clamp_pack4(float a, float b, float c, float d)
 {
     auto code_bits = [](float y) {
-        const float yc = __builtin_amdgcn_fmed3f(y, -127.0f, 127.0f);
+        const float yc = CLAMP ? __builtin_amdgcn_fmed3f(y, -127.0f, 127.0f) : y;
         return __float_as_uint(yc + 12582912.0f);
     };
     const uint32_t ab = __builtin_amdgcn_perm(code_bits(b), code_bits(a), 0x0c0c0400u);   // bytes: a, b, 0, 0
@@ -164,6 +180,10 @@ __device__ __forceinline__ v4i quantize16(const float v[16], float amax_eps, int
     BlockDivisor d(s);
     float y[16];
     d.div16(v, y);
+    if (!d.fast) {                                             // uniform, rare: a scale near the ends of the exponent range
+#pragma unroll                                                 // (a denormal s can be off by far more than an ulp)
+        for (int i = 0; i < 16; ++i) y[i] = __builtin_amdgcn_fmed3f(y[i], -127.0f, 127.0f);
+    }
     if (rounding == JF_ROUND_STOCHASTIC || rounding == JF_ROUND_STOCHASTIC_TRUNC) {
         float n[16];
         sr_noise16(seed, offset, e0, n);
@@ -182,12 +202,27 @@ __device__ __forceinline__ v4i quantize16(const float v[16], float amax_eps, int
         out.z = (int)pack4(c[8], c[9], c[10], c[11]);
         out.w = (int)pack4(c[12], c[13], c[14], c[15]);
     } else {
-        out.x = (int)round_clamp_pack4(y[0], y[1], y[2], y[3]);
-        out.y = (int)round_clamp_pack4(y[4], y[5], y[6], y[7]);
-        out.z = (int)round_clamp_pack4(y[8], y[9], y[10], y[11]);
-        out.w = (int)round_clamp_pack4(y[12], y[13], y[14], y[15]);
+        // no clamp here: |v| <= amax and s = amax/127 correctly rounded give |v/s| <= 127 * (1 + 2^-23) < 127.5 (scales
+        // outside the normal range were clamped above), and the stochastic path has limited |y| + noise to 127
+        out.x = (int)round_clamp_pack4<false>(y[0], y[1], y[2], y[3]);
+        out.y = (int)round_clamp_pack4<false>(y[4], y[5], y[6], y[7]);
+        out.z = (int)round_clamp_pack4<false>(y[8], y[9], y[10], y[11]);
+        out.w = (int)round_clamp_pack4<false>(y[12], y[13], y[14], y[15]);
     }
     return out;
+}
+
+// the 16 codes of a lane as floats (no scale applied)
+__device__ __forceinline__ void codes_to_float16(v4i p, float x[16])
+{
+    const int w[4] = {p.x, p.y, p.z, p.w};
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+        x[4 * i + 0] = (float)((w[i] << 24) >> 24);
+        x[4 * i + 1] = (float)((w[i] << 16) >> 24);
+        x[4 * i + 2] = (float)((w[i] << 8) >> 24);
+        x[4 * i + 3] = (float)(w[i] >> 24);
+    }
 }
 
 __device__ __forceinline__ void unpack16(v4i p, float scale, float x[16])

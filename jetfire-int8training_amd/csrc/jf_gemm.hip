@@ -84,14 +84,6 @@ __device__ __forceinline__ void tile_of_workgroup(int tiles_m, int tiles_n, bool
     tn = in_group / gm;
 }
 
-template <int I, int N, typename F> __device__ __forceinline__ void static_for(F &&f)
-{
-    if constexpr (I < N) {
-        f(std::integral_constant<int, I>{});
-        static_for<I + 1, N>(f);
-    }
-}
-
 // vmcnt(n), no wait on the other counters (gfx9 encoding: vmcnt = bits 3:0 and 15:14)
 #define JF_WAIT_VMCNT(n) __builtin_amdgcn_s_waitcnt(((n) & 0xF) | (((n) >> 4) << 14) | 0x0F70)
 

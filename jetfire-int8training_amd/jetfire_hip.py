@@ -28,7 +28,7 @@ EXPORTS = [
     "jf_error_string", "jf_igemm_workspace_bytes", "jf_igemm_s32", "jf_igemm_block_acc", "jf_igemm_block_fp",
     "jf_igemm_splitk_plan", "jf_igemm_block_fp_workspace_bytes", "jf_igemm_block_q_gelu", "jf_igemm_block_fp_noalloc",
     "jf_igemm_block_q", "jf_quantize", "jf_dequantize", "jf_transpose_s8", "jf_rowstats", "jf_layernorm_fwd",
-    "jf_layernorm_bwd_workspace_bytes", "jf_layernorm_bwd", "jf_gelu_fwd", "jf_gelu_bwd", "jf_add", "jf_calibrate",
+    "jf_layernorm_bwd_workspace_bytes", "jf_layernorm_bwd", "jf_gelu_fwd", "jf_gelu_bwd", "jf_add", "jf_calibrate", "jf_wall_clock_khz",
 ]
 
 _lib = None
@@ -66,7 +66,8 @@ def lib():
         L.jf_gelu_fwd.argtypes = [_p, _p, _i, _i, _i, _i, _f, _p, _p, _p]
         L.jf_gelu_bwd.argtypes = [_p, _p, _p, _p, _i, _i, _i, _i, _i, _u64, _u64, _p, _p, _p]
         L.jf_add.argtypes = [_p, _i, _p, _p, _i, _i, _i, _i, _u64, _u64, _p, _p, _p, _p, _p, _p]
-        L.jf_calibrate.argtypes = [_i, _i, _i, _i, _p, _p]
+        L.jf_wall_clock_khz.argtypes = []
+        L.jf_calibrate.argtypes = [_i, _i, _i, _i, _i, _i, _p, _p, _p]
         missing = [name for name in EXPORTS if not hasattr(L, name)]
         if missing:
             raise RuntimeError(f"{LIB_PATH} does not export {missing}")
@@ -418,13 +419,22 @@ def add(x1, q2, s2, rounding=ROUND_TRUNC, with_stats=False, seed=None, offset=No
     return (y1, q, s, rs, rq) if with_stats else (y1, q, s)
 
 
-def calibrate(with_mfma, valu_per_mfma, iters=2000, workgroups_per_cu=4):
-    """Seconds per launch of the register-only calibration kernel and the number of MFMA-sized work items it ran
-    (workgroups * 4 waves * iters * 4)."""
-    cus = torch.cuda.get_device_properties(0).multi_processor_count
+CAL_UNIFORM, CAL_SPLIT, CAL_STREAM = 0, 1, 2
+
+
+def calibrate(with_mfma, valu_per_mfma, iters=2000, workgroups_per_cu=4, threads=256, mode=CAL_UNIFORM):
+    """Runs the register-only calibration kernel (see jf_calibrate in the header) and returns a dict: seconds per launch
+    (events), the number of work items it ran (workgroups * waves * iters * 4; for CAL_SPLIT: items of the MFMA waves),
+    the resident waves per SIMD, and the shader clock in MHz the kernel ran at (cycles / wall-clock time, from the
+    per-workgroup readings)."""
+    props = torch.cuda.get_device_properties(0)
+    cus = props.multi_processor_count
     wgs = cus * workgroups_per_cu
+    waves = threads // 64
     scratch = torch.zeros(16, dtype=torch.float32, device="cuda")
-    run = lambda: check(lib().jf_calibrate(with_mfma, valu_per_mfma, iters, wgs, _ptr(scratch), _stream()))
+    clocks = torch.zeros(2 * wgs, dtype=torch.int64, device="cuda")
+    run = lambda: check(lib().jf_calibrate(mode, with_mfma, valu_per_mfma, iters, wgs, threads, _ptr(scratch), _ptr(clocks),
+                                           _stream()))
     run()
     e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
     e0.record()
@@ -432,4 +442,16 @@ def calibrate(with_mfma, valu_per_mfma, iters=2000, workgroups_per_cu=4):
         run()
     e1.record()
     torch.cuda.synchronize()
-    return e0.elapsed_time(e1) * 1e-3 / 3, wgs * 4 * iters * 4
+    c = clocks.view(wgs, 2).double().sum(0)
+    wall_hz = _wall_clock_hz()
+    items = wgs * (waves // 2 if mode == CAL_SPLIT else waves) * iters * 4
+    return {"seconds": e0.elapsed_time(e1) * 1e-3 / 3, "items": items, "waves_per_simd": workgroups_per_cu * waves / 4,
+            "shader_MHz": float(c[0] / c[1]) * wall_hz / 1e6, "simds": cus * 4}
+
+
+def _wall_clock_hz():
+    """Rate of the constant clock the kernel's wall-clock readings count in."""
+    khz = lib().jf_wall_clock_khz()
+    if khz <= 0:
+        raise RuntimeError("jf_wall_clock_khz: the device does not report a wall clock rate")
+    return khz * 1e3

@@ -22,7 +22,7 @@
  * Deliberate definitions where the reference is undefined or not reproducible:
  *   - all-zero block: scale 0, codes 0 (reference: 0/0 -> NaN)
  *   - divisions are IEEE (reference is built with -use_fast_math, setup.py:28)
- *   - stochastic rounding noise comes from Philox4x32-10 keyed by (seed, element
+ *   - stochastic rounding noise comes from Philox4x32-7 keyed by (seed, element
  *     index) instead of curand keyed by threadIdx (…Stochastic.cu:311-312,416)
  *     or a materialised torch noise tensor (Jetfire/Nonlinear/quantize.py:143-146)
  *   - stochastic GEMM epilogue clamps to +-127 (reference wraps 128 -> -128)
@@ -37,15 +37,15 @@
 #define QB 32
 
 /* ------------------------------------------------------------------------- */
-/* Philox4x32-10 (Salmon et al., "Parallel random numbers: as easy as 1,2,3",  */
-/* SC'11; the generator behind curandStatePhilox4_32_10_t used at             */
-/* …Stochastic.cu:311).  Pinned by the Random123 known-answer vectors.        */
+/* Philox4x32-R (Salmon et al., "Parallel random numbers: as easy as 1,2,3",   */
+/* SC'11; with R = 10 the generator behind curandStatePhilox4_32_10_t used at */
+/* …Stochastic.cu:311).  Pinned by the Random123 known-answer vectors (R=10). */
 /* ------------------------------------------------------------------------- */
-void jfo_philox4x32_10(const uint32_t ctr[4], const uint32_t key[2], uint32_t out[4])
+void jfo_philox4x32(const uint32_t ctr[4], const uint32_t key[2], int rounds, uint32_t out[4])
 {
     uint32_t c0 = ctr[0], c1 = ctr[1], c2 = ctr[2], c3 = ctr[3];
     uint32_t k0 = key[0], k1 = key[1];
-    for (int r = 0; r < 10; ++r) {
+    for (int r = 0; r < rounds; ++r) {
         uint64_t p0 = (uint64_t)0xD2511F53u * c0;
         uint64_t p1 = (uint64_t)0xCD9E8D57u * c2;
         uint32_t n0 = (uint32_t)(p1 >> 32) ^ c1 ^ k0;
@@ -59,9 +59,19 @@ void jfo_philox4x32_10(const uint32_t ctr[4], const uint32_t key[2], uint32_t ou
     out[0] = c0; out[1] = c1; out[2] = c2; out[3] = c3;
 }
 
+void jfo_philox4x32_10(const uint32_t ctr[4], const uint32_t key[2], uint32_t out[4])
+{
+    jfo_philox4x32(ctr, key, 10, out);
+}
+
+/* Rounds of the generator behind the rounding noise: 7, the smallest count Salmon et al. report as passing BigCrush
+ * (the kernels pay for every round with two quarter-rate multiplies per 8 elements).  The round function and key
+ * schedule are the ones the 10-round known answers pin. */
+#define JFO_NOISE_ROUNDS 7
+
 /*
  * Rounding noise for element `e` (flat row-major index r*C+c of the OUTPUT
- * tensor).  One Philox call serves 8 consecutive elements, 16 bits each:
+ * tensor).  One Philox4x32-7 call serves 8 consecutive elements, 16 bits each:
  *   counter = (offset + e/8) as 64-bit in words 0,1; words 2,3 = 0; key = seed
  *   h = 16-bit field (e%8): word (e%8)/2, low half for even e, high half for odd
  *   noise = (h + 0.5) * 2^-16 - 0.5      in (-0.5, 0.5), symmetric, exact in f32
@@ -74,7 +84,7 @@ float jfo_sr_noise(uint64_t seed, uint64_t offset, uint64_t e)
     uint32_t ctr[4] = { (uint32_t)c, (uint32_t)(c >> 32), 0u, 0u };
     uint32_t key[2] = { (uint32_t)seed, (uint32_t)(seed >> 32) };
     uint32_t o[4];
-    jfo_philox4x32_10(ctr, key, o);
+    jfo_philox4x32(ctr, key, JFO_NOISE_ROUNDS, o);
     unsigned lane = (unsigned)(e & 7u);
     uint32_t w = o[lane >> 1];
     uint32_t h = (lane & 1u) ? (w >> 16) : (w & 0xFFFFu);
@@ -483,7 +493,9 @@ void jfo_rowstats(const int8_t *q, const float *s, int R, int C, float eps, floa
     }
 }
 
-/* layernorm.py:74-190 with a real beta: y = fmaf((x-mean)*rstd, gamma, beta) */
+/* layernorm.py:74-190 with a real beta.  Dequantisation and normalisation are ONE fma per element with two constants
+ * per (row, block): a = s*rstd, b = -(mean*rstd), xhat = fmaf(q, a, b), y = fmaf(xhat, gamma, beta)   (this library's
+ * definition: the reference dequantises in binary16 first, layernorm.py:131; pinned to torch's layer_norm by tolerance) */
 void jfo_layernorm_fwd(const int8_t *q, const float *s, int R, int C, const float *gamma, const float *beta,
                        const float *mean, const float *rstd, int8_t *qy, float *sy)
 {
@@ -494,8 +506,8 @@ void jfo_layernorm_fwd(const int8_t *q, const float *s, int R, int C, const floa
         float sc = s[rb * SC + cb];
         for (int i = 0; i < QB; ++i)
             for (int j = 0; j < QB; ++j) {
-                float x = (float)q[o + (size_t)i * C + j] * sc;
-                float xh = (x - mean[rb * QB + i]) * rstd[rb * QB + i];
+                float a = sc * rstd[rb * QB + i], b = -(mean[rb * QB + i] * rstd[rb * QB + i]);
+                float xh = fmaf((float)q[o + (size_t)i * C + j], a, b);
                 tmp[i * QB + j] = fmaf(xh, gamma[cb * QB + j], beta ? beta[cb * QB + j] : 0.0f);
             }
         quantize_block(tmp, QB, qy + o, C, &sy[rb * SC + cb], 0, 0, 0, (uint64_t)o, (uint64_t)C, 0.0f, 0);
@@ -506,8 +518,9 @@ void jfo_layernorm_fwd(const int8_t *q, const float *s, int R, int C, const floa
  * LayerNorm backward, full-row (textbook) form of layernorm.py:197-402:
  *   wdy = gamma*dy; c1 = mean_row(xhat*wdy); c2 = mean_row(wdy)
  *   dx = (wdy - fmaf(xhat, c1, c2)) * rstd ;  dgamma = sum_rows dy*xhat ; dbeta = sum_rows dy
- * Row sums are defined as: 16-column partials (ascending, fmaf / add chain from 0),
- * then the C/16 partials added ascending.  c1 = sum/C.
+ * with xhat = fmaf(q_x, s_x*rstd, -(mean*rstd)) as in the forward and dy = q_g*s_g.
+ * Row sums are defined as: 16-column partials (ascending, fmaf / add chain from 0), the two partials of a
+ * block added; T_j = sum of the blocks j, j+8, ... ascending; S = ((T0+T1)+(T2+T3)) + ((T4+T5)+(T6+T7)).  c1 = S/C.
  * (The reference reduces c1,c2 over its 128-column tile only, :331-332 -- wrong for C>128.)
  */
 void jfo_layernorm_bwd(const int8_t *qx, const float *sx, const int8_t *qg, const float *sg, int R, int C,
@@ -519,22 +532,29 @@ void jfo_layernorm_bwd(const int8_t *qx, const float *sx, const int8_t *qg, cons
     float *c1 = (float *)malloc(sizeof(float) * R), *c2 = (float *)malloc(sizeof(float) * R);
     #pragma omp parallel for schedule(static)
     for (int r = 0; r < R; ++r) {
-        float t1 = 0.0f, t2 = 0.0f;
-        for (int h = 0; h < C / 16; ++h) {
-            float p1 = 0.0f, p2 = 0.0f;
-            float scx = sx[(r / QB) * SC + h / 2], scg = sg[(r / QB) * SC + h / 2];
-            for (int j = 0; j < 16; ++j) {
-                int c = h * 16 + j;
-                float x = (float)qx[(size_t)r * C + c] * scx;
-                float g = (float)qg[(size_t)r * C + c] * scg;
-                float xh = (x - mean[r]) * rstd[r];
-                float wdy = gamma[c] * g;
-                p1 = fmaf(xh, wdy, p1);
-                p2 = p2 + wdy;
+        /* per block: fma / add chains over columns 0..15 and 16..31, added; per row: T_j = blocks j, j+8, ... ascending,
+         * then ((T0+T1)+(T2+T3)) + ((T4+T5)+(T6+T7))  (the order the kernels reduce in) */
+        float t1[8] = { 0 }, t2[8] = { 0 };
+        float bx = -(mean[r] * rstd[r]);
+        for (int cb = 0; cb < SC; ++cb) {
+            float ax = sx[(r / QB) * SC + cb] * rstd[r], scg = sg[(r / QB) * SC + cb];
+            float h1[2], h2[2];
+            for (int h = 0; h < 2; ++h) {
+                float p1 = 0.0f, p2 = 0.0f;
+                for (int j = 0; j < 16; ++j) {
+                    int c = cb * QB + h * 16 + j;
+                    float xh = fmaf((float)qx[(size_t)r * C + c], ax, bx);
+                    float wdy = gamma[c] * ((float)qg[(size_t)r * C + c] * scg);
+                    p1 = fmaf(xh, wdy, p1);
+                    p2 = p2 + wdy;
+                }
+                h1[h] = p1; h2[h] = p2;
             }
-            t1 = t1 + p1; t2 = t2 + p2;
+            t1[cb & 7] = t1[cb & 7] + (h1[0] + h1[1]);
+            t2[cb & 7] = t2[cb & 7] + (h2[0] + h2[1]);
         }
-        c1[r] = t1 / (float)C; c2[r] = t2 / (float)C;
+        c1[r] = (((t1[0] + t1[1]) + (t1[2] + t1[3])) + ((t1[4] + t1[5]) + (t1[6] + t1[7]))) / (float)C;
+        c2[r] = (((t2[0] + t2[1]) + (t2[2] + t2[3])) + ((t2[4] + t2[5]) + (t2[6] + t2[7]))) / (float)C;
     }
     FOR_BLOCKS(R, C) {
         float tmp[QB * QB];
@@ -543,10 +563,8 @@ void jfo_layernorm_bwd(const int8_t *qx, const float *sx, const int8_t *qg, cons
         for (int i = 0; i < QB; ++i)
             for (int j = 0; j < QB; ++j) {
                 int r = rb * QB + i, c = cb * QB + j;
-                float x = (float)qx[o + (size_t)i * C + j] * scx;
-                float g = (float)qg[o + (size_t)i * C + j] * scg;
-                float xh = (x - mean[r]) * rstd[r];
-                float wdy = gamma[c] * g;
+                float xh = fmaf((float)qx[o + (size_t)i * C + j], scx * rstd[r], -(mean[r] * rstd[r]));
+                float wdy = gamma[c] * ((float)qg[o + (size_t)i * C + j] * scg);
                 tmp[i * QB + j] = (wdy - fmaf(xh, c1[r], c2[r])) * rstd[r];
             }
         quantize_block(tmp, QB, qdx + o, C, &sdx[rb * SC + cb], stochastic, seed, offset, (uint64_t)o, (uint64_t)C, 0.0f, 0);
@@ -556,9 +574,8 @@ void jfo_layernorm_bwd(const int8_t *qx, const float *sx, const int8_t *qg, cons
         for (int c = 0; c < C; ++c) {
             double a = 0.0, b = 0.0;       /* fp output: tolerance-compared, so a careful sum */
             for (int r = 0; r < R; ++r) {
-                float x = (float)qx[(size_t)r * C + c] * sx[(r / QB) * SC + c / QB];
                 float g = (float)qg[(size_t)r * C + c] * sg[(r / QB) * SC + c / QB];
-                float xh = (x - mean[r]) * rstd[r];
+                float xh = fmaf((float)qx[(size_t)r * C + c], sx[(r / QB) * SC + c / QB] * rstd[r], -(mean[r] * rstd[r]));
                 a += (double)g * (double)xh; b += (double)g;
             }
             if (dgamma) dgamma[c] = (float)a;

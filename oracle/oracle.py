@@ -48,6 +48,7 @@ _f = C.c_float
 
 def _declare(L):
     L.jfo_philox4x32_10.argtypes = [_p, _p, _p]
+    L.jfo_philox4x32.argtypes = [_p, _p, _i, _p]
     L.jfo_sr_noise.argtypes = [_u64, _u64, _u64]
     L.jfo_sr_noise.restype = _f
     L.jfo_f32_to_f16_bits.argtypes = [_f]
@@ -106,6 +107,17 @@ def philox4x32_10(ctr, key):
     k = np.asarray(key, dtype=np.uint32).copy()
     o = np.zeros(4, dtype=np.uint32)
     lib().jfo_philox4x32_10(_ptr(c), _ptr(k), _ptr(o))
+    return o
+
+
+NOISE_ROUNDS = 7            # rounds of the generator behind sr_noise (JFO_NOISE_ROUNDS)
+
+
+def philox4x32(ctr, key, rounds):
+    c = np.asarray(ctr, dtype=np.uint32).copy()
+    k = np.asarray(key, dtype=np.uint32).copy()
+    o = np.zeros(4, dtype=np.uint32)
+    lib().jfo_philox4x32(_ptr(c), _ptr(k), rounds, _ptr(o))
     return o
 
 
