@@ -118,6 +118,22 @@ def fused_fc_gelu(jf, torch, ops):
     return out
 
 
+def fused_fc2_dgrad_gelu_bwd(jf, torch, ops):
+    """The fc2 activation-gradient GEMM followed by the GELU backward kernel against the GEMM with the GELU backward in
+    its epilogue (same bits); the layer's quantised input stands in for the GELU's saved input (same shape)."""
+    o = ops[3]                                                     # fc2: 6400 -> 1600, so dX is [8192, 6400]
+    sg, sw = o["sg"].t(), o["sw"]
+
+    def separate():
+        q, s = jf.igemm_block_q(o["qg"], o["qw"], sg, sw, jf.B_KN, rounding=jf.ROUND_STOCHASTIC, seed=1, offset=0)
+        return jf.gelu_bwd(o["qx"], o["sx"], q, s, jf.GELU_ERF, jf.ROUND_STOCHASTIC, seed=2, offset=0)
+
+    def fused():
+        return jf.igemm_block_q_gelu_bwd(o["qg"], o["qw"], sg, sw, o["qx"], o["sx"], jf.GELU_ERF, jf.ROUND_STOCHASTIC,
+                                         seed=1, offset=0, gelu_seed=2, gelu_offset=0)
+    return {"gemm_then_gelu_bwd_us": round(timed_us(torch, separate, 30), 1), "fused_us": round(timed_us(torch, fused, 30), 1)}
+
+
 def deep_k_weight_gradients(jf, torch):
     """Weight gradients of BASELINE config 2 (GPT-2 small, 12288 tokens) and the smallest one of the XL set: few output
     tiles over a deep K.  One accumulation chain per output (the reference's arithmetic) against the library's K split
@@ -503,6 +519,7 @@ def main():
         out["memory_bound_kernels"] = nonlinear_extras(jf, torch)
         out["deep_k_weight_gradients"] = deep_k_weight_gradients(jf, torch)
         out["fc_forward_with_gelu"] = fused_fc_gelu(jf, torch, ops)
+        out["fc2_dgrad_with_gelu_backward"] = fused_fc2_dgrad_gelu_bwd(jf, torch, ops)
         out["xl_block_forward_backward"] = recipe_block(torch)
     if not a.no_cpu:
         out["cpu_baseline"] = cpu_baseline(ops, a.cpu_rows)

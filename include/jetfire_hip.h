@@ -144,6 +144,18 @@ int jf_igemm_block_q_gelu(const int8_t *A, const int8_t *B, const void *sa, cons
                           int scale_dtype, int sa_layout, int sb_layout, int gelu_approx, float gelu_amax_eps,
                           jf_stream_t stream);
 
+/* The activation-gradient GEMM (A = dY [M,K], B = W [K,N], stochastic rounding with (seed, offset)) with the GELU
+ * backward fused into its epilogue: (C, sc) is what jf_gelu_bwd(Xq, Xs, <the GEMM's requantised output>, ...,
+ * gelu_rounding, gelu_seed, gelu_offset) would return, bit for bit (the intermediate gradient is requantised to INT8
+ * with its scale rounded to scale_dtype exactly as jf_igemm_block_q stores it, but never written).  (Xq, Xs): the
+ * GELU's forward input, an [M,N] block tensor.  Replaces the pair igemm_output_int_quantize_stochastic
+ * (include/igemm.h:79-90) + int8_gelu_backward (Jetfire/Nonlinear/gelu_bwd.py:173-215) of the recipe's MLP backward
+ * (INT8_GPT2/qmodel.py:249-253), whose intermediate gradient has no other reader. */
+int jf_igemm_block_q_gelu_bwd(const int8_t *A, const int8_t *B, const void *sa, const void *sb, const int8_t *Xq,
+                              const void *Xs, int8_t *C, void *sc, int M, int N, int K, int scale_dtype, int sa_layout,
+                              int sb_layout, int gelu_approx, uint64_t seed, uint64_t offset, int gelu_rounding,
+                              uint64_t gelu_seed, uint64_t gelu_offset, jf_stream_t stream);
+
 /* Block quantise x[R,C] (x_dtype: JF_FP_*) -> (q, s); optionally also qT[C,R] = q transposed.
  * Replaces int8_quantize (Jetfire/Nonlinear/quantize.py:128-164) and, with qT != NULL,
  * int8_quantize_transpose (Jetfire/Nonlinear/quantize_transpose.py:131-171). */

@@ -107,3 +107,26 @@ def int8_linear_backward(X8_3D, SX16_3D, G8_3D, SG16_3D, G8T, W8, SW16, B, stoch
     if not dgrad_quantize:
         return _dequant_like(gx8, gsx, tuple(G8_3D.shape[:-1])), gw
     return (gx8.reshape(*G8_3D.shape[:-1], c_in), gsx.reshape(*SG16_3D.shape[:-1], SW16.shape[1]), gw)
+
+
+def int8_linear_backward_gelu(X8_3D, SX16_3D, G8_3D, SG16_3D, W8, SW16, PRE8_3D, SPRE16_3D, B, approximate="none",
+                              stochastic=True, wgrad_splitk=1):
+    """int8_linear_backward(...) followed by int8_gelu_backward(PRE8, SPRE, <its activation gradient>, ...), with the
+    GELU backward running in the epilogue of the activation-gradient GEMM (no counterpart in the reference, whose MLP
+    backward runs the two back to back, qmodel.py:249-253).  X8 / SX: the linear layer's input (= the GELU's output),
+    PRE8 / SPRE: the GELU's input; G8 [BS,T,N], W8 [N,K].  Returns (GPRE8, GSPRE, GW): the gradient with respect to the
+    GELU's input, requantised (`stochastic` as in int8_gelu_backward), and the weight gradient; bit-identical to the
+    two separate calls (which draw their rounding noise in the same order)."""
+    _check_block(B)
+    if approximate not in ("none", "tanh"):
+        raise RuntimeError("approximate must be 'none' or 'tanh'")
+    g2, sg2 = _flat2(G8_3D).contiguous(), _flat2(SG16_3D).contiguous()
+    x2, sx2 = _flat2(X8_3D).contiguous(), _flat2(SX16_3D).contiguous()
+    p2, sp2 = _flat2(PRE8_3D).contiguous(), _flat2(SPRE16_3D).contiguous()
+    tokens, c_out = g2.shape
+    c_in = W8.shape[1]
+    gp8, gsp = _jf.igemm_block_q_gelu_bwd(g2, W8.contiguous(), _k_major(sg2), SW16, p2, sp2,
+                                          _jf.GELU_TANH if approximate == "tanh" else _jf.GELU_ERF,
+                                          _jf.ROUND_STOCHASTIC if stochastic else _jf.ROUND_NEAREST)
+    gw = BQC.igemm_output_fp_no_quantize(g2.t(), x2, sg2, sx2, c_out, c_in, tokens, wgrad_splitk)
+    return (gp8.reshape(*G8_3D.shape[:-1], c_in), gsp.reshape(*SG16_3D.shape[:-1], SW16.shape[1]), gw)

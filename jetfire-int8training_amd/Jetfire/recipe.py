@@ -19,7 +19,7 @@ import torch
 import torch.nn as nn
 import torch.nn.functional as F
 
-from Linear import int8_linear_backward, int8_linear_forward, int8_linear_forward_gelu
+from Linear import int8_linear_backward, int8_linear_backward_gelu, int8_linear_forward, int8_linear_forward_gelu
 from Nonlinear import (int8_add_Ifp_Ig16_Ofp_Og, int8_add_Ifp_Ig16_Ofp_Og_MeanVar, int8_gelu_backward,
                        int8_layernorm_backward, int8_layernorm_forward, int8_quantize)
 
@@ -153,8 +153,9 @@ class MLPResidual(torch.autograd.Function):
     def backward(ctx, fpg, qg, sg, _m, _r):
         qx, sx, qn, sn, qh, sh, qa, sa, qw1, sw1, qw2, sw2, ln_w, mean, rstd = ctx.saved_tensors
         qg = _as_s8(qg)
-        qg, sg, gw2 = int8_linear_backward(qa, sa, qg, sg, None, qw2, sw2, QB, stochastic=True, wgrad_splitk=0)
-        qg, sg = int8_gelu_backward(qh, sh, qg, sg, QB, stochastic=True)
+        # proj's backward with the GELU backward in the epilogue of its activation-gradient GEMM (one kernel for
+        # int8_linear_backward's dgrad + int8_gelu_backward, same bits)
+        qg, sg, gw2 = int8_linear_backward_gelu(qa, sa, qg, sg, qw2, sw2, qh, sh, QB, stochastic=True, wgrad_splitk=0)
         qg, sg, gw1 = int8_linear_backward(qn, sn, qg, sg, None, qw1, sw1, QB, stochastic=True, wgrad_splitk=0)
         qg, sg, g_ln = int8_layernorm_backward(qx, sx, qg, sg, ln_w, QB, mean, rstd, stochastic=True)
         res_g, qg, sg = int8_add_Ifp_Ig16_Ofp_Og(fpg.contiguous(), qg, sg, QB, stochastic=True)

@@ -259,17 +259,10 @@ __global__ __launch_bounds__(NT) void gelu_bwd_kernel(const int8_t *qx, const ST
         v4i cx, cg; float scx, scg;
         inx.template take<SLOT>(cx, scx);
         ing.template take<SLOT>(cg, scg);
-        float x[16], g[16];
-        unpack16(cg, scg, g);
-        fill_code_table(tab, lane, scx, f0, [](float v, float &a, float &b) { dgelu_pair<APPROX>(v, a, b); });
-        gather16(tab, cx, x);
-        table_done();
+        float scale;
+        v4i codes = gelu_bwd_block<APPROX>(cx, scx, cg, scg, f0, tab, lane, rounding, seed, offset, e0, &scale);
         inx.template refill<SLOT>();                               // after the last use of the slot's registers
         ing.template refill<SLOT>();
-#pragma unroll
-        for (int k = 0; k < 16; ++k) x[k] = x[k] * g[k];
-        float scale;
-        v4i codes = quantize16(x, 0.0f, rounding, seed, offset, e0, &scale);
         *reinterpret_cast<v4i *>(qy + e0) = codes;
         if (lane == 0) store_scale(sy, w.rb * SC + w.cb, scale);
     });

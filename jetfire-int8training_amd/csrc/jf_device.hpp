@@ -435,6 +435,23 @@ __device__ __forceinline__ v4i gelu_fwd_block(v4i c, float sc, float f0, float a
     return codes;
 }
 
+// GELU backward of one block: codes / scale of the forward input (cx, scx) and of the incoming gradient (cg, scg), 16
+// per lane in the row layout -> packed codes of gelu'(x) * g requantised with `rounding`, *scale_out = its scale.
+// tab: 256 floats of LDS private to the wave; f0 = gelu'(+0), evaluated by the caller once.  (gelu_bwd.py:28-171)
+template <int APPROX>
+__device__ __forceinline__ v4i gelu_bwd_block(v4i cx, float scx, v4i cg, float scg, float f0, float *tab, int lane,
+                                              int rounding, uint64_t seed, uint64_t offset, uint64_t e0, float *scale_out)
+{
+    float x[16], g[16];
+    unpack16(cg, scg, g);
+    fill_code_table(tab, lane, scx, f0, [](float v, float &a, float &b) { dgelu_pair<APPROX>(v, a, b); });
+    gather16(tab, cx, x);
+    table_done();
+#pragma unroll
+    for (int k = 0; k < 16; ++k) x[k] = x[k] * g[k];
+    return quantize16(x, 0.0f, rounding, seed, offset, e0, scale_out);
+}
+
 // ---------------------------------------------------------------------------------------------
 // host-side argument checks shared by the entry points
 // The kernels exist as gfx950 code objects only: say so instead of failing at launch with "no binary for GPU".

@@ -39,7 +39,9 @@ constexpr int MAX_DEVICES = 64;                    // devices a process may use 
 constexpr int EPI_LD = 36;                          // floats per staged row (32 + pad, keeps 16B alignment)
 
 // EPI_QG: EPI_Q (deterministic) followed by the GELU forward of the block just requantised: two block tensors leave
-enum Epilogue { EPI_S32 = 0, EPI_FP = 1, EPI_Q = 2, EPI_QG = 3 };
+// EPI_QB: EPI_Q (stochastic: an activation gradient) followed by the GELU backward of the block just requantised against
+//         the saved forward input of the GELU: only the result of the GELU backward leaves
+enum Epilogue { EPI_S32 = 0, EPI_FP = 1, EPI_Q = 2, EPI_QG = 3, EPI_QB = 4 };
 
 struct GemmArgs {
     const int8_t *A;      // [M, lda] (K-contiguous) or, for the AKM kernels, [K, lda] (M-contiguous rows)
@@ -61,6 +63,10 @@ struct GemmArgs {
     void *C2, *sc2;       // s8 [M, N], [M/32, N/32]: GELU of the requantised result   (EPI_QG)
     int gelu_approx;      // JF_GELU_*
     float gelu_eps;       // added to the GELU output's block absmax (the reference: 5e-5, gelu_fwd.py:93)
+    const int8_t *Xq;     // s8 [M, N]: forward input of the GELU   (EPI_QB)
+    const void *Xs;       // [M/32, N/32]
+    uint64_t seed2, offset2;   // noise of the GELU backward's own requantisation   (EPI_QB)
+    int rounding2;        // JF_ROUND_NEAREST / JF_ROUND_STOCHASTIC   (EPI_QB)
 };
 
 // Logical tile (and K split) of this workgroup.  Workgroups are dealt round-robin to the 8 XCDs, each with a
@@ -577,7 +583,7 @@ __global__ __launch_bounds__(64 * WGM * WGN, WGPC * WGM * WGN / 4) void igemm_nt
     float *patch = reinterpret_cast<float *>(smem) + wave * (QB * EPI_LD);
     unsigned char *tile = smem + NW * (QB * EPI_LD) * sizeof(float);       // [BM][BN * out_bytes]
     const int rrow = lane >> 1, rcol = (lane & 1) * 16;
-    constexpr bool QUANT = EPI == EPI_Q || EPI == EPI_QG;
+    constexpr bool QUANT = EPI == EPI_Q || EPI == EPI_QG || EPI == EPI_QB;
     const float biasmax = (QUANT && p.biasmax) ? p.biasmax[0] : 0.0f;
     const int out_bytes = QUANT ? 1 : (EPI == EPI_FP && p.out_dtype != JF_FP_F32 ? 2 : 4);   // uniform
     unsigned char *tile2 = tile + BM * BN;                    // EPI_QG: image of the second output
@@ -586,6 +592,25 @@ __global__ __launch_bounds__(64 * WGM * WGN, WGPC * WGM * WGN / 4) void igemm_nt
         float zero = 0.0f;
         asm volatile("" : "+v"(zero));
         gelu_f0 = p.gelu_approx == JF_GELU_TANH ? gelu<JF_GELU_TANH>(zero) : gelu<JF_GELU_ERF>(zero);
+    }
+    // EPI_QB: the saved forward input of this wave's blocks is requested now, so that it has arrived when the
+    // requantisation of the first block is done
+    v4i xq_codes[WBM][WBN];
+    float xq_scale[WBM][WBN];
+    if (EPI == EPI_QB) {
+        float zero = 0.0f;
+        asm volatile("" : "+v"(zero));
+        gelu_f0 = p.gelu_approx == JF_GELU_TANH ? dgelu<JF_GELU_TANH>(zero) : dgelu<JF_GELU_ERF>(zero);
+#pragma unroll
+        for (int i = 0; i < WBM; ++i)
+#pragma unroll
+            for (int j = 0; j < WBN; ++j) {
+                const int bm = m0 + (wm * WBM + i) * QB, bn = n0 + (wn * WBN + j) * QB;
+                if (bm < p.M && bn < p.N) {
+                    xq_codes[i][j] = *reinterpret_cast<const v4i *>(p.Xq + (size_t)(bm + rrow) * p.N + bn + rcol);
+                    xq_scale[i][j] = load_scale(reinterpret_cast<const ST *>(p.Xs), (bm / QB) * SN + bn / QB);
+                }
+            }
     }
 
 #pragma unroll
@@ -676,6 +701,19 @@ __global__ __launch_bounds__(64 * WGM * WGN, WGPC * WGM * WGN / 4) void igemm_nt
                     codes.z = (int)round_clamp_pack4(t[8], t[9], t[10], t[11]);
                     codes.w = (int)round_clamp_pack4(t[12], t[13], t[14], t[15]);
                 }
+                if (EPI == EPI_QB) {
+                    // GELU backward of the gradient block as a reader of the stored tensor would see it (codes x the scale
+                    // rounded to ST) against the saved forward input, with the wave's patch (free again) as the code table
+                    const float stored = (float)(ST)scale;
+                    float scale2;
+                    codes = p.gelu_approx == JF_GELU_TANH
+                        ? gelu_bwd_block<JF_GELU_TANH>(xq_codes[i][j], xq_scale[i][j], codes, stored, gelu_f0, patch, lane,
+                                                       p.rounding2, p.seed2, p.offset2, (uint64_t)e0, &scale2)
+                        : gelu_bwd_block<JF_GELU_ERF>(xq_codes[i][j], xq_scale[i][j], codes, stored, gelu_f0, patch, lane,
+                                                      p.rounding2, p.seed2, p.offset2, (uint64_t)e0, &scale2);
+                    scale = scale2;
+                    wave_sync();                              // the table is the next block's patch
+                }
                 *reinterpret_cast<v4i *>(tile + (size_t)trow * BN + tcol) = codes;
                 if (lane == 0) store_scale(reinterpret_cast<ST *>(p.sc), (bm / QB) * SN + bn / QB, scale);
                 if (EPI == EPI_QG) {
@@ -752,7 +790,7 @@ static int launch_gemm_cfg(const GemmArgs &a, hipStream_t st)
 {
     constexpr int BM = QB * WBM * WGM, BN = QB * WBN * WGN, NT = 64 * WGM * WGN;
     constexpr int RING = NSTAGE * (BM + BN) * ROW_BYTES + WGM * WGN * NSTAGE * 256;   // operand ring + per-wave scale patches
-    constexpr int PATCH = WGM * WGN * QB * EPI_LD * (int)sizeof(float) + (EPI == EPI_S32 ? 0 : BM * BN * (EPI == EPI_Q ? 1 : 2));   // + tile image(s): bytes, 2-byte values, or two of bytes
+    constexpr int PATCH = WGM * WGN * QB * EPI_LD * (int)sizeof(float) + (EPI == EPI_S32 ? 0 : BM * BN * ((EPI == EPI_Q || EPI == EPI_QB) ? 1 : 2));   // + tile image(s): bytes, 2-byte values, or two of bytes
     constexpr int SMEM = RING > PATCH ? RING : PATCH;
     if (!device_is_gfx950()) return JF_ERR_DEVICE;
     GemmArgs p = a;
@@ -832,6 +870,9 @@ template <int EPI, typename ST> static int launch_gemm(const GemmArgs &a, hipStr
     if constexpr (EPI == EPI_QG) {                            // the forward form only: A [M,K], B [N,K]
         if (a_km || b_kn) return JF_ERR_UNSUPPORTED;
         return launch_gemm_cfg<EPI, ST, 2, 4, 2, 2, 0>(a, st);
+    } else if constexpr (EPI == EPI_QB) {                     // the activation-gradient form only: A [M,K], B [K,N]
+        if (a_km || !b_kn) return JF_ERR_UNSUPPORTED;
+        return launch_gemm_cfg<EPI, ST, 2, 4, 2, 2, 1>(a, st);
     } else {
         if (a_km) {
             if constexpr (EPI == EPI_FP) {
@@ -1074,6 +1115,30 @@ int jf_igemm_block_q_gelu(const int8_t *A, const int8_t *B, const void *sa, cons
         return JF_ERR_ENUM;
     hipStream_t st = (hipStream_t)stream;
     return scale_dtype == JF_SCALE_F16 ? launch_gemm<EPI_QG, half_t>(a, st, false) : launch_gemm<EPI_QG, float>(a, st, false);
+}
+
+int jf_igemm_block_q_gelu_bwd(const int8_t *A, const int8_t *B, const void *sa, const void *sb, const int8_t *Xq,
+                              const void *Xs, int8_t *C, void *sc, int M, int N, int K, int scale_dtype, int sa_layout,
+                              int sb_layout, int gelu_approx, uint64_t seed, uint64_t offset, int gelu_rounding,
+                              uint64_t gelu_seed, uint64_t gelu_offset, jf_stream_t stream)
+{
+    int rc = check_gemm_common(A, B, C, M, N, K, JF_B_KN);
+    if (rc) return rc;
+    if (!sa || !sb || !sc || !Xq || !Xs) return JF_ERR_NULL;
+    if ((scale_dtype != JF_SCALE_F16 && scale_dtype != JF_SCALE_F32) ||
+        (gelu_approx != JF_GELU_ERF && gelu_approx != JF_GELU_TANH) ||
+        (gelu_rounding != JF_ROUND_NEAREST && gelu_rounding != JF_ROUND_STOCHASTIC)) return JF_ERR_ENUM;
+    if (!aligned16(Xq) || !scale_ptr_ok(sa, scale_dtype) || !scale_ptr_ok(sb, scale_dtype) || !scale_ptr_ok(Xs, scale_dtype))
+        return JF_ERR_ALIGN;
+    GemmArgs a = {};
+    a.A = A; a.B = B; a.sa = sa; a.sb = sb; a.C = C; a.sc = sc; a.Xq = Xq; a.Xs = Xs;
+    a.M = M; a.N = N; a.K = K; a.lda = K; a.ldb = N;
+    a.rounding = JF_ROUND_STOCHASTIC; a.seed = seed; a.offset = offset;
+    a.gelu_approx = gelu_approx; a.rounding2 = gelu_rounding; a.seed2 = gelu_seed; a.offset2 = gelu_offset;
+    if (!scale_strides(sa_layout, K, M / QB, a.sa_ks, a.sa_is) || !scale_strides(sb_layout, K, N / QB, a.sb_ks, a.sb_is))
+        return JF_ERR_ENUM;
+    hipStream_t st = (hipStream_t)stream;
+    return scale_dtype == JF_SCALE_F16 ? launch_gemm<EPI_QB, half_t>(a, st, true) : launch_gemm<EPI_QB, float>(a, st, true);
 }
 
 int jf_transpose_s8(const int8_t *in, int R, int C, int8_t *out, jf_stream_t stream)

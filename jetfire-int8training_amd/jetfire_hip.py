@@ -26,7 +26,7 @@ GELU_ERF, GELU_TANH = 0, 1
 
 EXPORTS = [
     "jf_error_string", "jf_igemm_workspace_bytes", "jf_igemm_s32", "jf_igemm_block_acc", "jf_igemm_block_fp",
-    "jf_igemm_splitk_plan", "jf_igemm_block_fp_workspace_bytes", "jf_igemm_block_q_gelu", "jf_igemm_block_fp_noalloc",
+    "jf_igemm_splitk_plan", "jf_igemm_block_fp_workspace_bytes", "jf_igemm_block_q_gelu", "jf_igemm_block_fp_noalloc", "jf_igemm_block_q_gelu_bwd",
     "jf_igemm_block_q", "jf_quantize", "jf_dequantize", "jf_transpose_s8", "jf_rowstats", "jf_layernorm_fwd",
     "jf_layernorm_bwd_workspace_bytes", "jf_layernorm_bwd", "jf_gelu_fwd", "jf_gelu_bwd", "jf_add", "jf_calibrate", "jf_wall_clock_khz",
 ]
@@ -50,6 +50,7 @@ def lib():
         L.jf_igemm_block_acc.argtypes = [_p, _p, _p, _i, _i, _i, _i, _p, _sz, _p]
         L.jf_igemm_block_fp.argtypes = [_p, _p, _p, _p, _p, _i, _i, _i, _i, _i, _i, _i, _i, _i, _i, _p, _sz, _p]
         L.jf_igemm_block_fp_noalloc.argtypes = [_p, _p, _p, _p, _p, _i, _i, _i, _i, _i, _i, _i, _i, _i, _i, _p]
+        L.jf_igemm_block_q_gelu_bwd.argtypes = [_p, _p, _p, _p, _p, _p, _p, _p, _i, _i, _i, _i, _i, _i, _i, _u64, _u64, _i, _u64, _u64, _p]
         L.jf_igemm_block_q_gelu.argtypes = [_p, _p, _p, _p, _p, _p, _p, _p, _p, _p, _i, _i, _i, _i, _i, _i, _i, _f, _p]
         L.jf_igemm_splitk_plan.argtypes = [_i, _i, _i, _i, C.POINTER(C.c_int), C.POINTER(C.c_int)]
         L.jf_igemm_block_fp_workspace_bytes.argtypes = [_i, _i, _i, _i, _i]
@@ -266,6 +267,27 @@ def igemm_block_q_gelu(A, B, sa, sb, approx=GELU_ERF, amax_eps=5e-5, bias=None, 
     check(lib().jf_igemm_block_q_gelu(_ptr(A), _ptr(B), _ptr(sa), _ptr(sb), _ptr(bias), _ptr(biasmax), _ptr(q), _ptr(s),
                                       _ptr(qg), _ptr(sg), M, N, K, code, la, lb, approx, amax_eps, _stream()))
     return q, s, qg, sg
+
+
+def igemm_block_q_gelu_bwd(A, B, sa, sb, xq, xs, approx=GELU_ERF, gelu_rounding=ROUND_STOCHASTIC, seed=None, offset=None,
+                           gelu_seed=None, gelu_offset=None):
+    """Activation-gradient GEMM (B as [K,N], stochastic rounding) with the GELU backward fused into its epilogue:
+    returns what gelu_bwd(xq, xs, *igemm_block_q(A, B, sa, sb, B_KN, rounding=ROUND_STOCHASTIC), approx, gelu_rounding)
+    returns (the two draw their noise in that order)."""
+    M, N, K, _, _ = _gemm_operands(A, B, B_KN)
+    code, la, lb = _gemm_scales(sa, sb, M, N, K)
+    R2, C2, code2 = _block_tensor(xq, xs, "x")
+    if (R2, C2, code2) != (M, N, code):
+        raise RuntimeError(f"x must be an [M,N]={M, N} block tensor with the scale dtype of sa / sb")
+    if gelu_rounding not in (ROUND_NEAREST, ROUND_STOCHASTIC):
+        raise RuntimeError("gelu_rounding must be ROUND_NEAREST or ROUND_STOCHASTIC")
+    seed, offset = _rng(ROUND_STOCHASTIC, M * N, seed, offset, A.device)
+    gelu_seed, gelu_offset = _rng(gelu_rounding, M * N, gelu_seed, gelu_offset, A.device)
+    out = torch.empty((M, N), dtype=torch.int8, device=A.device)
+    sc = torch.empty((M // QB, N // QB), dtype=sa.dtype, device=A.device)
+    check(lib().jf_igemm_block_q_gelu_bwd(_ptr(A), _ptr(B), _ptr(sa), _ptr(sb), _ptr(xq), _ptr(xs), _ptr(out), _ptr(sc), M, N, K,
+                                          code, la, lb, approx, seed, offset, gelu_rounding, gelu_seed, gelu_offset, _stream()))
+    return out, sc
 
 
 def igemm_block_q(A, B, sa, sb, b_layout=B_KN, bias=None, biasmax=None, rounding=ROUND_NEAREST, seed=None, offset=None):

@@ -340,3 +340,30 @@ def test_stochastic_ops_share_one_counter_source(oracle):
     assert again_spans == spans
     for a, b in zip(first, again):
         assert torch.equal(a, b)
+
+
+@pytest.mark.gpu
+def test_linear_backward_with_fused_gelu_backward():
+    """Linear.int8_linear_backward_gelu = int8_linear_backward then int8_gelu_backward, bit for bit, when both start
+    from the same generator state (the fused kernel draws its two noise streams in the order of the two calls)."""
+    from Linear import int8_linear_backward, int8_linear_backward_gelu
+    from Nonlinear import int8_gelu_backward, int8_quantize
+    BS, T, Cin, Cout = 2, 128, 160, 96
+    gsrc = torch.Generator().manual_seed(9)
+    pre = torch.randn(BS, T, Cin, generator=gsrc).cuda()                  # the GELU's input
+    act = torch.nn.functional.gelu(pre)                                   # the linear layer's input
+    w = (torch.randn(Cout, Cin, generator=gsrc) * 0.02).cuda()
+    g = (torch.randn(BS, T, Cout, generator=gsrc) * 1e-3).cuda()
+    qp, sp = int8_quantize(pre, 32)
+    qa, sa = int8_quantize(act, 32)
+    qw, sw = int8_quantize(w, 32)
+    qg, sg = int8_quantize(g, 32)
+    for approximate in ("none", "tanh"):
+        torch.manual_seed(31)
+        gx8, gsx, gw = int8_linear_backward(qa, sa, qg, sg, None, qw, sw, 32, stochastic=True, wgrad_splitk=0)
+        d8, ds = int8_gelu_backward(qp, sp, gx8, gsx, 32, stochastic=True, approximate=approximate)
+        torch.manual_seed(31)
+        f8, fs, fw = int8_linear_backward_gelu(qa, sa, qg, sg, qw, sw, qp, sp, 32, approximate=approximate, stochastic=True,
+                                               wgrad_splitk=0)
+        assert tuple(f8.shape) == (BS, T, Cin) and tuple(fs.shape) == (BS, T // 32, Cin // 32)
+        assert torch.equal(f8, d8) and torch.equal(fs, ds) and torch.equal(fw, gw)

@@ -51,7 +51,7 @@ def layer_inputs(T, Cin, Cout, seed, outliers):
     return x, w, dy
 
 
-def check_linear_layer(jf, oracle, T, Cin, Cout, seed, outliers, gelu=None):
+def check_linear_layer(jf, oracle, T, Cin, Cout, seed, outliers, gelu=None, gelu_bwd=False):
     """forward (deterministic), dgrad (stochastic), wgrad (one chain from a transposed copy; and, as the recipe runs it,
     from the gradient in place with the library's K split) of one linear layer on quantised synthetic data."""
     print(f"layer T={T} {Cin}->{Cout} seed={seed}", flush=True)
@@ -73,6 +73,13 @@ def check_linear_layer(jf, oracle, T, Cin, Cout, seed, outliers, gelu=None):
         assert torch.equal(fq, y) and torch.equal(fs, sy), "fused forward differs from the plain forward"
         g2, gs2 = jf.gelu_fwd(y, sy, gelu, eps)
         assert torch.equal(fg, g2) and torch.equal(fgs, gs2), "fused GELU differs from the GELU kernel"
+    if gelu_bwd:
+        # this layer's input is the output of a GELU: its backward runs in the epilogue of the dgrad GEMM (the recipe's
+        # MLP path); qx / sx stand in for the GELU's saved input, an [T, Cin] block tensor like the gradient
+        fb, fbs = jf.igemm_block_q_gelu_bwd(qg, qw, sg.t(), sw, qx, sx, jf.GELU_ERF, jf.ROUND_STOCHASTIC, seed=seed + 1,
+                                            offset=17, gelu_seed=seed + 2, gelu_offset=5)
+        b2, bs2 = jf.gelu_bwd(qx, sx, dx, sdx, jf.GELU_ERF, jf.ROUND_STOCHASTIC, seed=seed + 2, offset=5)
+        assert torch.equal(fb, b2) and torch.equal(fbs, bs2), "fused GELU backward differs from the GELU backward kernel"
     torch.cuda.synchronize()
     X, W, G, GT = (t.cpu().numpy() for t in (qx, qw, qg, qgT))
     SX, SW, SG = (t.cpu().numpy() for t in (sx, sw, sg))
@@ -90,6 +97,10 @@ def check_linear_layer(jf, oracle, T, Cin, Cout, seed, outliers, gelu=None):
         wq, wsc = oracle.requant(acc, stochastic=True, seed=seed + 1, offset=17 + r0 * Cin // 8)
         same(dx[rows], wq, f"dgrad codes rows {r0}")
         same(sdx[rb], wsc, f"dgrad scales rows {r0}")
+        if gelu_bwd:
+            wb, wbs = oracle.gelu_bwd(X[rows], SX[rb], wq, wsc, 0, True, seed + 2, 5 + r0 * Cin // 8)
+            same(fb[rows], wb, f"fused GELU backward codes rows {r0}")
+            same(fbs[rb], wbs, f"fused GELU backward scales rows {r0}")
     for r0 in strips(Cout):
         rows, rb = slice(r0, r0 + QB), slice(r0 // QB, r0 // QB + 1)
         sa = cont(SG[:, rb])
@@ -131,8 +142,9 @@ def test_cfg2_gpt2_small_layer(jf, oracle, name, Cin, Cout):
 @pytest.mark.parametrize("name,Cin,Cout,gelu", [("qkv", 1600, 4800, None), ("proj", 1600, 1600, None),
                                                ("fc", 1600, 6400, 0), ("fc2", 6400, 1600, None)])
 def test_cfg3_gpt2_xl_layer(jf, oracle, name, Cin, Cout, gelu):
-    """fc also runs the forward with the GELU fused into the epilogue (the recipe's MLP path)."""
-    check_linear_layer(jf, oracle, 8192, Cin, Cout, seed=0, outliers=True, gelu=gelu)
+    """fc also runs the forward with the GELU fused into the epilogue, fc2 the activation gradient with the GELU
+    backward fused into the epilogue (the recipe's MLP path)."""
+    check_linear_layer(jf, oracle, 8192, Cin, Cout, seed=0, outliers=True, gelu=gelu, gelu_bwd=name == "fc2")
 
 
 def test_cfg4_layernorm_full_size(jf, oracle):

@@ -474,3 +474,31 @@ def test_forward_gemm_with_fused_gelu(jf, oracle, M, N, K, f16, approx):
     same(qg, wg, "gelu codes")
     same(sg, wgs, "gelu scales")
     assert qg.cpu().numpy().any()
+
+
+@pytest.mark.parametrize("approx", [0, 1])
+@pytest.mark.parametrize("f16", [True, False])
+@pytest.mark.parametrize("M,N,K", [(128, 256, 96), (96, 160, 224), (256, 384, 544), (32, 32, 32)])
+def test_dgrad_gemm_with_fused_gelu_backward(jf, oracle, M, N, K, f16, approx):
+    """The fused entry point returns, bit for bit, what the stochastic activation-gradient GEMM and then the GELU
+    backward kernel return (with the same two noise streams), and what the oracle computes for that sequence."""
+    print(f"case dgrad+gelu_bwd M={M} N={N} K={K} f16={f16} approx={approx}", flush=True)
+    A, Bkn, sa, sb = make_problem(M * 2 + N + K * 3, M, N, K, f16)
+    rng = np.random.default_rng(M + N + K)
+    st = np.float16 if f16 else np.float32
+    sdt = "f16" if f16 else "f32"
+    xq = rand_codes(rng, (M, N))
+    xs = (rand_scales(rng, (M // QB, N // QB), lo=-6, hi=-4, f16=f16)).astype(np.float32)    # pre-activations of a few units
+    dA, dB, dsa, dsb, dxq, dxs = dev(A), dev(Bkn), dev(sa.astype(st)), dev(sb.astype(st)), dev(xq), dev(xs.astype(st))
+    for rounding2, stochastic2 in ((jf.ROUND_STOCHASTIC, True), (jf.ROUND_NEAREST, False)):
+        q, s = jf.igemm_block_q_gelu_bwd(dA, dB, dsa, dsb, dxq, dxs, approx, rounding2, seed=11, offset=3, gelu_seed=12, gelu_offset=40)
+        q0, s0 = jf.igemm_block_q(dA, dB, dsa, dsb, jf.B_KN, rounding=jf.ROUND_STOCHASTIC, seed=11, offset=3)
+        q1, s1 = jf.gelu_bwd(dxq, dxs, q0, s0, approx, rounding2, seed=12, offset=40)
+        assert torch.equal(q, q1) and torch.equal(s, s1)
+        wq, ws = oracle.igemm_block_q(A, Bkn, sa, sb, 1, stochastic=True, seed=11, offset=3, scale_dtype=sdt)
+        wg, wgs = oracle.gelu_bwd(xq, xs, wq, ws.astype(np.float32), approx, stochastic2, 12, 40, scale_dtype=sdt)
+        same(q, wg, "codes")
+        same(s, wgs, "scales")
+        assert q.cpu().numpy().any()
+    with pytest.raises(RuntimeError):
+        jf.igemm_block_q_gelu_bwd(dA, dB, dsa, dsb, dxq[:, : N // 2].contiguous(), dxs[:, : N // 64].contiguous(), approx)
