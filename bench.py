@@ -89,10 +89,27 @@ def dominant_kernel_roofline(jf, torch, ops, iters=200):
     torch.cuda.synchronize()
     avg_s = e0.elapsed_time(e1) * 1e-3 / iters
     achieved = 2.0 * M * N * K / avg_s / 1e12
+    # the same launch once more, right behind the timed ones (the clock has settled), with the kernel's profiling build:
+    # when each workgroup's phases began and ended and the shader clock its main loop ran at
+    tiles = ((M + 127) // 128) * ((N + 127) // 128)
+    ph = jf.igemm_phases(lambda: jf.igemm_block_q(o["qx"], o["qw"], o["sxT"], o["swT"], jf.B_NK), tiles)
+    us, mhz = ph["us"], float(ph["k_loop_MHz"].mean())
+    span_us = float(us[:, 5].max())
+    products = (M // 32) * (N // 32) * (K // 32)              # 32x32x32 block products = MFMA instructions
+    simds = 4 * torch.cuda.get_device_properties(0).multi_processor_count
+    d = us[:, 1:] - us[:, :-1]
+    phases = {"workgroups": tiles, "span_us": round(span_us, 1), "main_loop_shader_MHz": round(mhz),
+              "simd_cycles_per_block_product": round(span_us * mhz * simds / products, 1),
+              "mean_us": {k: round(float(d[:, i].mean()), 2) for i, k in
+                          enumerate(("prologue", "main_loop", "sync", "requantise", "store"))},
+              "note": "simd_cycles_per_block_product = span x clock x SIMDs / MFMA count: everything the kernel does, per "
+                      "MFMA; the register-only stream of one MFMA + 32 VALU instructions takes the cycles the calibration "
+                      "table gives for gemm_k_block_stream"}
     return {"bound": "mfma", "kernel": "igemm_nt_kernel<EPI_Q,f32> fc forward 8192x6400x1600",
             "achieved": round(achieved, 2), "peak": INT8_PEAK_TOPS, "unit": "TOP/s",
             "frac": round(achieved / INT8_PEAK_TOPS, 4), "avg_launch_us": round(avg_s * 1e6, 2),
-            "launches": iters, "traffic": PROFILED_TRAFFIC_BYTES, "traffic_source": PROFILED_TRAFFIC_SOURCE}
+            "launches": iters, "traffic": PROFILED_TRAFFIC_BYTES, "traffic_source": PROFILED_TRAFFIC_SOURCE,
+            "phases": phases}
 
 
 def fused_fc_gelu(jf, torch, ops):
@@ -286,8 +303,13 @@ def calibration(jf, torch):
         stream = row("gemm_k_block_stream", 1, 32, workgroups_per_cu=wpc, mode=jf.CAL_STREAM)
     for wpc in (1, 2):                                            # 512-thread workgroups: waves w and w+4 share a SIMD
         row("mfma_and_32fmac_separate_waves", 1, 32, workgroups_per_cu=wpc, threads=512, mode=jf.CAL_SPLIT)
+    # the same stream on operands that change with every MFMA and use all 8 bits, held for ~150 ms: the shader clock
+    # depends on how much the datapaths toggle, and the first stream above runs on near-constant operands
+    sustained = row("gemm_k_block_stream_changing_operands_sustained", 1, 32, iters=20000, workgroups_per_cu=2, threads=512,
+                    mode=jf.CAL_STREAM_DATA, launches=10)
     out["ceiling_TOPs_independent"] = round(65536 / both * 1e9 * 1024 / 1e12, 1)
     out["ceiling_TOPs_k_block_stream"] = round(65536 / stream * 1e9 * 1024 / 1e12, 1)
+    out["ceiling_TOPs_k_block_stream_changing_operands"] = round(65536 / sustained * 1e9 * 1024 / 1e12, 1)
     a = torch.randn(TOKENS, 1600, device="cuda", dtype=torch.bfloat16)
     b = torch.randn(6400, 1600, device="cuda", dtype=torch.bfloat16)
     for _ in range(5):
@@ -301,7 +323,9 @@ def calibration(jf, torch):
     out["torch_bf16_fc_forward_TFLOPs"] = round(2.0 * TOKENS * 6400 * 1600 * 20 / (e0.elapsed_time(e1) * 1e-3) / 1e12, 1)
     out["note"] = ("the exact fp32 scale-accumulate needs 32 VALU instructions per MFMA; with two or more waves per SIMD "
                    "the times of the two pipes add (in cycles, not through a clock drop), also when they come from "
-                   "separate waves: the two ceilings are what any kernel with these semantics can reach at 4 waves per SIMD")
+                   "separate waves: the ceilings are what any kernel with these semantics can reach at 4 waves per SIMD; "
+                   "the last one is the same instruction stream at the lower clock the part sustains when operands change "
+                   "as they do on real tensors (still from registers: no LDS or memory traffic)")
     return out
 
 

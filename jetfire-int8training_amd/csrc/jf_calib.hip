@@ -16,6 +16,9 @@ namespace jf {
 //                        work and vector work from DIFFERENT waves.
 //   MODE JF_CAL_STREAM:  the instruction stream of the GEMM's K block: an MFMA whose accumulator input is the inline
 //                        constant, then 16 subtractions + 16 fmacs on the PREVIOUS product (real dependencies).
+//   MODE JF_CAL_STREAM_DATA: the same stream fed with operands that change from one MFMA to the next and use all
+//                        8 bits (four register sets of hashed bytes) and a scale with a full mantissa: what the same
+//                        instructions cost, in clock rate, when the datapaths toggle as they do on real tensors.
 template <int MODE, int WITH_MFMA, int NV>
 __global__ __launch_bounds__(512) void calib_kernel(int iters, float *out, unsigned long long *clocks)
 {
@@ -28,7 +31,35 @@ __global__ __launch_bounds__(512) void calib_kernel(int iters, float *out, unsig
     float f[32];
     for (int i = 0; i < 32; ++i) f[i] = (float)i;
     const float s = 1.0f + 1e-6f * threadIdx.x, m = 0.5f;
-    if (MODE == JF_CAL_STREAM) {
+    if (MODE == JF_CAL_STREAM_DATA) {
+        v4i ra[4], rb[4];
+        unsigned h = (unsigned)(blockIdx.x * blockDim.x + threadIdx.x) * 2654435761u + 12345u;
+        for (int i = 0; i < 4; ++i)
+            for (int w = 0; w < 4; ++w) {
+                h = h * 1664525u + 1013904223u; ra[i][w] = (int)(h ^ (h >> 13));
+                h = h * 1664525u + 1013904223u; rb[i][w] = (int)(h ^ (h >> 15));
+            }
+        const float sr = 1.0f + (float)(h >> 9) * (1.0f / 8388608.0f) * 1e-3f;   // ~1: the sums stay finite
+        v16i d_pend = c[0];
+        for (int it = 0; it < iters; ++it) {
+#pragma unroll
+            for (int i = 0; i < 4; ++i) {
+                v16i d_new;
+                asm volatile("v_mfma_i32_32x32x32_i8 %0, %1, %2, 0x3e22f983" : "=&v"(d_new) : "v"(ra[i]), "v"(rb[i]));
+                __builtin_amdgcn_sched_barrier(0);
+                float t[16];
+#pragma unroll
+                for (int v = 0; v < 16; ++v) t[v] = __int_as_float(d_pend[v]) - __int_as_float(0x3e22f983);
+#pragma unroll
+                for (int v = 0; v < 16; ++v) f[16 * (i & 1) + v] = __builtin_fmaf((i & 2) ? sr : -sr, t[v], f[16 * (i & 1) + v]);
+#pragma unroll
+                for (int v = 0; v < 32; ++v) asm volatile("" : "+v"(f[v]));
+                __builtin_amdgcn_sched_barrier(0);
+                d_pend = d_new;
+            }
+        }
+        c[0] = d_pend;
+    } else if (MODE == JF_CAL_STREAM) {
         v16i d_pend = c[0];
         for (int it = 0; it < iters; ++it) {
 #pragma unroll
@@ -102,7 +133,7 @@ extern "C" int jf_calibrate(int mode, int with_mfma, int valu_per_mfma, int iter
     }
     JF_CAL(JF_CAL_UNIFORM, 1, 0) JF_CAL(JF_CAL_UNIFORM, 0, 32) JF_CAL(JF_CAL_UNIFORM, 1, 32)
     JF_CAL(JF_CAL_UNIFORM, 0, 16) JF_CAL(JF_CAL_UNIFORM, 1, 16)
-    JF_CAL(JF_CAL_SPLIT, 1, 32) JF_CAL(JF_CAL_STREAM, 1, 32)
+    JF_CAL(JF_CAL_SPLIT, 1, 32) JF_CAL(JF_CAL_STREAM, 1, 32) JF_CAL(JF_CAL_STREAM_DATA, 1, 32)
 #undef JF_CAL
     return JF_ERR_ENUM;
 }

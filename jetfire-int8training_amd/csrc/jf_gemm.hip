@@ -67,6 +67,8 @@ struct GemmArgs {
     const void *Xs;       // [M/32, N/32]
     uint64_t seed2, offset2;   // noise of the GELU backward's own requantisation   (EPI_QB)
     int rounding2;        // JF_ROUND_NEAREST / JF_ROUND_STOCHASTIC   (EPI_QB)
+    unsigned long long *phases;   // PROF kernels: 8 words per workgroup (jf_igemm_phase_record), first phase_capacity workgroups
+    int phase_capacity;
 };
 
 // Logical tile (and K split) of this workgroup.  Workgroups are dealt round-robin to the 8 XCDs, each with a
@@ -100,10 +102,21 @@ constexpr int WBM = 2, WBN = 1;
 // AKM = 1: A is [K, lda] (M-contiguous rows), staged and read like a [K,N] B operand (below).
 // BKN = 0: B is [N, ldb] (K-contiguous rows, like A).  BKN = 1: B is [K, ldb] (N-contiguous rows); its tile is staged
 // as it lies in memory and the K-contiguous MFMA operand is produced by the transposing LDS read of gfx950.
-template <int EPI, typename ST, int WGM, int WGN, int NSTAGE, int WGPC, int BKN, int AKM = 0>
+// PROF = 1: the first wave of every workgroup also records when the workgroup's phases began and ended (wall clock) and
+// how many shader cycles its main loop took: a profiling build of the same code, launched only while a recording buffer
+// is set (jf_igemm_phase_record).
+template <int EPI, typename ST, int WGM, int WGN, int NSTAGE, int WGPC, int BKN, int AKM = 0, int PROF = 0>
 __global__ __launch_bounds__(64 * WGM * WGN, WGPC * WGM * WGN / 4) void igemm_nt_kernel(GemmArgs p_in)
 {
     GemmArgs p = p_in;                                        // K-split launches narrow it to the split's K range below
+    unsigned long long *const prof_buf = p_in.phases;
+    const int prof_cap = p_in.phase_capacity;
+    // (a macro, so that the clock is read by the one storing thread only)
+#define phase(k, v) do { if (PROF && threadIdx.x == 0 && (int)blockIdx.x < prof_cap) prof_buf[(size_t)blockIdx.x * 8 + (k)] = (v); } while (0)
+    if (PROF) {
+        phase(0, (unsigned long long)wall_clock64());
+        phase(6, (unsigned long long)__builtin_amdgcn_s_getreg((31 << 11) | 4));      // HW_ID: which CU it ran on
+    }
     constexpr int NW = WGM * WGN;
     constexpr int BM = QB * WBM * WGM, BN = QB * WBN * WGN;
     constexpr int A_BYTES = BM * ROW_BYTES;                  // one stage of A
@@ -451,7 +464,15 @@ __global__ __launch_bounds__(64 * WGM * WGN, WGPC * WGM * WGN / 4) void igemm_nt
     asm volatile("" ::: "memory");
     __builtin_amdgcn_s_barrier();                              // bare: __syncthreads() would drain every load
     asm volatile("" ::: "memory");
-    fetch(fa_u[0], fb_u[0], 0u, sc_v, c0{}, c0{}, c0{}, c0{});
+    // A wave whose blocks all lie beyond M or N (the ragged edge of the tile grid: GPT-2 XL's 1600 columns are 12.5
+    // tiles) keeps its part in the loads and barriers of the workgroup but neither reads operands nor multiplies: the
+    // SIMD it sits on is left to the waves of the other resident workgroup.  ACTIVE = false is that walk.
+    const bool wave_active = m0 + wm * (WBM * QB) < p.M && n0 + wn * (WBN * QB) < p.N;        // wave-uniform
+    long long prof_c0 = 0;
+    if (PROF) { phase(1, (unsigned long long)wall_clock64()); prof_c0 = clock64(); }
+    auto main_loop = [&](auto active_c) {
+    constexpr bool ACTIVE = decltype(active_c)::value;
+    if constexpr (ACTIVE) fetch(fa_u[0], fb_u[0], 0u, sc_v, c0{}, c0{}, c0{}, c0{});
 
     for (int s0 = 0; s0 < nfull; s0 += NSTAGE) static_for<0, NSTAGE>([&](auto slot_c) {
         constexpr int SLOT = decltype(slot_c)::value;         // ring slot of this stage, a compile-time constant
@@ -474,21 +495,25 @@ __global__ __launch_bounds__(64 * WGM * WGN, WGPC * WGM * WGN / 4) void igemm_nt
                     if (s + NSTAGE < nstages) issue_stage(s + NSTAGE);
                 }
                 // unconditional: past the last stage it reads bytes of the ring that nobody uses
-                fetch(fa_u[0], fb_u[0], 0u, sc_v, std::integral_constant<int, NEXT_SLOT * STAGE_BYTES>{},
-                      std::integral_constant<int, NEXT_SLOT * STAGE_BYTES>{},
-                      std::integral_constant<int, NEXT_SLOT * 64>{}, std::integral_constant<int, NXT>{});
+                if constexpr (ACTIVE)
+                    fetch(fa_u[0], fb_u[0], 0u, sc_v, std::integral_constant<int, NEXT_SLOT * STAGE_BYTES>{},
+                          std::integral_constant<int, NEXT_SLOT * STAGE_BYTES>{},
+                          std::integral_constant<int, NEXT_SLOT * 64>{}, std::integral_constant<int, NXT>{});
             } else {
-                fetch(fa_u[kb + 1], fb_u[kb + 1], 0u, sc_v, std::integral_constant<int, SLOT * STAGE_BYTES>{},
-                      std::integral_constant<int, SLOT * STAGE_BYTES + (kb + 1) * 4096>{},
-                      std::integral_constant<int, SLOT * 64 + (kb + 1) * 16>{}, std::integral_constant<int, NXT>{});
+                if constexpr (ACTIVE)
+                    fetch(fa_u[kb + 1], fb_u[kb + 1], 0u, sc_v, std::integral_constant<int, SLOT * STAGE_BYTES>{},
+                          std::integral_constant<int, SLOT * STAGE_BYTES + (kb + 1) * 4096>{},
+                          std::integral_constant<int, SLOT * 64 + (kb + 1) * 16>{}, std::integral_constant<int, NXT>{});
             }
-            fetched(std::integral_constant<int, FETCH_OPS>{}, std::integral_constant<int, CUR>{});
-            __builtin_amdgcn_sched_barrier(0);                // the reads above stay above the products below,
-            compute(std::integral_constant<int, CUR>{}, s * KB_STAGE + kb);
-            __builtin_amdgcn_sched_barrier(0);                // and K blocks are scheduled one by one (register pressure)
+            if constexpr (ACTIVE) {
+                fetched(std::integral_constant<int, FETCH_OPS>{}, std::integral_constant<int, CUR>{});
+                __builtin_amdgcn_sched_barrier(0);            // the reads above stay above the products below,
+                compute(std::integral_constant<int, CUR>{}, s * KB_STAGE + kb);
+                __builtin_amdgcn_sched_barrier(0);            // and K blocks are scheduled one by one (register pressure)
+            }
         });
     });
-    if (ktail) {
+    if (ACTIVE && ktail) {
         // short last stage (K not a multiple of 128): its first K block is already on its way to register set 0
         const unsigned slot = (unsigned)(nfull % NSTAGE);
         static_for<0, KB_STAGE - 1>([&](auto kb_c) {
@@ -504,8 +529,11 @@ __global__ __launch_bounds__(64 * WGM * WGN, WGPC * WGM * WGN / 4) void igemm_nt
             }
         });
     }
+    };
+    if (wave_active) main_loop(std::true_type{});
+    else main_loop(std::false_type{});
     __builtin_amdgcn_s_waitcnt(0xC07F);                        // the last, unused prefetch must land before its registers are reused
-    if (EPI != EPI_S32) {
+    if (EPI != EPI_S32 && wave_active) {
         accumulate(std::integral_constant<int, NBLK - 1>{});
         // The scaled factor sa*sb*2^26 overflows when sa*sb >= 2^102.  An infinite factor leaves every accumulator
         // it touches infinite or NaN (inf*0 included), so "some accumulator of the wave is not finite" catches all such
@@ -566,7 +594,9 @@ __global__ __launch_bounds__(64 * WGM * WGN, WGPC * WGM * WGN / 4) void igemm_nt
             });
         }
     }
+    if (PROF) { phase(2, (unsigned long long)wall_clock64()); phase(7, (unsigned long long)(clock64() - prof_c0)); }
     __syncthreads();           // the epilogue reuses the ring as scratch
+    if (PROF) phase(3, (unsigned long long)wall_clock64());
 
     // ---- epilogue ------------------------------------------------------------------------------------------
     // One 32x32 block at a time goes through a wave-private LDS patch that turns the MFMA result layout
@@ -733,6 +763,7 @@ __global__ __launch_bounds__(64 * WGM * WGN, WGPC * WGM * WGN / 4) void igemm_nt
             }
         }
 
+    if (PROF) phase(4, (unsigned long long)wall_clock64());
     if (out_bytes < 4) {
         __syncthreads();
         // the tile image leaves in whole rows: consecutive lanes write consecutive 16-byte chunks of a row
@@ -749,6 +780,8 @@ __global__ __launch_bounds__(64 * WGM * WGN, WGPC * WGM * WGN / 4) void igemm_nt
                     *reinterpret_cast<const v4i *>(tile2 + (size_t)row * row_bytes + ch * 16);
         }
     }
+    if (PROF) phase(5, (unsigned long long)wall_clock64());
+#undef phase
 }
 
 // -------------------------------------------------------------------------------------------------
@@ -785,7 +818,7 @@ static int launch_transpose(const int8_t *in, int R, int C, int8_t *out, hipStre
     return (int)hipGetLastError();
 }
 
-template <int EPI, typename ST, int WGM, int WGN, int NSTAGE, int WGPC, int BKN, int AKM = 0>
+template <int EPI, typename ST, int WGM, int WGN, int NSTAGE, int WGPC, int BKN, int AKM = 0, int PROF = 0>
 static int launch_gemm_cfg(const GemmArgs &a, hipStream_t st)
 {
     constexpr int BM = QB * WBM * WGM, BN = QB * WBN * WGN, NT = 64 * WGM * WGN;
@@ -796,7 +829,7 @@ static int launch_gemm_cfg(const GemmArgs &a, hipStream_t st)
     GemmArgs p = a;
     p.tiles_m = (p.M + BM - 1) / BM;
     p.tiles_n = (p.N + BN - 1) / BN;
-    auto kern = igemm_nt_kernel<EPI, ST, WGM, WGN, NSTAGE, WGPC, BKN, AKM>;
+    auto kern = igemm_nt_kernel<EPI, ST, WGM, WGN, NSTAGE, WGPC, BKN, AKM, PROF>;
     // more than 64 KiB of dynamic LDS has to be opted into, per function and device: once, not on every launch
     // (the reference sets its attribute on every call, igemm_BlockSquare32OutputIntQuantizeBiasRowCol.cu:418)
     static std::atomic<bool> opted_in[MAX_DEVICES] = {};
@@ -880,9 +913,17 @@ template <int EPI, typename ST> static int launch_gemm(const GemmArgs &a, hipStr
             }
             return JF_ERR_UNSUPPORTED;
         }
+        if constexpr (EPI == EPI_Q && std::is_same<ST, float>::value) {
+            if (a.phases)                                     // a recording buffer is set: the profiling build
+                return b_kn ? launch_gemm_cfg<EPI, ST, 2, 4, 2, 2, 1, 0, 1>(a, st) : launch_gemm_cfg<EPI, ST, 2, 4, 2, 2, 0, 0, 1>(a, st);
+        }
         return b_kn ? launch_gemm_cfg<EPI, ST, 2, 4, 2, 2, 1>(a, st) : launch_gemm_cfg<EPI, ST, 2, 4, 2, 2, 0>(a, st);
     }
 }
+
+// recording buffer of the profiling build (process-wide; set and cleared by jf_igemm_phase_record)
+static std::atomic<unsigned long long *> phase_buffer{nullptr};
+static std::atomic<int> phase_buffer_capacity{0};
 
 static int check_gemm_common(const void *A, const void *B, const void *C, int M, int N, int K, int b_layout)
 {
@@ -1093,7 +1134,21 @@ int jf_igemm_block_q(const int8_t *A, const int8_t *B, const void *sa, const voi
     if (!scale_strides(sa_layout, K, M / QB, a.sa_ks, a.sa_is) || !scale_strides(sb_layout, K, N / QB, a.sb_ks, a.sb_is))
         return JF_ERR_ENUM;
     hipStream_t st = (hipStream_t)stream;
+    if (scale_dtype == JF_SCALE_F32) {
+        a.phases = phase_buffer.load(std::memory_order_acquire);
+        a.phase_capacity = phase_buffer_capacity.load(std::memory_order_acquire);
+    }
     return scale_dtype == JF_SCALE_F16 ? launch_gemm<EPI_Q, half_t>(a, st, kn) : launch_gemm<EPI_Q, float>(a, st, kn);
+}
+
+int jf_igemm_phase_record(unsigned long long *phases, int capacity_workgroups)
+{
+    if (phases && capacity_workgroups <= 0) return JF_ERR_SHAPE;
+    if (!phases) capacity_workgroups = 0;
+    phase_buffer_capacity.store(0, std::memory_order_release);
+    phase_buffer.store(phases, std::memory_order_release);
+    phase_buffer_capacity.store(capacity_workgroups, std::memory_order_release);
+    return JF_OK;
 }
 
 int jf_igemm_block_q_gelu(const int8_t *A, const int8_t *B, const void *sa, const void *sb, const float *bias,

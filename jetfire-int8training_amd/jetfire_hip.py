@@ -28,7 +28,7 @@ EXPORTS = [
     "jf_error_string", "jf_igemm_workspace_bytes", "jf_igemm_s32", "jf_igemm_block_acc", "jf_igemm_block_fp",
     "jf_igemm_splitk_plan", "jf_igemm_block_fp_workspace_bytes", "jf_igemm_block_q_gelu", "jf_igemm_block_fp_noalloc", "jf_igemm_block_q_gelu_bwd",
     "jf_igemm_block_q", "jf_quantize", "jf_dequantize", "jf_transpose_s8", "jf_rowstats", "jf_layernorm_fwd",
-    "jf_layernorm_bwd_workspace_bytes", "jf_layernorm_bwd", "jf_gelu_fwd", "jf_gelu_bwd", "jf_add", "jf_calibrate", "jf_wall_clock_khz",
+    "jf_layernorm_bwd_workspace_bytes", "jf_layernorm_bwd", "jf_gelu_fwd", "jf_gelu_bwd", "jf_add", "jf_calibrate", "jf_wall_clock_khz", "jf_igemm_phase_record",
 ]
 
 _lib = None
@@ -55,6 +55,7 @@ def lib():
         L.jf_igemm_splitk_plan.argtypes = [_i, _i, _i, _i, C.POINTER(C.c_int), C.POINTER(C.c_int)]
         L.jf_igemm_block_fp_workspace_bytes.argtypes = [_i, _i, _i, _i, _i]
         L.jf_igemm_block_fp_workspace_bytes.restype = _sz
+        L.jf_igemm_phase_record.argtypes = [_p, _i]
         L.jf_igemm_block_q.argtypes = [_p, _p, _p, _p, _p, _p, _p, _p, _i, _i, _i, _i, _i, _i, _i, _i, _u64, _u64, _p, _sz, _p]
         L.jf_quantize.argtypes = [_p, _i, _i, _i, _p, _p, _p, _i, _i, _u64, _u64, _f, _p]
         L.jf_dequantize.argtypes = [_p, _p, _i, _i, _i, _p, _p]
@@ -441,14 +442,14 @@ def add(x1, q2, s2, rounding=ROUND_TRUNC, with_stats=False, seed=None, offset=No
     return (y1, q, s, rs, rq) if with_stats else (y1, q, s)
 
 
-CAL_UNIFORM, CAL_SPLIT, CAL_STREAM = 0, 1, 2
+CAL_UNIFORM, CAL_SPLIT, CAL_STREAM, CAL_STREAM_DATA = 0, 1, 2, 3
 
 
-def calibrate(with_mfma, valu_per_mfma, iters=2000, workgroups_per_cu=4, threads=256, mode=CAL_UNIFORM):
+def calibrate(with_mfma, valu_per_mfma, iters=2000, workgroups_per_cu=4, threads=256, mode=CAL_UNIFORM, launches=3):
     """Runs the register-only calibration kernel (see jf_calibrate in the header) and returns a dict: seconds per launch
     (events), the number of work items it ran (workgroups * waves * iters * 4; for CAL_SPLIT: items of the MFMA waves),
     the resident waves per SIMD, and the shader clock in MHz the kernel ran at (cycles / wall-clock time, from the
-    per-workgroup readings)."""
+    per-workgroup readings of the last launch)."""
     props = torch.cuda.get_device_properties(0)
     cus = props.multi_processor_count
     wgs = cus * workgroups_per_cu
@@ -460,15 +461,40 @@ def calibrate(with_mfma, valu_per_mfma, iters=2000, workgroups_per_cu=4, threads
     run()
     e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
     e0.record()
-    for _ in range(3):
+    for _ in range(launches):
         run()
     e1.record()
     torch.cuda.synchronize()
     c = clocks.view(wgs, 2).double().sum(0)
     wall_hz = _wall_clock_hz()
     items = wgs * (waves // 2 if mode == CAL_SPLIT else waves) * iters * 4
-    return {"seconds": e0.elapsed_time(e1) * 1e-3 / 3, "items": items, "waves_per_simd": workgroups_per_cu * waves / 4,
+    return {"seconds": e0.elapsed_time(e1) * 1e-3 / launches, "items": items, "waves_per_simd": workgroups_per_cu * waves / 4,
             "shader_MHz": float(c[0] / c[1]) * wall_hz / 1e6, "simds": cus * 4}
+
+
+def igemm_phases(fn, workgroups):
+    """Runs fn() (one jf_igemm_block_q call with fp32 scales) under the library's phase recording and returns, per
+    workgroup (one 128x128 output tile each), a dict of numpy arrays: 'us' [workgroups, 6] (start, main loop begins, main
+    loop ends, epilogue begins, blocks requantised, end; microseconds since the first workgroup started), 'cu' (an id
+    of the CU it ran on), 'k_loop_MHz' (shader clock during its main loop) and 'k_loop_cycles'."""
+    import numpy as np
+    buf = torch.zeros(workgroups * 8, dtype=torch.int64, device="cuda")
+    check(lib().jf_igemm_phase_record(_ptr(buf), workgroups))
+    try:
+        fn()
+        torch.cuda.synchronize()
+    finally:
+        check(lib().jf_igemm_phase_record(None, 0))
+    w = buf.view(workgroups, 8).cpu().numpy()
+    hz = _wall_clock_hz()
+    t = w[:, :6].astype(np.float64)
+    if (t[:, 5] <= 0).any():
+        raise RuntimeError("igemm_phases: the call launched fewer workgroups than asked for, or no profiling build")
+    us = (t - t[:, 0].min()) / hz * 1e6
+    hw = w[:, 6]
+    return {"us": us, "cu": hw & 0xFF00 | ((hw >> 16) & 0xFF),
+            "k_loop_cycles": w[:, 7].astype(np.float64),
+            "k_loop_MHz": w[:, 7] / np.maximum(t[:, 2] - t[:, 1], 1.0) * hz / 1e6}
 
 
 def _wall_clock_hz():
