@@ -99,11 +99,12 @@ def dominant_kernel_roofline(jf, torch, ops, iters=200):
     simds = 4 * torch.cuda.get_device_properties(0).multi_processor_count
     d = us[:, 1:] - us[:, :-1]
     phases = {"workgroups": tiles, "span_us": round(span_us, 1), "main_loop_shader_MHz": round(mhz),
-              "simd_cycles_per_block_product": round(span_us * mhz * simds / products, 1),
+              "simd_cycles_per_block_product": round(avg_s * 1e6 * mhz * simds / products, 1),
               "mean_us": {k: round(float(d[:, i].mean()), 2) for i, k in
                           enumerate(("prologue", "main_loop", "sync", "requantise", "store"))},
-              "note": "simd_cycles_per_block_product = span x clock x SIMDs / MFMA count: everything the kernel does, per "
-                      "MFMA; the register-only stream of one MFMA + 32 VALU instructions takes the cycles the calibration "
+              "note": "simd_cycles_per_block_product = average launch time (of the normal build, above) x this clock x "
+                      "SIMDs / MFMA count: everything the kernel does, per MFMA; span_us is the recorded launch alone, first "
+                      "workgroup start to last workgroup end; the register-only stream of one MFMA + 32 VALU instructions takes the cycles the calibration "
                       "table gives for gemm_k_block_stream"}
     return {"bound": "mfma", "kernel": "igemm_nt_kernel<EPI_Q,f32> fc forward 8192x6400x1600",
             "achieved": round(achieved, 2), "peak": INT8_PEAK_TOPS, "unit": "TOP/s",
