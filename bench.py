@@ -487,6 +487,7 @@ def main():
     ap.add_argument("--roofline-only", action="store_true", help="only the dominant-kernel measurement (for rocprofv3 --stats)")
     ap.add_argument("--extras-only", action="store_true", help="only the block-kernel section (for rocprofv3 --pmc)")
     ap.add_argument("--calibration-only", action="store_true", help="only the register-only calibration loops")
+    ap.add_argument("--block-only", action="store_true", help="only the transformer-block comparison (for rocprofv3 --stats)")
     a = ap.parse_args()
     if a.gpus != 1:
         sys.exit("bench.py: this build measures one GPU only (--gpus 1); nothing here uses a second GPU")
@@ -499,6 +500,9 @@ def main():
     torch.cuda.set_device(0)
     if a.calibration_only:
         print(json.dumps({"calibration": calibration(jf, torch)}))
+        return
+    if a.block_only:
+        print(json.dumps({"xl_block_forward_backward": recipe_block(torch)}))
         return
     ops = make_inputs(jf, torch)
     if a.pmc_probe:

@@ -163,8 +163,11 @@ int jf_quantize(const void *x, int x_dtype, int R, int C, int8_t *q, void *s, in
                 int scale_dtype, int rounding, uint64_t seed, uint64_t offset, float amax_eps,
                 jf_stream_t stream);
 
-/* out_f32[R,C] = q*s.  Replaces int8_dequantize (Jetfire/Nonlinear/dequantize.py:86-116). */
-int jf_dequantize(const int8_t *q, const void *s, int R, int C, int scale_dtype, float *out,
+/* out[R,C] = q*s, the fp32 product rounded to `out_dtype` (JF_FP_F32 / JF_FP_F16 / JF_FP_BF16; for binary16 scales and
+ * output this equals the reference's binary16 multiplication).  Replaces int8_dequantize
+ * (Jetfire/Nonlinear/dequantize.py:86-116) and the dequantisation int8_linear_forward does on its unquantised-output
+ * path (Jetfire/Linear/linear_fwd.py:29-31). */
+int jf_dequantize(const int8_t *q, const void *s, int R, int C, int scale_dtype, void *out, int out_dtype,
                   jf_stream_t stream);
 
 /* out[C,R] = in[R,C].  Replaces int8_transpose (Jetfire/Nonlinear/transpose.py:69-97). */
@@ -210,6 +213,13 @@ int jf_gelu_bwd(const int8_t *qx, const void *sx, const int8_t *qg, const void *
 int jf_add(const void *x1, int x1_dtype, const int8_t *q2, const void *s2, int R, int C,
            int scale_dtype, int rounding, uint64_t seed, uint64_t offset,
            float *y1, int8_t *q, void *s, float *rowsum, float *rowsq, jf_stream_t stream);
+
+/* mean[r] = (sum of rowsum[r, 0..parts-1], ascending) / C;  rstd[r] = 1 / sqrt((sum of rowsq[r, :]) / C - mean[r]^2)
+ * (no epsilon): the finishing step of int8_add_Ifp_Ig16_Ofp_Og_MeanVar (Jetfire/Nonlinear/add_mean_var.py:219-221), which
+ * the reference computes with torch operators on the kernel's partial sums.  rowsum, rowsq: [R, parts] fp32 as written by
+ * jf_add. */
+int jf_rowstats_finish(const float *rowsum, const float *rowsq, int R, int parts, int C, float *mean, float *rstd,
+                       jf_stream_t stream);
 
 /* Phase recording (no counterpart in the reference; a profiling aid for bench.py).  While a buffer is set, every
  * jf_igemm_block_q call with fp32 scales launches a profiling build of its kernel in which workgroup w (w <

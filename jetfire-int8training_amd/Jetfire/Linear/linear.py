@@ -47,7 +47,9 @@ def _check_block(B):
 
 
 def _dequant_like(q2d, s2d, lead_shape):
-    out = _jf.dequantize(q2d, s2d).to(s2d.dtype)
+    """codes x scales in the scales' dtype, as the reference's unquantised-output path computes it (linear_fwd.py:29-31):
+    one kernel, no fp32 intermediate."""
+    out = _jf.dequantize(q2d, s2d, out_dtype=s2d.dtype)
     return out.reshape(*lead_shape, q2d.shape[-1])
 
 
@@ -88,13 +90,14 @@ def int8_linear_forward_gelu(X8_3D, SX16_3D, W8, SW16, B, approximate="none"):
 
 
 def int8_linear_backward(X8_3D, SX16_3D, G8_3D, SG16_3D, G8T, W8, SW16, B, stochastic=True, dgrad_quantize=True,
-                         wgrad_splitk=1):
+                         wgrad_splitk=1, wgrad_dtype=None):
     """dX = dY W (requantised with stochastic rounding) and dW = dY^T X (fp16).
     G8 [BS,T,N] with SG [BS,T/32,N/32]; G8T = G8 transposed to [N, BS*T], or None (then G8 itself is read, no copy);
     W8 [N,K], SW [N/32,K/32].
     Returns (GX8, GSX, GW) or (GX_fp, GW) when dgrad_quantize=False (reference: linear_bwd.py:4-29; like
     there, the activation gradient is always rounded stochastically).  wgrad_splitk (not in the reference): 1 = its
-    arithmetic; 0 = let the library cut K into ordered partial sums when dW has too few tiles to fill the GPU."""
+    arithmetic; 0 = let the library cut K into ordered partial sums when dW has too few tiles to fill the GPU.
+    wgrad_dtype (not in the reference): None = float16 as there; float32 / bfloat16 = dW leaves the kernel in that type."""
     _check_block(B)
     g2, sg2 = _flat2(G8_3D).contiguous(), _flat2(SG16_3D).contiguous()
     x2, sx2 = _flat2(X8_3D).contiguous(), _flat2(SX16_3D).contiguous()
@@ -103,14 +106,14 @@ def int8_linear_backward(X8_3D, SX16_3D, G8_3D, SG16_3D, G8T, W8, SW16, B, stoch
     gx8, gsx = BQC.igemm_output_int_quantize_stochastic(g2, W8, _k_major(sg2), SW16, tokens, c_in, c_out)
     if G8T is None:
         G8T = g2.t()                                               # a view: the extension reads g2 as the [K, M] operand
-    gw = BQC.igemm_output_fp_no_quantize(G8T, x2, sg2, sx2, G8T.shape[0], c_in, G8T.shape[1], wgrad_splitk)
+    gw = BQC.igemm_output_fp_no_quantize(G8T, x2, sg2, sx2, G8T.shape[0], c_in, G8T.shape[1], wgrad_splitk, wgrad_dtype)
     if not dgrad_quantize:
         return _dequant_like(gx8, gsx, tuple(G8_3D.shape[:-1])), gw
     return (gx8.reshape(*G8_3D.shape[:-1], c_in), gsx.reshape(*SG16_3D.shape[:-1], SW16.shape[1]), gw)
 
 
 def int8_linear_backward_gelu(X8_3D, SX16_3D, G8_3D, SG16_3D, W8, SW16, PRE8_3D, SPRE16_3D, B, approximate="none",
-                              stochastic=True, wgrad_splitk=1):
+                              stochastic=True, wgrad_splitk=1, wgrad_dtype=None):
     """int8_linear_backward(...) followed by int8_gelu_backward(PRE8, SPRE, <its activation gradient>, ...), with the
     GELU backward running in the epilogue of the activation-gradient GEMM (no counterpart in the reference, whose MLP
     backward runs the two back to back, qmodel.py:249-253).  X8 / SX: the linear layer's input (= the GELU's output),
@@ -128,5 +131,5 @@ def int8_linear_backward_gelu(X8_3D, SX16_3D, G8_3D, SG16_3D, W8, SW16, PRE8_3D,
     gp8, gsp = _jf.igemm_block_q_gelu_bwd(g2, W8.contiguous(), _k_major(sg2), SW16, p2, sp2,
                                           _jf.GELU_TANH if approximate == "tanh" else _jf.GELU_ERF,
                                           _jf.ROUND_STOCHASTIC if stochastic else _jf.ROUND_NEAREST)
-    gw = BQC.igemm_output_fp_no_quantize(g2.t(), x2, sg2, sx2, c_out, c_in, tokens, wgrad_splitk)
+    gw = BQC.igemm_output_fp_no_quantize(g2.t(), x2, sg2, sx2, c_out, c_in, tokens, wgrad_splitk, wgrad_dtype)
     return (gp8.reshape(*G8_3D.shape[:-1], c_in), gsp.reshape(*SG16_3D.shape[:-1], SW16.shape[1]), gw)

@@ -98,6 +98,7 @@ class AttentionIn(torch.autograd.Function):
     @staticmethod
     def forward(ctx, residual, qx, sx, w_qkv, ln_w, mean, rstd):
         qw, sw = weight_codes.get(w_qkv)
+        ctx.wdtype = w_qkv.dtype          # the weight gradient leaves its GEMM in the parameter's type: no conversion kernel
         qx = _as_s8(qx)
         qn, sn, _ = int8_layernorm_forward(qx, sx, ln_w, mean, rstd, QB)
         qkv = int8_linear_forward(qn, sn, qw, sw, False, QB)
@@ -108,7 +109,7 @@ class AttentionIn(torch.autograd.Function):
     def backward(ctx, fpg, g):
         qx, sx, qn, sn, qw, sw, ln_w, mean, rstd = ctx.saved_tensors
         qg, sg = int8_quantize(g.contiguous(), QB, stochastic=True)
-        qg, sg, gw = int8_linear_backward(qn, sn, qg, sg, None, qw, sw, QB, stochastic=True, wgrad_splitk=0)
+        qg, sg, gw = int8_linear_backward(qn, sn, qg, sg, None, qw, sw, QB, stochastic=True, wgrad_splitk=0, wgrad_dtype=ctx.wdtype)
         qg, sg, g_ln = int8_layernorm_backward(qx, sx, qg, sg, ln_w, QB, mean, rstd, stochastic=True)
         res_g, qg, sg = int8_add_Ifp_Ig16_Ofp_Og(fpg.contiguous(), qg, sg, QB, stochastic=True)
         return res_g, _as_f8(qg), sg, gw, g_ln, None, None
@@ -120,6 +121,7 @@ class AttentionOut(torch.autograd.Function):
     @staticmethod
     def forward(ctx, residual, y, w_proj):
         qw, sw = weight_codes.get(w_proj)
+        ctx.wdtype = w_proj.dtype
         qy, sy = int8_quantize(y.contiguous(), QB)
         qo, so = int8_linear_forward(qy, sy, qw, sw, True, QB)
         fp, q, s, mean, rstd = int8_add_Ifp_Ig16_Ofp_Og_MeanVar(residual.contiguous(), qo, so, QB)
@@ -130,7 +132,7 @@ class AttentionOut(torch.autograd.Function):
     def backward(ctx, fpg, qg, sg, _m, _r):
         qy, sy, qw, sw = ctx.saved_tensors
         qg = _as_s8(qg)
-        g, gw = int8_linear_backward(qy, sy, qg, sg, None, qw, sw, QB, stochastic=True, dgrad_quantize=False, wgrad_splitk=0)
+        g, gw = int8_linear_backward(qy, sy, qg, sg, None, qw, sw, QB, stochastic=True, dgrad_quantize=False, wgrad_splitk=0, wgrad_dtype=ctx.wdtype)
         return fpg, g, gw
 
 
@@ -142,6 +144,7 @@ class MLPResidual(torch.autograd.Function):
         qx = _as_s8(qx)
         qw1, sw1 = weight_codes.get(w_fc)
         qw2, sw2 = weight_codes.get(w_proj)
+        ctx.wdtype = w_fc.dtype
         qn, sn, _ = int8_layernorm_forward(qx, sx, ln_w, mean, rstd, QB)
         qh, sh, qa, sa = int8_linear_forward_gelu(qn, sn, qw1, sw1, QB)      # fc and its GELU in one kernel
         qo, so = int8_linear_forward(qa, sa, qw2, sw2, True, QB)
@@ -155,8 +158,8 @@ class MLPResidual(torch.autograd.Function):
         qg = _as_s8(qg)
         # proj's backward with the GELU backward in the epilogue of its activation-gradient GEMM (one kernel for
         # int8_linear_backward's dgrad + int8_gelu_backward, same bits)
-        qg, sg, gw2 = int8_linear_backward_gelu(qa, sa, qg, sg, qw2, sw2, qh, sh, QB, stochastic=True, wgrad_splitk=0)
-        qg, sg, gw1 = int8_linear_backward(qn, sn, qg, sg, None, qw1, sw1, QB, stochastic=True, wgrad_splitk=0)
+        qg, sg, gw2 = int8_linear_backward_gelu(qa, sa, qg, sg, qw2, sw2, qh, sh, QB, stochastic=True, wgrad_splitk=0, wgrad_dtype=ctx.wdtype)
+        qg, sg, gw1 = int8_linear_backward(qn, sn, qg, sg, None, qw1, sw1, QB, stochastic=True, wgrad_splitk=0, wgrad_dtype=ctx.wdtype)
         qg, sg, g_ln = int8_layernorm_backward(qx, sx, qg, sg, ln_w, QB, mean, rstd, stochastic=True)
         res_g, qg, sg = int8_add_Ifp_Ig16_Ofp_Og(fpg.contiguous(), qg, sg, QB, stochastic=True)
         return res_g, _as_f8(qg), sg, gw1, gw2, g_ln, None, None

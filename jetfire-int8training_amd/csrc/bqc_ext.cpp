@@ -231,21 +231,28 @@ torch::Tensor igemm_basic_int8_gemm(torch::Tensor X, torch::Tensor W, const int 
 
 // include/igemm.h:14-25 : fp16 output, B [K,N]
 // splitk (not in the reference's signature; default 1 = its arithmetic): see jf_igemm_block_fp.
+// out_dtype (not in the reference's signature either; default float16 = its output): float32 or bfloat16 spare the caller a
+// conversion kernel when the weight gradient is accumulated in another type.
 torch::Tensor igemm_output_fp_no_quantize(torch::Tensor X, torch::Tensor W, torch::Tensor SX, torch::Tensor SW,
-                                          const int M, const int N, const int K, const int splitk)
+                                          const int M, const int N, const int K, const int splitk,
+                                          c10::optional<torch::ScalarType> out_dtype)
 {
+    const torch::ScalarType odt = out_dtype.value_or(torch::kFloat16);
+    TORCH_CHECK(odt == torch::kFloat16 || odt == torch::kFloat32 || odt == torch::kBFloat16,
+                "out_dtype must be float16, float32 or bfloat16");
+    const int ocode = odt == torch::kFloat16 ? JF_FP_F16 : odt == torch::kFloat32 ? JF_FP_F32 : JF_FP_BF16;
     check_dims(M, N, K);
     const int a_layout = check_a_any_layout(X, M, K);
     check_b_kn(W, X, K, N);
     int sxl, swl;
     const int code = check_scales(SX, SW, X, M, N, K, sxl, swl);
     c10::DeviceGuard guard(X.device());
-    torch::Tensor O = torch::empty({M, N}, X.options().dtype(torch::kFloat16));
+    torch::Tensor O = torch::empty({M, N}, X.options().dtype(odt));
     TORCH_CHECK(splitk >= 0, "splitk must be >= 0");
     Workspace ws(X, jf_igemm_block_fp_workspace_bytes(M, N, K, JF_B_KN, splitk));
     pybind11::gil_scoped_release nogil;
     check_rc(jf_igemm_block_fp((const int8_t *)X.data_ptr(), (const int8_t *)W.data_ptr(), SX.data_ptr(), SW.data_ptr(),
-                               O.data_ptr(), M, N, K, a_layout, JF_B_KN, code, sxl, swl, JF_FP_F16, splitk, ws.ptr, ws.bytes,
+                               O.data_ptr(), M, N, K, a_layout, JF_B_KN, code, sxl, swl, ocode, splitk, ws.ptr, ws.bytes,
                                current_stream(X)),
              "igemm_output_fp_no_quantize");
     return O;
@@ -320,7 +327,7 @@ PYBIND11_MODULE(TORCH_EXTENSION_NAME, m)
     m.def("igemm_output_fp_no_quantize", &igemm_output_fp_no_quantize,
           "dequantize + INT8 MFMA GEMM, fp16 output; B is [K,N]; backward weight gradient", pybind11::arg("X"),
           pybind11::arg("W"), pybind11::arg("SX"), pybind11::arg("SW"), pybind11::arg("M"), pybind11::arg("N"),
-          pybind11::arg("K"), pybind11::arg("splitk") = 1);
+          pybind11::arg("K"), pybind11::arg("splitk") = 1, pybind11::arg("out_dtype") = pybind11::none());
     m.def("igemm_basic_int8_gemm", &igemm_basic_int8_gemm, "INT8 MFMA GEMM, INT32 output; B is [K,N]");
     m.def("hgemm_v1", &hgemm_v1, "fp16 GEMM (library)");
     // not in the reference: makes the stochastic entry point reproducible from Python

@@ -56,6 +56,17 @@ __device__ __forceinline__ void store16_f32(float *p, const float x[16])
     }
 }
 
+// 16 consecutive values, rounded to nearest even, as two 16-byte stores
+template <typename OT> __device__ __forceinline__ void store16_as(OT *p, const float x[16])
+{
+    OT h[16];
+#pragma unroll
+    for (int k = 0; k < 16; ++k) h[k] = (OT)x[k];
+    reinterpret_cast<v4i *>(p)[0] = *reinterpret_cast<v4i *>(&h[0]);
+    reinterpret_cast<v4i *>(p)[1] = *reinterpret_cast<v4i *>(&h[8]);
+}
+template <> __device__ __forceinline__ void store16_as<float>(float *p, const float x[16]) { store16_f32(p, x); }
+
 // Position of this wave's block / this lane's 16 elements.
 struct BlockPos {
     int rb, cb, row, col;     // block coordinates; absolute row / first column of the lane
@@ -110,15 +121,15 @@ __global__ __launch_bounds__(NT) void quantize_kernel(const T *x, int R, int C, 
 }
 
 // dequantize.py:28-84
-template <typename ST>
-__global__ __launch_bounds__(NT) void dequantize_kernel(const int8_t *q, const ST *s, int R, int C, float *out)
+template <typename ST, typename OT>
+__global__ __launch_bounds__(NT) void dequantize_kernel(const int8_t *q, const ST *s, int R, int C, OT *out)
 {
     JF_FOR_EACH_BLOCK(R, C)
     {
         BlockPos pos(blk, SC, C, lane);
         float x[16];
         unpack16(*reinterpret_cast<const v4i *>(q + pos.e0), load_scale(s, pos.rb * SC + pos.cb), x);
-        store16_f32(out + pos.e0, x);
+        store16_as<OT>(out + pos.e0, x);
     }
 }
 
@@ -682,6 +693,22 @@ static inline bool rounding_ok(int r) { return r >= JF_ROUND_NEAREST && r <= JF_
 
 using namespace jf;
 
+// mean and 1/sqrt(variance) of every row from its per-32-column partial sums (rowsum, rowsq: [R, parts], what add_kernel
+// leaves): the partials are added in ascending order, var = E[y^2] - mean^2, no epsilon (add_mean_var.py:219-221).
+__global__ __launch_bounds__(256) void rowstats_finish_kernel(const float *rowsum, const float *rowsq, int R, int parts,
+                                                              float n, float *mean, float *rstd)
+{
+    const int r = blockIdx.x * 256 + threadIdx.x;
+    if (r >= R) return;
+    const float *ps = rowsum + (size_t)r * parts, *pq = rowsq + (size_t)r * parts;
+    float a = 0.0f, b = 0.0f;
+    for (int j = 0; j < parts; ++j) { a = a + ps[j]; b = b + pq[j]; }
+    const float m = a / n;
+    const float var = b / n - m * m;
+    mean[r] = m;
+    rstd[r] = 1.0f / __builtin_sqrtf(var);
+}
+
 #define JF_LAUNCH(kern, grid, smem, st, ...)                         \
     do {                                                             \
         if (!device_is_gfx950()) return JF_ERR_DEVICE;               \
@@ -715,16 +742,25 @@ int jf_quantize(const void *x, int x_dtype, int R, int C, int8_t *q, void *s, in
 #undef JF_Q
 }
 
-int jf_dequantize(const int8_t *q, const void *s, int R, int C, int scale_dtype, float *out, jf_stream_t stream)
+int jf_dequantize(const int8_t *q, const void *s, int R, int C, int scale_dtype, void *out, int out_dtype, jf_stream_t stream)
 {
     int rc = check_block_tensor(q, s, R, C, scale_dtype);
     if (rc) return rc;
     if (!out) return JF_ERR_NULL;
+    if (out_dtype != JF_FP_F32 && out_dtype != JF_FP_F16 && out_dtype != JF_FP_BF16) return JF_ERR_ENUM;
     if (!aligned16(out)) return JF_ERR_ALIGN;
     hipStream_t st = (hipStream_t)stream;
     const int grid = grid_for_blocks(R, C);
-    if (scale_dtype == JF_SCALE_F16) JF_LAUNCH(dequantize_kernel<half_t>, grid, 0, st, q, (const half_t *)s, R, C, out);
-    JF_LAUNCH(dequantize_kernel<float>, grid, 0, st, q, (const float *)s, R, C, out);
+#define JF_DQ(ST, OT) JF_LAUNCH((dequantize_kernel<ST, OT>), grid, 0, st, q, (const ST *)s, R, C, (OT *)out)
+    if (scale_dtype == JF_SCALE_F16) {
+        if (out_dtype == JF_FP_F32) JF_DQ(half_t, float);
+        if (out_dtype == JF_FP_F16) JF_DQ(half_t, half_t);
+        JF_DQ(half_t, __bf16);
+    }
+    if (out_dtype == JF_FP_F32) JF_DQ(float, float);
+    if (out_dtype == JF_FP_F16) JF_DQ(float, half_t);
+    JF_DQ(float, __bf16);
+#undef JF_DQ
 }
 
 int jf_rowstats(const int8_t *q, const void *s, int R, int C, int scale_dtype, float eps, float *mean, float *rstd,
@@ -872,6 +908,17 @@ int jf_add(const void *x1, int x1_dtype, const int8_t *q2, const void *s2, int R
         JF_ADD(__bf16, float);
     }
 #undef JF_ADD
+}
+
+int jf_rowstats_finish(const float *rowsum, const float *rowsq, int R, int parts, int C, float *mean, float *rstd,
+                       jf_stream_t stream)
+{
+    if (!rowsum || !rowsq || !mean || !rstd) return JF_ERR_NULL;
+    if (R <= 0 || parts <= 0 || C <= 0) return JF_ERR_SHAPE;
+    if (!device_is_gfx950()) return JF_ERR_DEVICE;
+    hipLaunchKernelGGL(rowstats_finish_kernel, dim3((R + 255) / 256), dim3(256), 0, (hipStream_t)stream, rowsum, rowsq, R,
+                       parts, (float)C, mean, rstd);
+    return (int)hipGetLastError();
 }
 
 }  // extern "C"

@@ -28,7 +28,7 @@ EXPORTS = [
     "jf_error_string", "jf_igemm_workspace_bytes", "jf_igemm_s32", "jf_igemm_block_acc", "jf_igemm_block_fp",
     "jf_igemm_splitk_plan", "jf_igemm_block_fp_workspace_bytes", "jf_igemm_block_q_gelu", "jf_igemm_block_fp_noalloc", "jf_igemm_block_q_gelu_bwd",
     "jf_igemm_block_q", "jf_quantize", "jf_dequantize", "jf_transpose_s8", "jf_rowstats", "jf_layernorm_fwd",
-    "jf_layernorm_bwd_workspace_bytes", "jf_layernorm_bwd", "jf_gelu_fwd", "jf_gelu_bwd", "jf_add", "jf_calibrate", "jf_wall_clock_khz", "jf_igemm_phase_record",
+    "jf_layernorm_bwd_workspace_bytes", "jf_layernorm_bwd", "jf_gelu_fwd", "jf_gelu_bwd", "jf_add", "jf_calibrate", "jf_wall_clock_khz", "jf_igemm_phase_record", "jf_rowstats_finish",
 ]
 
 _lib = None
@@ -56,9 +56,10 @@ def lib():
         L.jf_igemm_block_fp_workspace_bytes.argtypes = [_i, _i, _i, _i, _i]
         L.jf_igemm_block_fp_workspace_bytes.restype = _sz
         L.jf_igemm_phase_record.argtypes = [_p, _i]
+        L.jf_rowstats_finish.argtypes = [_p, _p, _i, _i, _i, _p, _p, _p]
         L.jf_igemm_block_q.argtypes = [_p, _p, _p, _p, _p, _p, _p, _p, _i, _i, _i, _i, _i, _i, _i, _i, _u64, _u64, _p, _sz, _p]
         L.jf_quantize.argtypes = [_p, _i, _i, _i, _p, _p, _p, _i, _i, _u64, _u64, _f, _p]
-        L.jf_dequantize.argtypes = [_p, _p, _i, _i, _i, _p, _p]
+        L.jf_dequantize.argtypes = [_p, _p, _i, _i, _i, _p, _i, _p]
         L.jf_transpose_s8.argtypes = [_p, _i, _i, _p, _p]
         L.jf_rowstats.argtypes = [_p, _p, _i, _i, _i, _f, _p, _p, _p]
         L.jf_layernorm_fwd.argtypes = [_p, _p, _p, _p, _p, _p, _i, _i, _i, _p, _p, _p]
@@ -338,10 +339,13 @@ def _block_tensor(q, s, name):
     return R, Cc, _scale_code(s, name)
 
 
-def dequantize(q, s):
+def dequantize(q, s, out_dtype=torch.float32):
+    """codes x scales as float32 (default), float16 or bfloat16 (the fp32 product rounded once)."""
     R, Cc, code = _block_tensor(q, s, "x")
-    out = torch.empty((R, Cc), dtype=torch.float32, device=q.device)
-    check(lib().jf_dequantize(_ptr(q), _ptr(s), R, Cc, code, _ptr(out), _stream()))
+    if out_dtype not in _FP_CODE:
+        raise RuntimeError("dequantize: out_dtype must be float32, float16 or bfloat16")
+    out = torch.empty((R, Cc), dtype=out_dtype, device=q.device)
+    check(lib().jf_dequantize(_ptr(q), _ptr(s), R, Cc, code, _ptr(out), _FP_CODE[out_dtype], _stream()))
     return out
 
 
@@ -440,6 +444,20 @@ def add(x1, q2, s2, rounding=ROUND_TRUNC, with_stats=False, seed=None, offset=No
     check(lib().jf_add(_ptr(x1), _FP_CODE[x1.dtype], _ptr(q2), _ptr(s2), R, Cc, code, rounding, seed, offset,
                        _ptr(y1), _ptr(q), _ptr(s), _ptr(rs), _ptr(rq), _stream()))
     return (y1, q, s, rs, rq) if with_stats else (y1, q, s)
+
+
+def rowstats_finish(rowsum, rowsq, n_cols):
+    """(mean, rstd) per row from add(..., with_stats=True)'s partial sums [R, parts]: partials added in ascending order,
+    var = E[y^2] - mean^2, rstd = 1/sqrt(var), no epsilon."""
+    _need(rowsum, torch.float32, "rowsum", 2)
+    _need(rowsq, torch.float32, "rowsq", 2)
+    if rowsum.shape != rowsq.shape:
+        raise RuntimeError("rowsum and rowsq must have the same shape")
+    R, parts = rowsum.shape
+    mean = torch.empty(R, dtype=torch.float32, device=rowsum.device)
+    rstd = torch.empty(R, dtype=torch.float32, device=rowsum.device)
+    check(lib().jf_rowstats_finish(_ptr(rowsum), _ptr(rowsq), R, parts, int(n_cols), _ptr(mean), _ptr(rstd), _stream()))
+    return mean, rstd
 
 
 CAL_UNIFORM, CAL_SPLIT, CAL_STREAM, CAL_STREAM_DATA = 0, 1, 2, 3

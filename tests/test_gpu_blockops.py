@@ -81,6 +81,16 @@ def test_dequantize(jf, oracle, f16):
     s = rand_scales(rng, (3, 5), f16=f16)
     got = jf.dequantize(dev(q), dev(s.astype(np.float16 if f16 else np.float32)))
     same(got, oracle.dequantize(q, s), "dequantize")
+    # 16-bit outputs: the fp32 product rounded once (for binary16 scales: the reference's binary16 multiplication)
+    want = torch.from_numpy(oracle.dequantize(q, s))
+    for dt in (torch.float16, torch.bfloat16):
+        got16 = jf.dequantize(dev(q), dev(s.astype(np.float16 if f16 else np.float32)), out_dtype=dt)
+        assert got16.dtype == dt and torch.equal(got16.cpu(), want.to(dt)), f"dequantize to {dt}"
+    if f16:
+        prod = torch.from_numpy(q).to(torch.float16).reshape(q.shape[0] // 32, 32, q.shape[1] // 32, 32) * \
+            torch.from_numpy(s.astype(np.float16)).unsqueeze(1).unsqueeze(3)
+        assert torch.equal(jf.dequantize(dev(q), dev(s.astype(np.float16)), out_dtype=torch.float16).cpu(),
+                           prod.reshape(q.shape)), "binary16 product (linear_fwd.py:29)"
 
 
 @pytest.mark.parametrize("f16", [True, False])
@@ -186,6 +196,16 @@ def test_add(jf, oracle, dtype, mode):
     same(s, ws, "scales")
     same(rs, wrs, "row sums")
     same(rq, wrq, "row square sums")
+    # the finishing step: partials added in ascending order, var = E[y^2] - mean^2, rstd = 1/sqrt(var), all in binary32
+    mean, rstd = jf.rowstats_finish(rs, rq, C)
+    a, b = np.zeros(R, np.float32), np.zeros(R, np.float32)
+    for j in range(C // 32):
+        a, b = a + wrs[:, j], b + wrq[:, j]
+    m = a / np.float32(C)
+    var = b / np.float32(C) - m * m
+    same(mean, m, "mean")
+    same(rstd, np.float32(1) / np.sqrt(var), "rstd")
+    assert np.allclose(m, wy.mean(-1), atol=1e-5) and np.allclose(rstd.cpu().numpy(), 1 / np.sqrt(wy.var(-1)), rtol=1e-4)
 
 
 def test_full_size_nonlinear_properties(jf, oracle):
