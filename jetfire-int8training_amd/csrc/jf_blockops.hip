@@ -695,18 +695,36 @@ using namespace jf;
 
 // mean and 1/sqrt(variance) of every row from its per-32-column partial sums (rowsum, rowsq: [R, parts], what add_kernel
 // leaves): the partials are added in ascending order, var = E[y^2] - mean^2, no epsilon (add_mean_var.py:219-221).
+constexpr int RSF_ROWS = 32;                       // rows per workgroup
 __global__ __launch_bounds__(256) void rowstats_finish_kernel(const float *rowsum, const float *rowsq, int R, int parts,
                                                               float n, float *mean, float *rstd)
 {
-    const int r = blockIdx.x * 256 + threadIdx.x;
-    if (r >= R) return;
-    const float *ps = rowsum + (size_t)r * parts, *pq = rowsq + (size_t)r * parts;
-    float a = 0.0f, b = 0.0f;
-    for (int j = 0; j < parts; ++j) { a = a + ps[j]; b = b + pq[j]; }
-    const float m = a / n;
-    const float var = b / n - m * m;
-    mean[r] = m;
-    rstd[r] = 1.0f / __builtin_sqrtf(var);
+    // the partial sums of RSF_ROWS consecutive rows are one contiguous run of each array: fetched by all threads, then
+    // one thread per row (and array) adds its row's partials in ascending order from LDS
+    extern __shared__ float rsf_lds[];                                // [2][RSF_ROWS * parts]
+    const int r0 = blockIdx.x * RSF_ROWS;
+    const int rows = (R - r0) < RSF_ROWS ? (R - r0) : RSF_ROWS;
+    const int count = rows * parts;
+    for (int i = threadIdx.x; i < count; i += 256) {
+        rsf_lds[i] = rowsum[(size_t)r0 * parts + i];
+        rsf_lds[RSF_ROWS * parts + i] = rowsq[(size_t)r0 * parts + i];
+    }
+    __syncthreads();
+    const int row = threadIdx.x & (RSF_ROWS - 1), which = threadIdx.x / RSF_ROWS;     // which: 0 = sums, 1 = squares
+    float acc = 0.0f;
+    if (which < 2 && row < rows) {
+        const float *p = rsf_lds + which * (RSF_ROWS * parts) + row * parts;
+        for (int j = 0; j < parts; ++j) acc = acc + p[j];
+    }
+    __syncthreads();
+    if (which == 1 && row < rows) rsf_lds[row] = acc;                 // hand the sum of squares to the row's other thread
+    __syncthreads();
+    if (which == 0 && row < rows) {
+        const float m = acc / n;
+        const float var = rsf_lds[row] / n - m * m;
+        mean[r0 + row] = m;
+        rstd[r0 + row] = 1.0f / __builtin_sqrtf(var);
+    }
 }
 
 #define JF_LAUNCH(kern, grid, smem, st, ...)                         \
@@ -916,8 +934,10 @@ int jf_rowstats_finish(const float *rowsum, const float *rowsq, int R, int parts
     if (!rowsum || !rowsq || !mean || !rstd) return JF_ERR_NULL;
     if (R <= 0 || parts <= 0 || C <= 0) return JF_ERR_SHAPE;
     if (!device_is_gfx950()) return JF_ERR_DEVICE;
-    hipLaunchKernelGGL(rowstats_finish_kernel, dim3((R + 255) / 256), dim3(256), 0, (hipStream_t)stream, rowsum, rowsq, R,
-                       parts, (float)C, mean, rstd);
+    if ((size_t)parts * RSF_ROWS * 2 * sizeof(float) > LDS_VECTOR_LIMIT) return JF_ERR_SHAPE;
+    hipLaunchKernelGGL(rowstats_finish_kernel, dim3((R + RSF_ROWS - 1) / RSF_ROWS), dim3(256),
+                       (size_t)parts * RSF_ROWS * 2 * sizeof(float), (hipStream_t)stream, rowsum, rowsq, R, parts, (float)C,
+                       mean, rstd);
     return (int)hipGetLastError();
 }
 
