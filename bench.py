@@ -35,7 +35,7 @@ LAYERS = [("qkv", 1600, 4800), ("proj", 1600, 1600), ("fc", 1600, 6400), ("fc2",
 
 
 def make_inputs(jf, torch, seed=0):
-    """BASELINE config 3: activations ~N(0,1) with 1% of channels x20, weights ~N(0,0.02), grads ~N(0,1e-3);
+    """benchmark configuration 3: activations ~N(0,1) with 1% of channels x20, weights ~N(0,0.02), grads ~N(0,1e-3);
     all block-quantised with fp32 scales (gradients with stochastic rounding)."""
     g = torch.Generator().manual_seed(seed)
     ops = []
@@ -153,7 +153,7 @@ def fused_fc2_dgrad_gelu_bwd(jf, torch, ops):
 
 
 def deep_k_weight_gradients(jf, torch):
-    """Weight gradients of BASELINE config 2 (GPT-2 small, 12288 tokens) and the smallest one of the XL set: few output
+    """Weight gradients of benchmark configuration 2 (GPT-2 small, 12288 tokens) and the smallest one of the XL set: few output
     tiles over a deep K.  One accumulation chain per output (the reference's arithmetic) against the library's K split
     (ordered fp32 partial sums, `splitk=0`); both read the gradient [tokens, C_out] in place."""
     out = {}
@@ -221,7 +221,7 @@ def recipe_block(torch):
 
 
 def nonlinear_extras(jf, torch):
-    """Achieved GB/s (algorithmic bytes / event time) of the memory-bound kernels at the GPT-2 XL sizes of BASELINE
+    """Achieved GB/s (algorithmic bytes / event time) of the memory-bound kernels at the GPT-2 XL sizes of benchmark
     config 4 (LayerNorm on 8192x1600, GELU on 8192x6400), fp32 scales."""
     def t(fn, n=20, replays=5):
         """Seconds per call.  Several of these kernels run for 5-15 us, less than one call of the Python wrapper

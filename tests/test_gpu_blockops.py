@@ -209,7 +209,7 @@ def test_add(jf, oracle, dtype, mode):
 
 
 def test_full_size_nonlinear_properties(jf, oracle):
-    """BASELINE config 4 sizes.  Checked bit-exactly against the oracle on row slabs (the kernels are
+    """benchmark configuration 4 sizes.  Checked bit-exactly against the oracle on row slabs (the kernels are
     block-local, so a slab of the input is a complete problem), and by size-independent properties."""
     g = torch.Generator().manual_seed(0)
     x = torch.randn(8192, 6400, generator=g)

@@ -321,7 +321,7 @@ def test_sr_mean_converges(jf, oracle):
 
 
 def _xl_inputs(T, Cin, Cout, seed):
-    """BASELINE config 3 style data: 1% outlier channels x20, weights ~N(0,0.02), grads ~N(0,1e-3)."""
+    """benchmark configuration 3 style data: 1% outlier channels x20, weights ~N(0,0.02), grads ~N(0,1e-3)."""
     g = torch.Generator().manual_seed(seed)
     x = torch.randn(T, Cin, generator=g)
     idx = torch.randperm(Cin, generator=g)[: (Cin + 99) // 100]
@@ -369,7 +369,7 @@ def test_full_size_xl_fc_slabs(jf, oracle):
 
 
 def test_full_size_stress_cube_slabs(jf, oracle):
-    """BASELINE config 5: M = N = K = 8192, heavy-tailed A (Student-t, 3 degrees of freedom), B ~ N(0, 0.02);
+    """benchmark configuration 5: M = N = K = 8192, heavy-tailed A (Student-t, 3 degrees of freedom), B ~ N(0, 0.02);
     requantised output in deterministic and stochastic mode, checked bit-exactly on row slabs."""
     n = 8192
     g = torch.Generator().manual_seed(0)
@@ -395,7 +395,7 @@ def test_full_size_stress_cube_slabs(jf, oracle):
 
 
 def test_full_size_small_wgrad_deep_k(jf, oracle):
-    """BASELINE config 2 (GPT-2 small, 12288 tokens): the weight gradient of the qkv layer, K = 12288 deep with few
+    """benchmark configuration 2 (GPT-2 small, 12288 tokens): the weight gradient of the qkv layer, K = 12288 deep with few
     output tiles (2304 x 768), both operands read in place from their token-major arrays' natural layouts."""
     T, Cin, Cout = 12288, 768, 2304
     g = torch.Generator().manual_seed(0)
