@@ -67,6 +67,7 @@ struct GemmArgs {
     const void *Xs;       // [M/32, N/32]
     uint64_t seed2, offset2;   // noise of the GELU backward's own requantisation   (EPI_QB)
     int rounding2;        // JF_ROUND_NEAREST / JF_ROUND_STOCHASTIC   (EPI_QB)
+    int even_pace;        // wave priorities that keep the resident workgroups of a CU in step (set by the launcher, see there)
     unsigned long long *phases;   // PROF kernels: 8 words per workgroup (jf_igemm_phase_record), first phase_capacity workgroups
     int phase_capacity;
 };
@@ -102,6 +103,8 @@ constexpr int WBM = 2, WBN = 1;
 // AKM = 1: A is [K, lda] (M-contiguous rows), staged and read like a [K,N] B operand (below).
 // BKN = 0: B is [N, ldb] (K-contiguous rows, like A).  BKN = 1: B is [K, ldb] (N-contiguous rows); its tile is staged
 // as it lies in memory and the K-contiguous MFMA operand is produced by the transposing LDS read of gfx950.
+static int cu_count();
+
 // PROF = 1: the first wave of every workgroup also records when the workgroup's phases began and ended (wall clock) and
 // how many shader cycles its main loop took: a profiling build of the same code, launched only while a recording buffer
 // is set (jf_igemm_phase_record).
@@ -468,10 +471,11 @@ __global__ __launch_bounds__(64 * WGM * WGN, WGPC * WGM * WGN / 4) void igemm_nt
     // tiles) keeps its part in the loads and barriers of the workgroup but neither reads operands nor multiplies: the
     // SIMD it sits on is left to the waves of the other resident workgroup.  ACTIVE = false is that walk.
     const bool wave_active = m0 + wm * (WBM * QB) < p.M && n0 + wn * (WBN * QB) < p.N;        // wave-uniform
+    const bool even_pace = p.even_pace != 0;
     long long prof_c0 = 0;
     if (PROF) { phase(1, (unsigned long long)wall_clock64()); prof_c0 = clock64(); }
-    auto main_loop = [&](auto active_c) {
-    constexpr bool ACTIVE = decltype(active_c)::value;
+    auto main_loop = [&](auto active_c, auto pace_c) {
+    constexpr bool ACTIVE = decltype(active_c)::value, PACE = decltype(pace_c)::value;
     if constexpr (ACTIVE) fetch(fa_u[0], fb_u[0], 0u, sc_v, c0{}, c0{}, c0{}, c0{});
 
     for (int s0 = 0; s0 < nfull; s0 += NSTAGE) static_for<0, NSTAGE>([&](auto slot_c) {
@@ -505,6 +509,11 @@ __global__ __launch_bounds__(64 * WGM * WGN, WGPC * WGM * WGN / 4) void igemm_nt
                           std::integral_constant<int, SLOT * STAGE_BYTES + (kb + 1) * 4096>{},
                           std::integral_constant<int, SLOT * 64 + (kb + 1) * 16>{}, std::integral_constant<int, NXT>{});
             }
+            // Wave priority rises with the K block of the stage (and falls back at the next stage): the arbiter of a SIMD
+            // otherwise always serves its oldest wave first, so the older of two resident workgroups runs about 1.4 times
+            // as fast as the younger one and the second wave of a workgroup on a SIMD trails the first by a quarter of a
+            // stage.
+            if constexpr (PACE) __builtin_amdgcn_s_setprio(kb);
             if constexpr (ACTIVE) {
                 fetched(std::integral_constant<int, FETCH_OPS>{}, std::integral_constant<int, CUR>{});
                 __builtin_amdgcn_sched_barrier(0);            // the reads above stay above the products below,
@@ -530,8 +539,9 @@ __global__ __launch_bounds__(64 * WGM * WGN, WGPC * WGM * WGN / 4) void igemm_nt
         });
     }
     };
-    if (wave_active) main_loop(std::true_type{});
-    else main_loop(std::false_type{});
+    if (!wave_active) main_loop(std::false_type{}, std::false_type{});
+    else if (even_pace) main_loop(std::true_type{}, std::true_type{});
+    else main_loop(std::true_type{}, std::false_type{});
     __builtin_amdgcn_s_waitcnt(0xC07F);                        // the last, unused prefetch must land before its registers are reused
     if (EPI != EPI_S32 && wave_active) {
         accumulate(std::integral_constant<int, NBLK - 1>{});
@@ -595,6 +605,7 @@ __global__ __launch_bounds__(64 * WGM * WGN, WGPC * WGM * WGN / 4) void igemm_nt
         }
     }
     if (PROF) { phase(2, (unsigned long long)wall_clock64()); phase(7, (unsigned long long)(clock64() - prof_c0)); }
+    if (even_pace) __builtin_amdgcn_s_setprio(0);
     __syncthreads();           // the epilogue reuses the ring as scratch
     if (PROF) phase(3, (unsigned long long)wall_clock64());
 
@@ -841,6 +852,14 @@ static int launch_gemm_cfg(const GemmArgs &a, hipStream_t st)
         opted_in[dev].store(true, std::memory_order_release);
     }
     if (EPI != EPI_FP || p.splits < 1) p.splits = 1;
+    // Pace of the workgroups that share a CU.  Left to the hardware, the older one runs ahead: a launch ends with every CU
+    // half empty while the younger workgroups finish alone, at two thirds of the shared throughput (two waves per SIMD
+    // meeting at a barrier).  Kept in step by wave priorities they finish together: 5-16 % faster for launches of up to
+    // two rounds of workgroups.  The exception is a launch of between 1 and 1.5 rounds: there the early finishers are what
+    // starts the short second round early, and the hardware's order is up to 9 % better.  Beyond two rounds the two
+    // orders are within 3 % of each other, either way depending on shape and data: left to the hardware.
+    const long wgs = (long)p.tiles_m * p.tiles_n * p.splits, slots = (long)WGPC * cu_count();
+    p.even_pace = wgs <= slots || (2 * wgs >= 3 * slots && wgs <= 2 * slots);
     hipLaunchKernelGGL(kern, dim3(p.tiles_m * p.tiles_n * p.splits), dim3(NT), SMEM, st, p);
     return (int)hipGetLastError();
 }
