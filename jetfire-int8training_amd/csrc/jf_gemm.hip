@@ -42,6 +42,8 @@ constexpr int EPI_LD = 36;                          // floats per staged row (32
 // EPI_QB: EPI_Q (stochastic: an activation gradient) followed by the GELU backward of the block just requantised against
 //         the saved forward input of the GELU: only the result of the GELU backward leaves
 enum Epilogue { EPI_S32 = 0, EPI_FP = 1, EPI_Q = 2, EPI_QG = 3, EPI_QB = 4 };
+// Wave-priority schemes of the main loop (launch_gemm_cfg picks one per launch)
+enum Pace { PACE_HARDWARE = 0, PACE_EVEN = 1, PACE_ORDERED = 2 };
 
 struct GemmArgs {
     const int8_t *A;      // [M, lda] (K-contiguous) or, for the AKM kernels, [K, lda] (M-contiguous rows)
@@ -67,7 +69,7 @@ struct GemmArgs {
     const void *Xs;       // [M/32, N/32]
     uint64_t seed2, offset2;   // noise of the GELU backward's own requantisation   (EPI_QB)
     int rounding2;        // JF_ROUND_NEAREST / JF_ROUND_STOCHASTIC   (EPI_QB)
-    int even_pace;        // wave priorities that keep the resident workgroups of a CU in step (set by the launcher, see there)
+    int pace;             // PACE_*: wave priorities that order the resident workgroups of a CU (set by the launcher, see there)
     unsigned long long *phases;   // PROF kernels: 8 words per workgroup (jf_igemm_phase_record), first phase_capacity workgroups
     int phase_capacity;
 };
@@ -471,11 +473,13 @@ __global__ __launch_bounds__(64 * WGM * WGN, WGPC * WGM * WGN / 4) void igemm_nt
     // tiles) keeps its part in the loads and barriers of the workgroup but neither reads operands nor multiplies: the
     // SIMD it sits on is left to the waves of the other resident workgroup.  ACTIVE = false is that walk.
     const bool wave_active = m0 + wm * (WBM * QB) < p.M && n0 + wn * (WBN * QB) < p.N;        // wave-uniform
-    const bool even_pace = p.even_pace != 0;
+    // which of the CU's two workgroup slots this is: the base of its LDS allocation (bits 7:0 of the LDS_ALLOC register)
+    const bool second_slot = (__builtin_amdgcn_s_getreg((31 << 11) | 6) & 0xFF) != 0;
     long long prof_c0 = 0;
     if (PROF) { phase(1, (unsigned long long)wall_clock64()); prof_c0 = clock64(); }
     auto main_loop = [&](auto active_c, auto pace_c) {
-    constexpr bool ACTIVE = decltype(active_c)::value, PACE = decltype(pace_c)::value;
+    constexpr bool ACTIVE = decltype(active_c)::value;
+    constexpr int PACE = decltype(pace_c)::value;
     if constexpr (ACTIVE) fetch(fa_u[0], fb_u[0], 0u, sc_v, c0{}, c0{}, c0{}, c0{});
 
     for (int s0 = 0; s0 < nfull; s0 += NSTAGE) static_for<0, NSTAGE>([&](auto slot_c) {
@@ -509,11 +513,14 @@ __global__ __launch_bounds__(64 * WGM * WGN, WGPC * WGM * WGN / 4) void igemm_nt
                           std::integral_constant<int, SLOT * STAGE_BYTES + (kb + 1) * 4096>{},
                           std::integral_constant<int, SLOT * 64 + (kb + 1) * 16>{}, std::integral_constant<int, NXT>{});
             }
-            // Wave priority rises with the K block of the stage (and falls back at the next stage): the arbiter of a SIMD
-            // otherwise always serves its oldest wave first, so the older of two resident workgroups runs about 1.4 times
-            // as fast as the younger one and the second wave of a workgroup on a SIMD trails the first by a quarter of a
-            // stage.
-            if constexpr (PACE) __builtin_amdgcn_s_setprio(kb);
+            // The arbiter of a SIMD serves its oldest wave first, so the older of two resident workgroups runs about 1.4
+            // times as fast as the younger one and the second wave of a workgroup on a SIMD trails the first by a quarter
+            // of a stage.  PACE_EVEN: priority rises with the K block of the stage (and falls back at the next stage):
+            // all four waves of a SIMD advance together.  PACE_ORDERED: the workgroup in the CU's second LDS slot always
+            // goes before the one in the first, and inside a workgroup the wave that is behind goes first.
+            if constexpr (PACE == PACE_EVEN) __builtin_amdgcn_s_setprio(kb);
+            if constexpr (PACE == PACE_ORDERED && kb == 0) { if (second_slot) __builtin_amdgcn_s_setprio(3); else __builtin_amdgcn_s_setprio(1); }
+            if constexpr (PACE == PACE_ORDERED && kb == 2) { if (second_slot) __builtin_amdgcn_s_setprio(2); else __builtin_amdgcn_s_setprio(0); }
             if constexpr (ACTIVE) {
                 fetched(std::integral_constant<int, FETCH_OPS>{}, std::integral_constant<int, CUR>{});
                 __builtin_amdgcn_sched_barrier(0);            // the reads above stay above the products below,
@@ -539,9 +546,10 @@ __global__ __launch_bounds__(64 * WGM * WGN, WGPC * WGM * WGN / 4) void igemm_nt
         });
     }
     };
-    if (!wave_active) main_loop(std::false_type{}, std::false_type{});
-    else if (even_pace) main_loop(std::true_type{}, std::true_type{});
-    else main_loop(std::true_type{}, std::false_type{});
+    if (!wave_active) main_loop(std::false_type{}, std::integral_constant<int, PACE_HARDWARE>{});
+    else if (p.pace == PACE_EVEN) main_loop(std::true_type{}, std::integral_constant<int, PACE_EVEN>{});
+    else if (p.pace == PACE_ORDERED) main_loop(std::true_type{}, std::integral_constant<int, PACE_ORDERED>{});
+    else main_loop(std::true_type{}, std::integral_constant<int, PACE_HARDWARE>{});
     __builtin_amdgcn_s_waitcnt(0xC07F);                        // the last, unused prefetch must land before its registers are reused
     if (EPI != EPI_S32 && wave_active) {
         accumulate(std::integral_constant<int, NBLK - 1>{});
@@ -605,7 +613,7 @@ __global__ __launch_bounds__(64 * WGM * WGN, WGPC * WGM * WGN / 4) void igemm_nt
         }
     }
     if (PROF) { phase(2, (unsigned long long)wall_clock64()); phase(7, (unsigned long long)(clock64() - prof_c0)); }
-    if (even_pace) __builtin_amdgcn_s_setprio(0);
+    if (p.pace != PACE_HARDWARE) __builtin_amdgcn_s_setprio(0);
     __syncthreads();           // the epilogue reuses the ring as scratch
     if (PROF) phase(3, (unsigned long long)wall_clock64());
 
@@ -854,12 +862,17 @@ static int launch_gemm_cfg(const GemmArgs &a, hipStream_t st)
     if (EPI != EPI_FP || p.splits < 1) p.splits = 1;
     // Pace of the workgroups that share a CU.  Left to the hardware, the older one runs ahead: a launch ends with every CU
     // half empty while the younger workgroups finish alone, at two thirds of the shared throughput (two waves per SIMD
-    // meeting at a barrier).  Kept in step by wave priorities they finish together: 5-16 % faster for launches of up to
-    // two rounds of workgroups.  The exception is a launch of between 1 and 1.5 rounds: there the early finishers are what
-    // starts the short second round early, and the hardware's order is up to 9 % better.  Beyond two rounds the two
-    // orders are within 3 % of each other, either way depending on shape and data: left to the hardware.
+    // meeting at a barrier).  Kept in step by wave priorities (PACE_EVEN) they finish together: 5-16 % faster for launches
+    // of up to two rounds of workgroups.  The exception is a launch of between 1 and 1.5 rounds: there the early finishers
+    // are what starts the short second round early, and an even pace is 5-9 % slower than the hardware's order.  A strict
+    // order with fairness inside each workgroup (PACE_ORDERED) does that job 4-6 % better than the hardware when tiles are
+    // long (K >= 4096) and 5-16 % worse when they are short.  Beyond two rounds the schemes are within 3 % of each other,
+    // either way depending on shape and data: left to the hardware.  (All measured; results do not depend on the scheme.)
     const long wgs = (long)p.tiles_m * p.tiles_n * p.splits, slots = (long)WGPC * cu_count();
-    p.even_pace = wgs <= slots || (2 * wgs >= 3 * slots && wgs <= 2 * slots);
+    const bool short_second_round = wgs > slots && 2 * wgs < 3 * slots;
+    const int k_per_wg = p.splits > 1 ? p.kb_per_split * QB : p.K;
+    p.pace = short_second_round ? (k_per_wg >= 4096 ? PACE_ORDERED : PACE_HARDWARE)
+                                : (wgs <= 2 * slots ? PACE_EVEN : PACE_HARDWARE);
     hipLaunchKernelGGL(kern, dim3(p.tiles_m * p.tiles_n * p.splits), dim3(NT), SMEM, st, p);
     return (int)hipGetLastError();
 }
