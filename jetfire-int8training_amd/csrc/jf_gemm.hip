@@ -473,8 +473,9 @@ __global__ __launch_bounds__(64 * WGM * WGN, WGPC * WGM * WGN / 4) void igemm_nt
     // tiles) keeps its part in the loads and barriers of the workgroup but neither reads operands nor multiplies: the
     // SIMD it sits on is left to the waves of the other resident workgroup.  ACTIVE = false is that walk.
     const bool wave_active = m0 + wm * (WBM * QB) < p.M && n0 + wn * (WBN * QB) < p.N;        // wave-uniform
-    // which of the CU's two workgroup slots this is: the base of its LDS allocation (bits 7:0 of the LDS_ALLOC register)
-    const bool second_slot = (__builtin_amdgcn_s_getreg((31 << 11) | 6) & 0xFF) != 0;
+    // which of the CU's two workgroup slots this is: the base of its LDS allocation (the low field of the LDS_ALLOC
+    // register; its size field starts at bit 12)
+    const bool second_slot = (__builtin_amdgcn_s_getreg((31 << 11) | 6) & 0xFFF) != 0;
     long long prof_c0 = 0;
     if (PROF) { phase(1, (unsigned long long)wall_clock64()); prof_c0 = clock64(); }
     auto main_loop = [&](auto active_c, auto pace_c) {
