@@ -622,21 +622,21 @@ __global__ __launch_bounds__(64 * WGM * WGN, WGPC * WGM * WGN / 4) void igemm_nt
     // One 32x32 block at a time goes through a wave-private LDS patch that turns the MFMA result layout
     //   (lane l, register v  <->  row 8*(v/4) + 4*(l/32) + v%4, column l%32)
     // into a row layout (lane l <-> row l/2, columns 16*(l%2) .. +15): 16 consecutive columns per lane are what the
-    // Philox noise (8 elements per call) and 16-byte packing want.  One- and two-byte outputs are then collected in
-    // a workgroup-wide LDS image of the tile and written out in full 128-byte (or 256-byte) rows; four-byte outputs
-    // (INT32, fp32) are stored straight from the row layout (64 contiguous bytes per lane).
+    // Philox noise (8 elements per call) and 16-byte packing want.  Two-byte outputs are then collected in a
+    // workgroup-wide LDS image of the tile and written out in full 256-byte rows; INT8 codes (16 bytes per lane, two
+    // lanes per row of the block: measured 1 % faster than through an image and a barrier) and four-byte outputs (64
+    // contiguous bytes per lane) are stored straight from the row layout.
     auto wave_sync = [] {
         __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
         __builtin_amdgcn_wave_barrier();
         __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
     };
     float *patch = reinterpret_cast<float *>(smem) + wave * (QB * EPI_LD);
-    unsigned char *tile = smem + NW * (QB * EPI_LD) * sizeof(float);       // [BM][BN * out_bytes]
+    unsigned char *tile = smem + NW * (QB * EPI_LD) * sizeof(float);       // [BM][BN * 2]: two-byte outputs only
     const int rrow = lane >> 1, rcol = (lane & 1) * 16;
     constexpr bool QUANT = EPI == EPI_Q || EPI == EPI_QG || EPI == EPI_QB;
     const float biasmax = (QUANT && p.biasmax) ? p.biasmax[0] : 0.0f;
     const int out_bytes = QUANT ? 1 : (EPI == EPI_FP && p.out_dtype != JF_FP_F32 ? 2 : 4);   // uniform
-    unsigned char *tile2 = tile + BM * BN;                    // EPI_QG: image of the second output
     float gelu_f0 = 0.0f;                                     // gelu(+0), evaluated on the device like every table entry
     if (EPI == EPI_QG) {
         float zero = 0.0f;
@@ -764,7 +764,7 @@ __global__ __launch_bounds__(64 * WGM * WGN, WGPC * WGM * WGN / 4) void igemm_nt
                     scale = scale2;
                     wave_sync();                              // the table is the next block's patch
                 }
-                *reinterpret_cast<v4i *>(tile + (size_t)trow * BN + tcol) = codes;
+                *reinterpret_cast<v4i *>(reinterpret_cast<int8_t *>(p.C) + e0) = codes;     // 16 of a row's 32 bytes
                 if (lane == 0) store_scale(reinterpret_cast<ST *>(p.sc), (bm / QB) * SN + bn / QB, scale);
                 if (EPI == EPI_QG) {
                     // GELU of the block as a reader of the stored tensor would see it (codes x the scale rounded to ST),
@@ -776,7 +776,7 @@ __global__ __launch_bounds__(64 * WGM * WGN, WGPC * WGM * WGN / 4) void igemm_nt
                     const v4i codes2 = p.gelu_approx == JF_GELU_TANH
                         ? gelu_fwd_block<JF_GELU_TANH>(codes, stored, gelu_f0, p.gelu_eps, tab, qtab, lane, &scale2)
                         : gelu_fwd_block<JF_GELU_ERF>(codes, stored, gelu_f0, p.gelu_eps, tab, qtab, lane, &scale2);
-                    *reinterpret_cast<v4i *>(tile2 + (size_t)trow * BN + tcol) = codes2;
+                    *reinterpret_cast<v4i *>(reinterpret_cast<int8_t *>(p.C2) + e0) = codes2;
                     if (lane == 0) store_scale(reinterpret_cast<ST *>(p.sc2), (bm / QB) * SN + bn / QB, scale2);
                     wave_sync();                              // the tables are the next block's patch
                 }
@@ -784,7 +784,7 @@ __global__ __launch_bounds__(64 * WGM * WGN, WGPC * WGM * WGN / 4) void igemm_nt
         }
 
     if (PROF) phase(4, (unsigned long long)wall_clock64());
-    if (out_bytes < 4) {
+    if (out_bytes == 2) {
         __syncthreads();
         // the tile image leaves in whole rows: consecutive lanes write consecutive 16-byte chunks of a row
         const int row_bytes = BN * out_bytes, chunks_per_row = row_bytes / 16;
@@ -795,9 +795,6 @@ __global__ __launch_bounds__(64 * WGM * WGN, WGPC * WGM * WGN / 4) void igemm_nt
             if (gm < p.M && gn < p.N)
                 *reinterpret_cast<v4i *>(cbase + ((size_t)gm * p.N + gn) * out_bytes) =
                     *reinterpret_cast<const v4i *>(tile + (size_t)row * row_bytes + ch * 16);
-            if (EPI == EPI_QG && gm < p.M && gn < p.N)
-                *reinterpret_cast<v4i *>(reinterpret_cast<unsigned char *>(p.C2) + (size_t)gm * p.N + gn) =
-                    *reinterpret_cast<const v4i *>(tile2 + (size_t)row * row_bytes + ch * 16);
         }
     }
     if (PROF) phase(5, (unsigned long long)wall_clock64());
@@ -843,7 +840,7 @@ static int launch_gemm_cfg(const GemmArgs &a, hipStream_t st)
 {
     constexpr int BM = QB * WBM * WGM, BN = QB * WBN * WGN, NT = 64 * WGM * WGN;
     constexpr int RING = NSTAGE * (BM + BN) * ROW_BYTES + WGM * WGN * NSTAGE * 256;   // operand ring + per-wave scale patches
-    constexpr int PATCH = WGM * WGN * QB * EPI_LD * (int)sizeof(float) + (EPI == EPI_S32 ? 0 : BM * BN * ((EPI == EPI_Q || EPI == EPI_QB) ? 1 : 2));   // + tile image(s): bytes, 2-byte values, or two of bytes
+    constexpr int PATCH = WGM * WGN * QB * EPI_LD * (int)sizeof(float) + (EPI == EPI_FP ? BM * BN * 2 : 0);   // + the tile image of 2-byte outputs
     constexpr int SMEM = RING > PATCH ? RING : PATCH;
     if (!device_is_gfx950()) return JF_ERR_DEVICE;
     GemmArgs p = a;
