@@ -622,21 +622,18 @@ __global__ __launch_bounds__(64 * WGM * WGN, WGPC * WGM * WGN / 4) void igemm_nt
     // One 32x32 block at a time goes through a wave-private LDS patch that turns the MFMA result layout
     //   (lane l, register v  <->  row 8*(v/4) + 4*(l/32) + v%4, column l%32)
     // into a row layout (lane l <-> row l/2, columns 16*(l%2) .. +15): 16 consecutive columns per lane are what the
-    // Philox noise (8 elements per call) and 16-byte packing want.  Two-byte outputs are then collected in a
-    // workgroup-wide LDS image of the tile and written out in full 256-byte rows; INT8 codes (16 bytes per lane, two
-    // lanes per row of the block: measured 1 % faster than through an image and a barrier) and four-byte outputs (64
-    // contiguous bytes per lane) are stored straight from the row layout.
+    // Philox noise (8 elements per call) and 16-byte packing want.  Results are stored straight from the row layout: 16,
+    // 32 or 64 contiguous bytes per lane, two lanes per row of the block (measured 1 % faster than collecting one- and
+    // two-byte outputs in a workgroup-wide LDS image of the tile and writing that out in whole rows behind a barrier).
     auto wave_sync = [] {
         __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
         __builtin_amdgcn_wave_barrier();
         __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
     };
     float *patch = reinterpret_cast<float *>(smem) + wave * (QB * EPI_LD);
-    unsigned char *tile = smem + NW * (QB * EPI_LD) * sizeof(float);       // [BM][BN * 2]: two-byte outputs only
     const int rrow = lane >> 1, rcol = (lane & 1) * 16;
     constexpr bool QUANT = EPI == EPI_Q || EPI == EPI_QG || EPI == EPI_QB;
     const float biasmax = (QUANT && p.biasmax) ? p.biasmax[0] : 0.0f;
-    const int out_bytes = QUANT ? 1 : (EPI == EPI_FP && p.out_dtype != JF_FP_F32 ? 2 : 4);   // uniform
     float gelu_f0 = 0.0f;                                     // gelu(+0), evaluated on the device like every table entry
     if (EPI == EPI_QG) {
         float zero = 0.0f;
@@ -692,8 +689,6 @@ __global__ __launch_bounds__(64 * WGM * WGN, WGPC * WGM * WGN / 4) void igemm_nt
             }
             wave_sync();
             const size_t e0 = (size_t)(bm + rrow) * p.N + bn + rcol;
-            // position of the lane's 16 values inside the workgroup's tile image
-            const int trow = (wm * WBM + i) * QB + rrow, tcol = (wn * WBN + j) * QB + rcol;
             if (EPI == EPI_S32) {
                 v4i *dst = reinterpret_cast<v4i *>(reinterpret_cast<int32_t *>(p.C) + e0);
 #pragma unroll
@@ -723,7 +718,7 @@ __global__ __launch_bounds__(64 * WGM * WGN, WGPC * WGM * WGN / 4) void igemm_nt
                         for (int k = 0; k < 16; ++k) h[k] = (__bf16)x[k];
                         lo = *reinterpret_cast<v4i *>(&h[0]); hi = *reinterpret_cast<v4i *>(&h[8]);
                     }
-                    v4i *dst = reinterpret_cast<v4i *>(tile + (size_t)trow * (BN * 2) + tcol * 2);
+                    v4i *dst = reinterpret_cast<v4i *>(reinterpret_cast<unsigned char *>(p.C) + e0 * 2);   // 32 of a row's 64 bytes
                     dst[0] = lo; dst[1] = hi;
                 }
             } else {
@@ -784,19 +779,6 @@ __global__ __launch_bounds__(64 * WGM * WGN, WGPC * WGM * WGN / 4) void igemm_nt
         }
 
     if (PROF) phase(4, (unsigned long long)wall_clock64());
-    if (out_bytes == 2) {
-        __syncthreads();
-        // the tile image leaves in whole rows: consecutive lanes write consecutive 16-byte chunks of a row
-        const int row_bytes = BN * out_bytes, chunks_per_row = row_bytes / 16;
-        unsigned char *cbase = reinterpret_cast<unsigned char *>(p.C);
-        for (int idx = tid; idx < BM * chunks_per_row; idx += 64 * NW) {
-            const int row = idx / chunks_per_row, ch = idx - row * chunks_per_row;
-            const int gm = m0 + row, gn = n0 + ch * (16 / out_bytes);
-            if (gm < p.M && gn < p.N)
-                *reinterpret_cast<v4i *>(cbase + ((size_t)gm * p.N + gn) * out_bytes) =
-                    *reinterpret_cast<const v4i *>(tile + (size_t)row * row_bytes + ch * 16);
-        }
-    }
     if (PROF) phase(5, (unsigned long long)wall_clock64());
 #undef phase
 }
@@ -840,7 +822,7 @@ static int launch_gemm_cfg(const GemmArgs &a, hipStream_t st)
 {
     constexpr int BM = QB * WBM * WGM, BN = QB * WBN * WGN, NT = 64 * WGM * WGN;
     constexpr int RING = NSTAGE * (BM + BN) * ROW_BYTES + WGM * WGN * NSTAGE * 256;   // operand ring + per-wave scale patches
-    constexpr int PATCH = WGM * WGN * QB * EPI_LD * (int)sizeof(float) + (EPI == EPI_FP ? BM * BN * 2 : 0);   // + the tile image of 2-byte outputs
+    constexpr int PATCH = WGM * WGN * QB * EPI_LD * (int)sizeof(float);     // the epilogue's per-wave transposition patches
     constexpr int SMEM = RING > PATCH ? RING : PATCH;
     if (!device_is_gfx950()) return JF_ERR_DEVICE;
     GemmArgs p = a;
