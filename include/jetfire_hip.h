@@ -156,6 +156,18 @@ int jf_igemm_block_q_gelu_bwd(const int8_t *A, const int8_t *B, const void *sa, 
                               int sb_layout, int gelu_approx, uint64_t seed, uint64_t offset, int gelu_rounding,
                               uint64_t gelu_seed, uint64_t gelu_offset, jf_stream_t stream);
 
+/* jf_igemm_block_q with the dequantisation of its result fused into the epilogue: out[M,N] (out_dtype: JF_FP_*) =
+ * codes x scales of the block tensor jf_igemm_block_q would have stored (scales rounded to scale_dtype as it stores
+ * them), i.e. what jf_dequantize of that result returns, bit for bit; the INT8 tensor itself is never written.
+ * Replaces the reference's unquantised-output path, which runs the quantising GEMM and multiplies codes by scales in a
+ * second pass: int8_linear_forward(..., output_quantized=False) (Jetfire/Linear/linear_fwd.py:22-32; the QKV projection,
+ * INT8_GPT2/qmodel.py:103) and int8_linear_backward(..., dgrad_quantize=False) (Jetfire/Linear/linear_bwd.py:17-29; the
+ * activation gradient of the attention output projection, INT8_GPT2/qmodel.py:168). */
+int jf_igemm_block_q_dequant(const int8_t *A, const int8_t *B, const void *sa, const void *sb, const float *bias,
+                             const float *biasmax, void *out, int M, int N, int K, int b_layout, int scale_dtype,
+                             int sa_layout, int sb_layout, int out_dtype, int rounding, uint64_t seed, uint64_t offset,
+                             jf_stream_t stream);
+
 /* Block quantise x[R,C] (x_dtype: JF_FP_*) -> (q, s); optionally also qT[C,R] = q transposed.
  * Replaces int8_quantize (Jetfire/Nonlinear/quantize.py:128-164) and, with qT != NULL,
  * int8_quantize_transpose (Jetfire/Nonlinear/quantize_transpose.py:131-171). */

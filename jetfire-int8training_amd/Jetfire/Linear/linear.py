@@ -46,13 +46,6 @@ def _check_block(B):
         raise RuntimeError(f"the INT8 GEMM kernels use 32x32 quantisation blocks, got B={B}")
 
 
-def _dequant_like(q2d, s2d, lead_shape):
-    """codes x scales in the scales' dtype, as the reference's unquantised-output path computes it (linear_fwd.py:29-31):
-    one kernel, no fp32 intermediate."""
-    out = _jf.dequantize(q2d, s2d, out_dtype=s2d.dtype)
-    return out.reshape(*lead_shape, q2d.shape[-1])
-
-
 def int8_linear_forward(X8_3D, SX16_3D, W8, SW16, output_quantized, B):
     """Y = X W^T.  X8 [BS,T,K] (or [M,K]), SX [BS,T/32,K/32]; W8 [N,K], SW [N/32,K/32].
     Returns (O8 [BS,T,N], SO [BS,T/32,N/32]) or, with output_quantized=False, the dequantised
@@ -65,10 +58,13 @@ def int8_linear_forward(X8_3D, SX16_3D, W8, SW16, output_quantized, B):
     n_out = W8.shape[0]
     m, k = x2.shape
     zero_bias, zero_biasmax = _zero_bias(n_out, W8.device)
+    if not output_quantized:
+        # the quantising GEMM and the codes x scales product of the reference (linear_fwd.py:22-31) in one kernel: same bits
+        out = _jf.igemm_block_q_dequant(x2.contiguous(), W8.contiguous(), _k_major(sx2), _k_major(SW16), _jf.B_NK,
+                                        out_dtype=SW16.dtype)
+        return out.reshape(*lead, n_out)
     o8, so = BQC.igemm_output_int_quantize_bias_rowcol(x2.contiguous(), W8.t(), zero_bias, zero_biasmax,
                                                        _k_major(sx2), _k_major(SW16), m, n_out, k)
-    if not output_quantized:
-        return _dequant_like(o8, so, lead)
     return o8.reshape(*lead, n_out), so.reshape(*s_lead, SW16.shape[0])
 
 
@@ -103,12 +99,18 @@ def int8_linear_backward(X8_3D, SX16_3D, G8_3D, SG16_3D, G8T, W8, SW16, B, stoch
     x2, sx2 = _flat2(X8_3D).contiguous(), _flat2(SX16_3D).contiguous()
     tokens, c_out = g2.shape
     c_in = W8.shape[1]
-    gx8, gsx = BQC.igemm_output_int_quantize_stochastic(g2, W8, _k_major(sg2), SW16, tokens, c_in, c_out)
+    if dgrad_quantize:
+        gx8, gsx = BQC.igemm_output_int_quantize_stochastic(g2, W8, _k_major(sg2), SW16, tokens, c_in, c_out)
+    else:
+        # the stochastic quantising GEMM and the codes x scales product of the reference (linear_bwd.py:17,26-28) in one
+        # kernel: same bits, same noise counters
+        gx = _jf.igemm_block_q_dequant(g2, W8.contiguous(), _k_major(sg2), SW16, _jf.B_KN, out_dtype=SW16.dtype,
+                                       rounding=_jf.ROUND_STOCHASTIC)
     if G8T is None:
         G8T = g2.t()                                               # a view: the extension reads g2 as the [K, M] operand
     gw = BQC.igemm_output_fp_no_quantize(G8T, x2, sg2, sx2, G8T.shape[0], c_in, G8T.shape[1], wgrad_splitk, wgrad_dtype)
     if not dgrad_quantize:
-        return _dequant_like(gx8, gsx, tuple(G8_3D.shape[:-1])), gw
+        return gx.reshape(*G8_3D.shape[:-1], c_in), gw
     return (gx8.reshape(*G8_3D.shape[:-1], c_in), gsx.reshape(*SG16_3D.shape[:-1], SW16.shape[1]), gw)
 
 

@@ -282,13 +282,13 @@ __global__ __launch_bounds__(NT) void gelu_bwd_kernel(const int8_t *qx, const ST
 // layernorm.py:74-190, with a real beta.  Arithmetic (this library's definition; the reference dequantises in binary16):
 //   a = s * rstd[r],  b = -(mean[r] * rstd[r]),  xhat = fma(float(q), a, b),  y = fma(xhat, gamma[c], beta[c])
 // i.e. dequantisation and normalisation are one fma per element with two per-row, per-block constants.
-// The codes, scales and row statistics of the next PF blocks of a wave are requested ahead of their use.
 // One wave: one column block x CW_ROWS consecutive row blocks (gamma and beta are loaded once per wave); the four waves
-// of a workgroup take four adjacent column blocks, i.e. whole 128-byte lines per row.  A wave requests everything it
-// will read before it computes anything (per-column vectors first: they are needed first), works through its blocks in
-// the order their data arrives, and stores all results at the end: no wait ever follows a store (the vector-memory
-// counter cannot tell a finished load from an unfinished store, so a wait behind a store waits for the store too).
-constexpr int CW_ROWS = 4;
+// of a workgroup take four adjacent column blocks, i.e. whole 128-byte lines per row.  The source asks for everything a
+// wave reads before it computes anything and stores at the end.  Measured at 8192x1600: storing each block as soon as it
+// is done, or pinning the requests above the arithmetic (the compiler moves those of the later blocks behind the first
+// block's), changes nothing; what counts is how evenly the waves fill the SIMDs: 9.1 us with 2 row blocks per wave (6.5
+// waves per SIMD), 10.0 us with 4 (3.25: a quarter of the SIMDs get a fourth wave), 11.6 us with 8.
+constexpr int CW_ROWS = 2;
 template <typename ST>
 __global__ __launch_bounds__(NT) void layernorm_fwd_kernel(const int8_t *q, const ST *s, const float *gamma,
                                                            const float *beta, const float *mean, const float *rstd,

@@ -41,7 +41,9 @@ constexpr int EPI_LD = 36;                          // floats per staged row (32
 // EPI_QG: EPI_Q (deterministic) followed by the GELU forward of the block just requantised: two block tensors leave
 // EPI_QB: EPI_Q (stochastic: an activation gradient) followed by the GELU backward of the block just requantised against
 //         the saved forward input of the GELU: only the result of the GELU backward leaves
-enum Epilogue { EPI_S32 = 0, EPI_FP = 1, EPI_Q = 2, EPI_QG = 3, EPI_QB = 4 };
+// EPI_QD: EPI_Q followed by the dequantisation of the block just requantised (codes x stored scale), written as float /
+//         binary16 / bfloat16: the requantised tensor itself is never written.
+enum Epilogue { EPI_S32 = 0, EPI_FP = 1, EPI_Q = 2, EPI_QG = 3, EPI_QB = 4, EPI_QD = 5 };
 // Wave-priority schemes of the main loop (launch_gemm_cfg picks one per launch)
 enum Pace { PACE_HARDWARE = 0, PACE_EVEN = 1, PACE_ORDERED = 2 };
 
@@ -632,7 +634,7 @@ __global__ __launch_bounds__(64 * WGM * WGN, WGPC * WGM * WGN / 4) void igemm_nt
     };
     float *patch = reinterpret_cast<float *>(smem) + wave * (QB * EPI_LD);
     const int rrow = lane >> 1, rcol = (lane & 1) * 16;
-    constexpr bool QUANT = EPI == EPI_Q || EPI == EPI_QG || EPI == EPI_QB;
+    constexpr bool QUANT = EPI == EPI_Q || EPI == EPI_QG || EPI == EPI_QB || EPI == EPI_QD;
     const float biasmax = (QUANT && p.biasmax) ? p.biasmax[0] : 0.0f;
     float gelu_f0 = 0.0f;                                     // gelu(+0), evaluated on the device like every table entry
     if (EPI == EPI_QG) {
@@ -660,6 +662,32 @@ __global__ __launch_bounds__(64 * WGM * WGN, WGPC * WGM * WGN / 4) void igemm_nt
             }
     }
 
+    // 16 consecutive results of a row as float / binary16 / bfloat16 (rounded to nearest even): 64 or 32 contiguous bytes
+    auto store_fp = [&](const float (&x)[16], const size_t e0) {
+        if (p.out_dtype == JF_FP_F32) {
+            v4f *dst = reinterpret_cast<v4f *>(reinterpret_cast<float *>(p.C) + e0);
+#pragma unroll
+            for (int k = 0; k < 4; ++k) {
+                v4f t = {x[4 * k], x[4 * k + 1], x[4 * k + 2], x[4 * k + 3]};
+                dst[k] = t;
+            }
+        } else {
+            v4i lo, hi;
+            if (p.out_dtype == JF_FP_F16) {
+                half_t h[16];
+#pragma unroll
+                for (int k = 0; k < 16; ++k) h[k] = (half_t)x[k];
+                lo = *reinterpret_cast<v4i *>(&h[0]); hi = *reinterpret_cast<v4i *>(&h[8]);
+            } else {
+                __bf16 h[16];
+#pragma unroll
+                for (int k = 0; k < 16; ++k) h[k] = (__bf16)x[k];
+                lo = *reinterpret_cast<v4i *>(&h[0]); hi = *reinterpret_cast<v4i *>(&h[8]);
+            }
+            v4i *dst = reinterpret_cast<v4i *>(reinterpret_cast<unsigned char *>(p.C) + e0 * 2);   // 32 of a row's 64 bytes
+            dst[0] = lo; dst[1] = hi;
+        }
+    };
 #pragma unroll
     for (int i = 0; i < WBM; ++i)
 #pragma unroll
@@ -698,29 +726,7 @@ __global__ __launch_bounds__(64 * WGM * WGN, WGPC * WGM * WGN / 4) void igemm_nt
                     dst[k] = t;
                 }
             } else if (EPI == EPI_FP) {
-                if (p.out_dtype == JF_FP_F32) {
-                    v4f *dst = reinterpret_cast<v4f *>(reinterpret_cast<float *>(p.C) + e0);
-#pragma unroll
-                    for (int k = 0; k < 4; ++k) {
-                        v4f t = {x[4 * k], x[4 * k + 1], x[4 * k + 2], x[4 * k + 3]};
-                        dst[k] = t;
-                    }
-                } else {
-                    v4i lo, hi;
-                    if (p.out_dtype == JF_FP_F16) {
-                        half_t h[16];
-#pragma unroll
-                        for (int k = 0; k < 16; ++k) h[k] = (half_t)x[k];
-                        lo = *reinterpret_cast<v4i *>(&h[0]); hi = *reinterpret_cast<v4i *>(&h[8]);
-                    } else {
-                        __bf16 h[16];
-#pragma unroll
-                        for (int k = 0; k < 16; ++k) h[k] = (__bf16)x[k];
-                        lo = *reinterpret_cast<v4i *>(&h[0]); hi = *reinterpret_cast<v4i *>(&h[8]);
-                    }
-                    v4i *dst = reinterpret_cast<v4i *>(reinterpret_cast<unsigned char *>(p.C) + e0 * 2);   // 32 of a row's 64 bytes
-                    dst[0] = lo; dst[1] = hi;
-                }
+                store_fp(x, e0);
             } else {
                 v4i codes = {0, 0, 0, 0};
                 float scale = 0.0f;
@@ -759,8 +765,15 @@ __global__ __launch_bounds__(64 * WGM * WGN, WGPC * WGM * WGN / 4) void igemm_nt
                     scale = scale2;
                     wave_sync();                              // the table is the next block's patch
                 }
-                *reinterpret_cast<v4i *>(reinterpret_cast<int8_t *>(p.C) + e0) = codes;     // 16 of a row's 32 bytes
-                if (lane == 0) store_scale(reinterpret_cast<ST *>(p.sc), (bm / QB) * SN + bn / QB, scale);
+                if (EPI == EPI_QD) {
+                    // the block as a reader of the stored tensor would dequantise it: codes x the scale rounded to ST
+                    float y[16];
+                    unpack16(codes, (float)(ST)scale, y);
+                    store_fp(y, e0);
+                } else {
+                    *reinterpret_cast<v4i *>(reinterpret_cast<int8_t *>(p.C) + e0) = codes;     // 16 of a row's 32 bytes
+                    if (lane == 0) store_scale(reinterpret_cast<ST *>(p.sc), (bm / QB) * SN + bn / QB, scale);
+                }
                 if (EPI == EPI_QG) {
                     // GELU of the block as a reader of the stored tensor would see it (codes x the scale rounded to ST),
                     // with the wave's patch (free again) as the code tables
@@ -1151,6 +1164,28 @@ int jf_igemm_block_q(const int8_t *A, const int8_t *B, const void *sa, const voi
         a.phase_capacity = phase_buffer_capacity.load(std::memory_order_acquire);
     }
     return scale_dtype == JF_SCALE_F16 ? launch_gemm<EPI_Q, half_t>(a, st, kn) : launch_gemm<EPI_Q, float>(a, st, kn);
+}
+
+int jf_igemm_block_q_dequant(const int8_t *A, const int8_t *B, const void *sa, const void *sb, const float *bias,
+                             const float *biasmax, void *out, int M, int N, int K, int b_layout, int scale_dtype,
+                             int sa_layout, int sb_layout, int out_dtype, int rounding, uint64_t seed, uint64_t offset,
+                             jf_stream_t stream)
+{
+    int rc = check_gemm_common(A, B, out, M, N, K, b_layout);
+    if (rc) return rc;
+    if (!sa || !sb) return JF_ERR_NULL;
+    if ((scale_dtype != JF_SCALE_F16 && scale_dtype != JF_SCALE_F32) ||
+        (rounding != JF_ROUND_NEAREST && rounding != JF_ROUND_STOCHASTIC) ||
+        (out_dtype != JF_FP_F16 && out_dtype != JF_FP_F32 && out_dtype != JF_FP_BF16)) return JF_ERR_ENUM;
+    if (!scale_ptr_ok(sa, scale_dtype) || !scale_ptr_ok(sb, scale_dtype)) return JF_ERR_ALIGN;
+    const bool kn = b_layout == JF_B_KN;
+    GemmArgs a = {};
+    a.A = A; a.B = B; a.sa = sa; a.sb = sb; a.C = out; a.bias = bias; a.biasmax = biasmax; a.out_dtype = out_dtype;
+    a.M = M; a.N = N; a.K = K; a.lda = K; a.ldb = kn ? N : K; a.rounding = rounding; a.seed = seed; a.offset = offset;
+    if (!scale_strides(sa_layout, K, M / QB, a.sa_ks, a.sa_is) || !scale_strides(sb_layout, K, N / QB, a.sb_ks, a.sb_is))
+        return JF_ERR_ENUM;
+    hipStream_t st = (hipStream_t)stream;
+    return scale_dtype == JF_SCALE_F16 ? launch_gemm<EPI_QD, half_t>(a, st, kn) : launch_gemm<EPI_QD, float>(a, st, kn);
 }
 
 int jf_igemm_phase_record(unsigned long long *phases, int capacity_workgroups)

@@ -29,6 +29,7 @@ EXPORTS = [
     "jf_igemm_splitk_plan", "jf_igemm_block_fp_workspace_bytes", "jf_igemm_block_q_gelu", "jf_igemm_block_fp_noalloc", "jf_igemm_block_q_gelu_bwd",
     "jf_igemm_block_q", "jf_quantize", "jf_dequantize", "jf_transpose_s8", "jf_rowstats", "jf_layernorm_fwd",
     "jf_layernorm_bwd_workspace_bytes", "jf_layernorm_bwd", "jf_gelu_fwd", "jf_gelu_bwd", "jf_add", "jf_calibrate", "jf_wall_clock_khz", "jf_igemm_phase_record", "jf_rowstats_finish",
+    "jf_igemm_block_q_dequant",
 ]
 
 _lib = None
@@ -51,6 +52,7 @@ def lib():
         L.jf_igemm_block_fp.argtypes = [_p, _p, _p, _p, _p, _i, _i, _i, _i, _i, _i, _i, _i, _i, _i, _p, _sz, _p]
         L.jf_igemm_block_fp_noalloc.argtypes = [_p, _p, _p, _p, _p, _i, _i, _i, _i, _i, _i, _i, _i, _i, _i, _p]
         L.jf_igemm_block_q_gelu_bwd.argtypes = [_p, _p, _p, _p, _p, _p, _p, _p, _i, _i, _i, _i, _i, _i, _i, _u64, _u64, _i, _u64, _u64, _p]
+        L.jf_igemm_block_q_dequant.argtypes = [_p, _p, _p, _p, _p, _p, _p, _i, _i, _i, _i, _i, _i, _i, _i, _i, _u64, _u64, _p]
         L.jf_igemm_block_q_gelu.argtypes = [_p, _p, _p, _p, _p, _p, _p, _p, _p, _p, _i, _i, _i, _i, _i, _i, _i, _f, _p]
         L.jf_igemm_splitk_plan.argtypes = [_i, _i, _i, _i, C.POINTER(C.c_int), C.POINTER(C.c_int)]
         L.jf_igemm_block_fp_workspace_bytes.argtypes = [_i, _i, _i, _i, _i]
@@ -309,6 +311,31 @@ def igemm_block_q(A, B, sa, sb, b_layout=B_KN, bias=None, biasmax=None, rounding
     check(lib().jf_igemm_block_q(_ptr(A), _ptr(B), _ptr(sa), _ptr(sb), _ptr(bias), _ptr(biasmax), _ptr(out), _ptr(sc),
                                  M, N, K, b_layout, code, la, lb, rounding, seed, offset, _ptr(ws), nb, _stream()))
     return out, sc
+
+
+def igemm_block_q_dequant(A, B, sa, sb, b_layout=B_KN, out_dtype=None, bias=None, biasmax=None, rounding=ROUND_NEAREST,
+                          seed=None, offset=None):
+    """dequantize(*igemm_block_q(...), out_dtype) in one kernel: the requantised block tensor is formed in the GEMM's
+    epilogue and leaves it as codes x scales (out_dtype: float16 / bfloat16 / float32, default the scales' dtype); same
+    bits as the two calls, same noise counters."""
+    M, N, K, _, _ = _gemm_operands(A, B, b_layout)
+    code, la, lb = _gemm_scales(sa, sb, M, N, K)
+    out_dtype = sa.dtype if out_dtype is None else out_dtype
+    if out_dtype not in _FP_CODE:
+        raise RuntimeError(f"out_dtype: unsupported {out_dtype}")
+    if bias is not None:
+        _need(bias, torch.float32, "bias", 1)
+        if bias.numel() != N:
+            raise RuntimeError("bias must have N elements")
+    if biasmax is not None:
+        _need(biasmax, torch.float32, "biasmax", None)
+    if rounding not in (ROUND_NEAREST, ROUND_STOCHASTIC):
+        raise RuntimeError("rounding must be ROUND_NEAREST or ROUND_STOCHASTIC")
+    seed, offset = _rng(rounding, M * N, seed, offset, A.device)
+    out = torch.empty((M, N), dtype=out_dtype, device=A.device)
+    check(lib().jf_igemm_block_q_dequant(_ptr(A), _ptr(B), _ptr(sa), _ptr(sb), _ptr(bias), _ptr(biasmax), _ptr(out), M, N, K,
+                                         b_layout, code, la, lb, _FP_CODE[out_dtype], rounding, seed, offset, _stream()))
+    return out
 
 
 # ------------------------------------------------------------------------------------------------ block ops

@@ -196,8 +196,15 @@ def test_linear_package_3d_shapes_and_values(oracle):
     assert eq(gx8.reshape(-1, Cin), wq) and eq(gsx.reshape(-1, Cin // 32), ws)
     wgw = oracle.igemm_block_fp(qgt.cpu().numpy(), qx.reshape(-1, Cin).cpu().numpy(), sg2, sx2.float().cpu().numpy(), 1, "f16")
     assert eq(gw, wgw)
+    seed2, off2 = BQC.philox_peek(0)
     gx, gw2 = int8_linear_backward(qx, sx, qg, sg, qgt, qw, sw, 32, stochastic=True, dgrad_quantize=False)
     assert gx.dtype == torch.float16 and tuple(gx.shape) == (BS, T, Cin) and torch.equal(gw2, gw)
+    # the unquantised activation gradient = codes x scales of the stochastic requantisation drawn at (seed2, off2)
+    wq2, ws2 = oracle.igemm_block_q(qg.reshape(-1, Cout).cpu().numpy(), qw.cpu().numpy(), np.ascontiguousarray(sg2.T),
+                                    sw.float().cpu().numpy(), 1, stochastic=True, seed=seed2, offset=off2, scale_dtype="f16")
+    want_gx = (wq2.astype(np.float32).reshape(BS * T // 32, 32, Cin // 32, 32)
+               * ws2.astype(np.float32)[:, None, :, None]).reshape(BS * T, Cin).astype(np.float16)
+    assert eq(gx.reshape(-1, Cin), want_gx)
     # without a materialised transpose: G8T=None, or the .t() view of the gradient handed to the extension
     _, gw3 = int8_linear_backward(qx, sx, qg, sg, None, qw, sw, 32, stochastic=True, dgrad_quantize=False)
     gw4 = BQC.igemm_output_fp_no_quantize(qg.reshape(-1, Cout).t(), qx.reshape(-1, Cin), sg.reshape(-1, Cout // 32),

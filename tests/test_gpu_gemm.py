@@ -504,6 +504,39 @@ def test_dgrad_gemm_with_fused_gelu_backward(jf, oracle, M, N, K, f16, approx):
         jf.igemm_block_q_gelu_bwd(dA, dB, dsa, dsb, dxq[:, : N // 2].contiguous(), dxs[:, : N // 64].contiguous(), approx)
 
 
+@pytest.mark.parametrize("f16", [True, False])
+@pytest.mark.parametrize("layout", [0, 1])
+@pytest.mark.parametrize("M,N,K", [(128, 256, 96), (96, 160, 224), (256, 384, 544), (32, 32, 32), (160, 1632, 64)])
+def test_gemm_with_fused_dequantisation(jf, oracle, M, N, K, layout, f16):
+    """jf_igemm_block_q_dequant returns, bit for bit, the dequantisation of what jf_igemm_block_q stores (both roundings,
+    every output type), and the oracle's requantised result times its stored scale."""
+    print(f"case q+dequant M={M} N={N} K={K} layout={layout} f16={f16}", flush=True)
+    A, Bkn, sa, sb = make_problem(M + 5 * N + K, M, N, K, f16)
+    st = np.float16 if f16 else np.float32
+    dA, dB, dsa, dsb = dev(A), dev(b_of(Bkn, layout)), dev(sa.astype(st)), dev(sb.astype(st))
+    bias = torch.linspace(-0.5, 0.5, N).cuda()
+    biasmax = bias.abs().max().reshape(1)
+    for rounding in (jf.ROUND_NEAREST, jf.ROUND_STOCHASTIC):
+        q, s = jf.igemm_block_q(dA, dB, dsa, dsb, layout, rounding=rounding, seed=21, offset=8)
+        assert q.cpu().numpy().any()
+        for odt in (torch.float16, torch.bfloat16, torch.float32):
+            got = jf.igemm_block_q_dequant(dA, dB, dsa, dsb, layout, out_dtype=odt, rounding=rounding, seed=21, offset=8)
+            want = jf.dequantize(q, s, out_dtype=odt)
+            assert got.dtype == odt and torch.equal(got.view(torch.int16 if odt != torch.float32 else torch.int32),
+                                                    want.view(torch.int16 if odt != torch.float32 else torch.int32))
+        wq, ws = oracle.igemm_block_q(A, Bkn, sa, sb, 1, stochastic=rounding == jf.ROUND_STOCHASTIC, seed=21, offset=8,
+                                      scale_dtype="f16" if f16 else "f32")
+        want32 = (wq.astype(np.float32).reshape(M // QB, QB, N // QB, QB) * ws.astype(np.float32)[:, None, :, None]).reshape(M, N)
+        got32 = jf.igemm_block_q_dequant(dA, dB, dsa, dsb, layout, out_dtype=torch.float32, rounding=rounding, seed=21, offset=8)
+        same(got32, want32, "dequantised result")
+    # with a bias and its maximum (deterministic forward form), default output type = the scales' type
+    qb, sbb = jf.igemm_block_q(dA, dB, dsa, dsb, layout, bias=bias, biasmax=biasmax)
+    gotb = jf.igemm_block_q_dequant(dA, dB, dsa, dsb, layout, bias=bias, biasmax=biasmax)
+    assert gotb.dtype == dsa.dtype and torch.equal(gotb, jf.dequantize(qb, sbb, out_dtype=dsa.dtype))
+    with pytest.raises(RuntimeError):
+        jf.igemm_block_q_dequant(dA, dB, dsa, dsb, layout, out_dtype=torch.float64)
+
+
 @pytest.mark.gpu
 def test_phase_recording_build_gives_the_same_bits_and_ordered_phases(jf):
     """The profiling build of the requantising GEMM (jf_igemm_phase_record) stores the same codes and scales as the
