@@ -10,6 +10,8 @@
 // Reference kernels being replaced: the Triton kernels of Jetfire/Nonlinear/*.py (cited per kernel).
 #include "jf_device.hpp"
 
+#include <atomic>
+
 namespace jf {
 
 constexpr int NT = 256;                 // threads per workgroup
@@ -417,9 +419,11 @@ __device__ __forceinline__ float colsum16_over_rows(const float (&v)[16], int la
 //   S = ((T0+T1)+(T2+T3)) + ((T4+T5)+(T6+T7));  c1 = S1 / C, c2 = S2 / C;   dx = (wdy - fma(xhat, c1, c2)) * rstd[r]
 //   dgamma[c] = sum over rows of g * xhat, dbeta[c] = sum over rows of g  (fp32, order fixed by the kernels below).
 //
-// Two launches.  layernorm_bwd_stats_kernel: one wave per (column block, group of LNB_RPW row blocks) walks down its
-// column block (the four waves of a workgroup take four adjacent column blocks, i.e. whole 128-byte lines); the lane keeps gamma and its dgamma / dbeta accumulators in registers (the cross-lane reduction over
-// the 32 rows of a block happens once per wave, not once per block) and stores the per-row block partials b1, b2.
+// Rows of up to 2048 columns take one pass over the inputs (layernorm_bwd_strip_kernel, further down).  Wider rows take
+// two launches.  layernorm_bwd_stats_kernel: one wave per (column block, group of LNB_RPW row blocks) walks down its
+// column block (the four waves of a workgroup take four adjacent column blocks, i.e. whole 128-byte lines); the lane
+// keeps gamma and its dgamma / dbeta accumulators in registers (the cross-lane reduction over the 32 rows of a block
+// happens once per wave, not once per block) and stores the per-row block partials b1, b2.
 // layernorm_bwd_dx_kernel: one workgroup per 32-row strip first adds its rows' partials (c1, c2), then computes and
 // requantises dx block by block; at its end the launch also adds the row groups' dgamma / dbeta partials.
 constexpr int LNB_RPW = 4;                 // row blocks per wave of the statistics kernel
@@ -621,6 +625,160 @@ __global__ __launch_bounds__(WAVE * LNB_DX_WAVES) void layernorm_bwd_dx_kernel(
             *reinterpret_cast<v4i *>(qdx + (size_t)row * C + cb * QB + (lane & 1) * 16) = out[I];
             if (lane == 0) store_scale(sdx, rb * SC + cb, so[I]);
         });
+    }
+}
+
+// LayerNorm backward of rows of up to LNS_WAVES * LNS_BPW column blocks (2048 columns) in ONE pass over the inputs: a
+// workgroup owns a 32-row strip and keeps the strip's codes in registers (wave w: column blocks w, w + 16, ...) from the
+// first read to the store of dx.  Phase 1 forms the per-row block partials of sum(xhat * wdy) and sum(wdy) (into LDS)
+// and, when dgamma / dbeta are wanted, the strip's column sums of g * xhat and g (to pdg / pdb [R/32][C], finished by
+// layernorm_bwd_colsum_finish_kernel); the row sums are then added in the order given above (T_j over the blocks j,
+// j + 8, ..., the tree over T_0..T_7), and phase 2 converts the codes again (cheaper than keeping 32 floats per block
+// alive), forms dx and requantises it.  Same arithmetic, bit for bit, as the two-launch form above, which stays for
+// wider rows.
+constexpr int LNS_WAVES = 16, LNS_BPW = 4;
+template <typename ST, bool WANT_DW>
+__global__ __launch_bounds__(WAVE * LNS_WAVES) void layernorm_bwd_strip_kernel(
+    const int8_t *qx, const ST *sx, const int8_t *qg, const ST *sg, const float *gamma, const float *mean,
+    const float *rstd, int R, int C, int rounding, uint64_t seed, uint64_t offset, int8_t *qdx, ST *sdx, float *pdg,
+    float *pdb)
+{
+    extern __shared__ __attribute__((aligned(16))) float lds_f[];  // gamma[C], part[2][C/32][32], T[2][8][32], c[2][32], patches
+    const int lane = threadIdx.x & 63, wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
+    const int SC = C / QB, rb = blockIdx.x;
+    float *gl = lds_f, *part = gl + C, *tj = part + 2 * SC * QB, *cs = tj + 2 * 8 * QB;
+    float *cpatch = cs + 2 * QB + wave * COLSUM_PATCH;             // (only with WANT_DW)
+    const int row = rb * QB + (lane >> 1);
+    v4i cx[LNS_BPW], cg[LNS_BPW];
+    float scx[LNS_BPW], scg[LNS_BPW];
+    static_for<0, LNS_BPW>([&](auto i_c) {
+        constexpr int I = decltype(i_c)::value;
+        const int cb = wave + I * LNS_WAVES;
+        if (cb < SC) {
+            const size_t e0 = (size_t)row * C + cb * QB + (lane & 1) * 16;
+            cx[I] = *reinterpret_cast<const v4i *>(qx + e0);
+            cg[I] = *reinterpret_cast<const v4i *>(qg + e0);
+            scx[I] = load_scale(sx, rb * SC + cb);
+            scg[I] = load_scale(sg, rb * SC + cb);
+        }
+    });
+    const float mu = mean[row], rs = rstd[row];
+    for (int c = threadIdx.x * 4; c < C; c += WAVE * LNS_WAVES * 4)
+        *reinterpret_cast<v4f *>(gl + c) = *reinterpret_cast<const v4f *>(gamma + c);
+    __syncthreads();
+    const float b = -(mu * rs);
+    // phase 1: block partials of the two row sums; column sums of the strip
+    static_for<0, LNS_BPW>([&](auto i_c) {
+        constexpr int I = decltype(i_c)::value;
+        const int cb = wave + I * LNS_WAVES;
+        if (cb >= SC) return;                                      // uniform
+        const int col = cb * QB + (lane & 1) * 16;
+        const float a = scx[I] * rs, sgk = scg[I];
+        float x[16], g[16], w[16];
+        Load16<float>::run(gl + col, w);
+        codes_to_float16(cx[I], x);
+        codes_to_float16(cg[I], g);
+        float p1 = 0.0f, p2 = 0.0f;
+#pragma unroll
+        for (int j = 0; j < 16; ++j) {
+            const float xh = __builtin_fmaf(x[j], a, b);
+            const float gj = g[j] * sgk;
+            const float wdy = w[j] * gj;
+            p1 = __builtin_fmaf(xh, wdy, p1);
+            p2 = p2 + wdy;
+            if (WANT_DW) { x[j] = gj * xh; g[j] = gj; }            // this strip's terms of dgamma / dbeta
+        }
+        // the two half blocks of a row: the same two operands in both lanes of the pair
+        p1 = p1 + __int_as_float(__builtin_amdgcn_update_dpp(0, __float_as_int(p1), 0xB1, 0xF, 0xF, false));
+        p2 = p2 + __int_as_float(__builtin_amdgcn_update_dpp(0, __float_as_int(p2), 0xB1, 0xF, 0xF, false));
+        if ((lane & 1) == 0) {
+            part[cb * QB + (lane >> 1)] = p1;
+            part[(SC + cb) * QB + (lane >> 1)] = p2;
+        }
+        if (WANT_DW) {
+            // output of lane j (j even): value index j/4 of column set (j/2)%2
+            const size_t dst = (size_t)rb * C + cb * QB + ((lane >> 1) & 1) * 16 + (lane >> 2);
+            const float tg = colsum16_over_rows(x, lane, cpatch);
+            if ((lane & 1) == 0) pdg[dst] = tg;
+            const float tb = colsum16_over_rows(g, lane, cpatch);
+            if ((lane & 1) == 0) pdb[dst] = tb;
+        }
+        __builtin_amdgcn_sched_barrier(0);                         // block by block: interleaved, their temporaries do not fit
+    });
+    __syncthreads();
+    if (threadIdx.x < 512) {
+        // threads 0..255: first sum, 256..511: second; thread (j, r) adds the blocks j, j+8, ... of row r in ascending order
+        const int t = threadIdx.x & 255, j = t >> 5, r = t & 31, which = threadIdx.x >> 8;
+        const float *src = part + (size_t)which * SC * QB + r;
+        float acc = 0.0f;
+        for (int cb = j; cb < SC; cb += 8) acc = acc + src[cb * QB];
+        tj[(which * 8 + j) * QB + r] = acc;
+    }
+    __syncthreads();
+    if (threadIdx.x < 2 * QB) {
+        // S = ((T0+T1)+(T2+T3)) + ((T4+T5)+(T6+T7)),  c = S / C
+        const float *T = tj + (threadIdx.x >> 5) * 8 * QB + (threadIdx.x & 31);
+        const float S = ((T[0] + T[QB]) + (T[2 * QB] + T[3 * QB])) + ((T[4 * QB] + T[5 * QB]) + (T[6 * QB] + T[7 * QB]));
+        cs[threadIdx.x] = S / (float)C;
+    }
+    __syncthreads();
+    const float k1 = cs[lane >> 1], k2 = cs[QB + (lane >> 1)];
+    // phase 2: dx of the blocks still held as codes
+    static_for<0, LNS_BPW>([&](auto i_c) {
+        constexpr int I = decltype(i_c)::value;
+        const int cb = wave + I * LNS_WAVES;
+        if (cb >= SC) return;                                      // uniform
+        const int col = cb * QB + (lane & 1) * 16;
+        const size_t e0 = (size_t)row * C + col;
+        const float a = scx[I] * rs, sgk = scg[I];
+        float x[16], g[16], w[16];
+        Load16<float>::run(gl + col, w);
+        // (opaque copies: otherwise the optimiser keeps phase 1's 32 converted values per block alive across the barriers,
+        // in registers this kernel does not have)
+        v4i kx = cx[I], kg = cg[I];
+        asm volatile("" : "+v"(kx), "+v"(kg));
+        codes_to_float16(kx, x);
+        codes_to_float16(kg, g);
+#pragma unroll
+        for (int jj = 0; jj < 16; ++jj) {
+            const float xh = __builtin_fmaf(x[jj], a, b);
+            const float wdy = w[jj] * (g[jj] * sgk);
+            x[jj] = (wdy - __builtin_fmaf(xh, k1, k2)) * rs;
+        }
+        float so;
+        const v4i out = quantize16(x, 0.0f, rounding, seed, offset, e0, &so);
+        *reinterpret_cast<v4i *>(qdx + e0) = out;
+        if (lane == 0) store_scale(sdx, rb * SC + cb, so);
+        __builtin_amdgcn_sched_barrier(0);
+    });
+}
+
+// dgamma / dbeta from the per-strip column sums (pdg, pdb: [strips][C]).  Workgroup (32 columns, which array) of 1024
+// threads; thread (g, column) adds the strips g, g+32, ... in ascending order (8 independent loads at a time: one round
+// trip for 256 strips), then thread (0, column) adds the 32 partial sums in ascending order.
+__global__ __launch_bounds__(1024) void layernorm_bwd_colsum_finish_kernel(const float *pdg, const float *pdb, int strips,
+                                                                           int C, float *dgamma, float *dbeta)
+{
+    __shared__ float red[32][QB + 1];
+    const float *src = blockIdx.y ? pdb : pdg;
+    float *dst = blockIdx.y ? dbeta : dgamma;
+    if (!dst) return;                                              // uniform
+    const int k = threadIdx.x & 31, c = blockIdx.x * QB + k, g = threadIdx.x >> 5;
+    float acc = 0.0f;
+    for (int s0 = g; s0 < strips; s0 += 256) {
+        float v[8];
+#pragma unroll
+        for (int i = 0; i < 8; ++i) { const int s = s0 + 32 * i; v[i] = s < strips ? src[(size_t)s * C + c] : 0.0f; }
+#pragma unroll
+        for (int i = 0; i < 8; ++i) acc = acc + v[i];
+    }
+    red[g][k] = acc;
+    __syncthreads();
+    if (g == 0) {
+        float t = red[0][k];
+#pragma unroll
+        for (int i = 1; i < 32; ++i) t = t + red[i][k];
+        dst[c] = t;
     }
 }
 
@@ -838,6 +996,33 @@ int jf_layernorm_bwd(const int8_t *qx, const void *sx, const int8_t *qg, const v
     hipStream_t st = (hipStream_t)stream;
     const bool want_dw = dgamma || dbeta;
     const int SC = C / QB, groups = lnb_groups(R);
+    if (SC <= LNS_WAVES * LNS_BPW) {
+        // rows of up to 2048 columns: one pass over the inputs, the strip's codes held in registers
+        float *sdg = (float *)workspace, *sdb = sdg + (size_t)(R / QB) * C;      // [R/32][C] each: fits the size above
+        const size_t lds = ((size_t)C + 2 * SC * QB + 2 * 8 * QB + 2 * QB + (want_dw ? LNS_WAVES * COLSUM_PATCH : 0)) * sizeof(float);
+        int dev = 0;
+        if (hipGetDevice(&dev) != hipSuccess || dev < 0 || dev >= 64) return JF_ERR_DEVICE;
+#define JF_LNS(ST, DW)                                                                                                 \
+        do {                                                                                                           \
+            auto kern = layernorm_bwd_strip_kernel<ST, DW>;                                                            \
+            static std::atomic<bool> opted_in[64] = {};           /* more than 64 KiB of LDS: once per device */        \
+            if (lds > 64 * 1024 && !opted_in[dev].load(std::memory_order_acquire)) {                                   \
+                hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void *>(kern),                               \
+                                                   hipFuncAttributeMaxDynamicSharedMemorySize, 160 * 1024);            \
+                if (e != hipSuccess) return (int)e;                                                                    \
+                opted_in[dev].store(true, std::memory_order_release);                                                  \
+            }                                                                                                          \
+            hipLaunchKernelGGL(kern, dim3(R / QB), dim3(WAVE * LNS_WAVES), lds, st, qx, (const ST *)sx, qg,            \
+                               (const ST *)sg, gamma, mean, rstd, R, C, rounding, seed, offset, qdx, (ST *)sdx,        \
+                               DW ? sdg : nullptr, DW ? sdb : nullptr);                                                \
+        } while (0)
+        if (scale_dtype == JF_SCALE_F16) { if (want_dw) JF_LNS(half_t, true); else JF_LNS(half_t, false); }
+        else { if (want_dw) JF_LNS(float, true); else JF_LNS(float, false); }
+#undef JF_LNS
+        if (want_dw)
+            hipLaunchKernelGGL(layernorm_bwd_colsum_finish_kernel, dim3(SC, 2), dim3(1024), 0, st, sdg, sdb, R / QB, C, dgamma, dbeta);
+        return (int)hipGetLastError();
+    }
     const size_t smem = ((size_t)C + 2 * QB + 16 * QB) * sizeof(float);   // gamma, c1, c2 and the row-sum partials in LDS
     if (smem > LDS_VECTOR_LIMIT) return JF_ERR_SHAPE;
     float *part1 = (float *)workspace, *part2 = part1 + (size_t)R * SC;
