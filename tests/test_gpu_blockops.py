@@ -236,6 +236,15 @@ def _random_block_shapes(n, seed):
         yield int(rng.integers(1, 11)) * 32, int(rng.integers(1, 130)) * 32, bool(rng.integers(0, 2)), int(rng.integers(0, 2))
 
 
+@pytest.mark.parametrize("R,C", [(64, 2048), (64, 2080), (32, 1632), (96, 512), (32, 544)])
+def test_layernorm_backward_single_pass_and_two_launch_forms(jf, oracle, R, C):
+    """Rows of up to 64 column blocks (2048 columns) take the single-pass strip kernel, wider rows the two-launch form:
+    the widest row of the first, the narrowest of the second, rows whose block count is not a multiple of the 16 waves
+    of a strip, and rows of exactly / just over 16 blocks."""
+    test_rowstats_layernorm(jf, oracle, R, C, False)
+    test_rowstats_layernorm(jf, oracle, R, C, True)
+
+
 @pytest.mark.parametrize("R,C,f16,approx", list(_random_block_shapes(12, 7)))
 def test_random_shapes(jf, oracle, R, C, f16, approx):
     """The GELU and LayerNorm checks above on random tensor shapes (up to 320 x 4128: rows of more column blocks than a
