@@ -230,7 +230,7 @@ __global__ __launch_bounds__(NT) void gelu_fwd_kernel(const int8_t *q, const ST 
                                                       int8_t *qy, ST *sy)
 {
     __shared__ __attribute__((aligned(16))) float table[WPB][256];
-    __shared__ __attribute__((aligned(16))) int qtable[WPB][256];
+    __shared__ __attribute__((aligned(16))) int qtable[WPB][64];      // 256 one-byte entries per wave
     float *tab = table[threadIdx.x >> 6];
     int *qtab = qtable[threadIdx.x >> 6];
     const int lane = threadIdx.x & 63, SC = C / QB, RB = R / QB, stride = gridDim.x * WPB;

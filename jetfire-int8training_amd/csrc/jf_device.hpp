@@ -393,7 +393,7 @@ __device__ __forceinline__ void table_done()
 }
 
 // GELU forward of one block: 16 codes per lane (lane l: row l/2, columns 16*(l%2) .. +15) with scale sc -> packed codes
-// of the requantised result, *scale_out = its scale (all lanes).  tab / qtab: 256 floats / 256 ints of LDS private to the
+// of the requantised result, *scale_out = its scale (all lanes).  tab / qtab: 256 floats / 64 ints (256 bytes) of LDS private to the
 // wave.  f0 = gelu(+0), evaluated by the caller once (the same for every block).  (gelu_fwd.py:34-126)
 template <int APPROX>
 __device__ __forceinline__ v4i gelu_fwd_block(v4i c, float sc, float f0, float amax_eps, float *tab, int *qtab, int lane,
@@ -417,17 +417,19 @@ __device__ __forceinline__ v4i gelu_fwd_block(v4i c, float sc, float f0, float a
         const float t[4] = {t4.x, t4.y, t4.z, t4.w};
         float y[4];
         d.divn<4>(t, y);
-        v4i q4 = {clamp127(__builtin_rintf(y[0])), clamp127(__builtin_rintf(y[1])), clamp127(__builtin_rintf(y[2])),
-                  clamp127(__builtin_rintf(y[3]))};
-        *reinterpret_cast<v4i *>(qtab + 4 * lane) = q4;
+        // the requantised table is a BYTE table (entry e at byte e: lane l writes the word of its four entries): 64 words
+        // instead of 256, so twice as many of a gather's lanes meet in the same word (a broadcast, not a bank conflict)
+        qtab[lane] = (int)pack4(clamp127(__builtin_rintf(y[0])), clamp127(__builtin_rintf(y[1])),
+                                clamp127(__builtin_rintf(y[2])), clamp127(__builtin_rintf(y[3])));
         __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
         __builtin_amdgcn_wave_barrier();
         __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
+        const unsigned char *q8 = reinterpret_cast<const unsigned char *>(qtab);
         const uint32_t wd[4] = {(uint32_t)c.x, (uint32_t)c.y, (uint32_t)c.z, (uint32_t)c.w};
         int o[4];
 #pragma unroll
         for (int i = 0; i < 4; ++i)
-            o[i] = (int)pack4(qtab[wd[i] & 0xFF], qtab[(wd[i] >> 8) & 0xFF], qtab[(wd[i] >> 16) & 0xFF], qtab[wd[i] >> 24]);
+            o[i] = (int)pack4(q8[wd[i] & 0xFF], q8[(wd[i] >> 8) & 0xFF], q8[(wd[i] >> 16) & 0xFF], q8[wd[i] >> 24]);
         codes = v4i{o[0], o[1], o[2], o[3]};
     }
     table_done();
