@@ -219,16 +219,17 @@ int jf_gelu_bwd(const int8_t *qx, const void *sx, const int8_t *qg, const void *
                 int8_t *qy, void *sy, jf_stream_t stream);
 
 /* y1_f32 = x1 + q2*s2, (q, s) = block quantisation of y1; optional per-row, per-32-column partial
- * sums of y1 and y1^2 (rowsum, rowsq: [R, C/32] fp32, may be NULL).
+ * sums of y1 and y1^2 (rowsum, rowsq: [C/32, R] fp32 -- part-major, so that a block's 32 rows are one contiguous store;
+ * may be NULL).
  * Replaces int8_add_Ifp_Ig16_Ofp_Og (Jetfire/Nonlinear/add.py:164-211) and
  * int8_add_Ifp_Ig16_Ofp_Og_MeanVar (Jetfire/Nonlinear/add_mean_var.py:179-230). */
 int jf_add(const void *x1, int x1_dtype, const int8_t *q2, const void *s2, int R, int C,
            int scale_dtype, int rounding, uint64_t seed, uint64_t offset,
            float *y1, int8_t *q, void *s, float *rowsum, float *rowsq, jf_stream_t stream);
 
-/* mean[r] = (sum of rowsum[r, 0..parts-1], ascending) / C;  rstd[r] = 1 / sqrt((sum of rowsq[r, :]) / C - mean[r]^2)
+/* mean[r] = (sum of rowsum[0..parts-1, r], ascending) / C;  rstd[r] = 1 / sqrt((sum of rowsq[:, r]) / C - mean[r]^2)
  * (no epsilon): the finishing step of int8_add_Ifp_Ig16_Ofp_Og_MeanVar (Jetfire/Nonlinear/add_mean_var.py:219-221), which
- * the reference computes with torch operators on the kernel's partial sums.  rowsum, rowsq: [R, parts] fp32 as written by
+ * the reference computes with torch operators on the kernel's partial sums.  rowsum, rowsq: [parts, R] fp32 as written by
  * jf_add. */
 int jf_rowstats_finish(const float *rowsum, const float *rowsq, int R, int parts, int C, float *mean, float *rstd,
                        jf_stream_t stream);

@@ -783,11 +783,19 @@ __global__ __launch_bounds__(1024) void layernorm_bwd_colsum_finish_kernel(const
 }
 
 // add.py:29-162 / add_mean_var.py:28-177
+// The fp32 sum leaves through a wave-private LDS patch: in the layout the arithmetic uses (lane l: row l/2, 16 columns)
+// a store instruction would write 64 separate 16-byte pieces; read back as "lane l: row 8i + l/8, columns 4*(l%8) .. +3"
+// each of the four store instructions writes 8 whole 128-byte rows of the block (measured on an fp32 copy of 8192x1600:
+// 17.0 against 22.9 us; the mapping of the loads makes no difference).
+// rowsum / rowsq: [C/32][R] (a wave stores the 32 consecutive rows of its block).
+constexpr int ADD_PITCH = QB + 4;                  // floats per patch row (16-byte aligned rows, rotated over the banks)
 template <typename T, typename ST>
 __global__ __launch_bounds__(NT) void add_kernel(const T *x1, const int8_t *q2, const ST *s2, int R, int C,
                                                  int rounding, uint64_t seed, uint64_t offset, float *y1, int8_t *q,
                                                  ST *s, float *rowsum, float *rowsq)
 {
+    __shared__ __attribute__((aligned(16))) float ypatch_all[WPB][QB * ADD_PITCH];
+    float *ypatch = ypatch_all[threadIdx.x >> 6];
     JF_FOR_EACH_BLOCK(R, C)
     {
         BlockPos pos(blk, SC, C, lane);
@@ -796,15 +804,29 @@ __global__ __launch_bounds__(NT) void add_kernel(const T *x1, const int8_t *q2, 
         unpack16(*reinterpret_cast<const v4i *>(q2 + pos.e0), load_scale(s2, pos.rb * SC + pos.cb), b);
 #pragma unroll
         for (int k = 0; k < 16; ++k) a[k] = a[k] + b[k];
-        store16_f32(y1 + pos.e0, a);
+        {
+            float *w = ypatch + (lane >> 1) * ADD_PITCH + (lane & 1) * 16;
+#pragma unroll
+            for (int k = 0; k < 4; ++k) *reinterpret_cast<v4f *>(w + 4 * k) = v4f{a[4 * k], a[4 * k + 1], a[4 * k + 2], a[4 * k + 3]};
+            __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
+            __builtin_amdgcn_wave_barrier();
+            __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
+            float *dst = y1 + (size_t)(pos.rb * QB + (lane >> 3)) * C + pos.cb * QB + (lane & 7) * 4;
+#pragma unroll
+            for (int i = 0; i < 4; ++i)
+                *reinterpret_cast<v4f *>(dst + (size_t)(8 * i) * C) =
+                    *reinterpret_cast<const v4f *>(ypatch + (8 * i + (lane >> 3)) * ADD_PITCH + (lane & 7) * 4);
+            __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
+            __builtin_amdgcn_wave_barrier();                       // the patch may be rewritten
+        }
         if (rowsum) {
             float t1 = 0.0f, t2 = 0.0f;
 #pragma unroll
             for (int k = 0; k < 16; ++k) { t1 = t1 + a[k]; t2 = __builtin_fmaf(a[k], a[k], t2); }
             const float o1 = __shfl_xor(t1, 1, WAVE), o2 = __shfl_xor(t2, 1, WAVE);
             if ((lane & 1) == 0) {
-                rowsum[(size_t)pos.row * SC + pos.cb] = t1 + o1;     // columns 0..15 partial + 16..31 partial
-                rowsq[(size_t)pos.row * SC + pos.cb] = t2 + o2;
+                rowsum[(size_t)pos.cb * R + pos.row] = t1 + o1;     // columns 0..15 partial + 16..31 partial
+                rowsq[(size_t)pos.cb * R + pos.row] = t2 + o2;
             }
         }
         float scale;
@@ -851,28 +873,31 @@ static inline bool rounding_ok(int r) { return r >= JF_ROUND_NEAREST && r <= JF_
 
 using namespace jf;
 
-// mean and 1/sqrt(variance) of every row from its per-32-column partial sums (rowsum, rowsq: [R, parts], what add_kernel
+// mean and 1/sqrt(variance) of every row from its per-32-column partial sums (rowsum, rowsq: [parts][R], what add_kernel
 // leaves): the partials are added in ascending order, var = E[y^2] - mean^2, no epsilon (add_mean_var.py:219-221).
 constexpr int RSF_ROWS = 32;                       // rows per workgroup
 __global__ __launch_bounds__(256) void rowstats_finish_kernel(const float *rowsum, const float *rowsq, int R, int parts,
                                                               float n, float *mean, float *rstd)
 {
-    // the partial sums of RSF_ROWS consecutive rows are one contiguous run of each array: fetched by all threads, then
-    // one thread per row (and array) adds its row's partials in ascending order from LDS
-    extern __shared__ float rsf_lds[];                                // [2][RSF_ROWS * parts]
+    // the partial sums of RSF_ROWS consecutive rows are fetched by all threads (128 contiguous bytes per part and array),
+    // then one thread per row (and array) adds its row's partials in ascending order from LDS
+    extern __shared__ float rsf_lds[];                                // [2][parts][RSF_ROWS]
     const int r0 = blockIdx.x * RSF_ROWS;
     const int rows = (R - r0) < RSF_ROWS ? (R - r0) : RSF_ROWS;
-    const int count = rows * parts;
+    const int count = parts * RSF_ROWS;
     for (int i = threadIdx.x; i < count; i += 256) {
-        rsf_lds[i] = rowsum[(size_t)r0 * parts + i];
-        rsf_lds[RSF_ROWS * parts + i] = rowsq[(size_t)r0 * parts + i];
+        const int j = i / RSF_ROWS, r = i % RSF_ROWS;
+        if (r < rows) {
+            rsf_lds[i] = rowsum[(size_t)j * R + r0 + r];
+            rsf_lds[count + i] = rowsq[(size_t)j * R + r0 + r];
+        }
     }
     __syncthreads();
     const int row = threadIdx.x & (RSF_ROWS - 1), which = threadIdx.x / RSF_ROWS;     // which: 0 = sums, 1 = squares
     float acc = 0.0f;
     if (which < 2 && row < rows) {
-        const float *p = rsf_lds + which * (RSF_ROWS * parts) + row * parts;
-        for (int j = 0; j < parts; ++j) acc = acc + p[j];
+        const float *p = rsf_lds + which * count + row;
+        for (int j = 0; j < parts; ++j) acc = acc + p[j * RSF_ROWS];
     }
     __syncthreads();
     if (which == 1 && row < rows) rsf_lds[row] = acc;                 // hand the sum of squares to the row's other thread

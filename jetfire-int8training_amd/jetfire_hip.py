@@ -466,21 +466,21 @@ def add(x1, q2, s2, rounding=ROUND_TRUNC, with_stats=False, seed=None, offset=No
     y1 = torch.empty((R, Cc), dtype=torch.float32, device=x1.device)
     q = torch.empty_like(q2)
     s = torch.empty_like(s2)
-    rs = torch.empty((R, Cc // QB), dtype=torch.float32, device=x1.device) if with_stats else None
-    rq = torch.empty((R, Cc // QB), dtype=torch.float32, device=x1.device) if with_stats else None
+    rs = torch.empty((Cc // QB, R), dtype=torch.float32, device=x1.device) if with_stats else None   # part-major
+    rq = torch.empty((Cc // QB, R), dtype=torch.float32, device=x1.device) if with_stats else None
     check(lib().jf_add(_ptr(x1), _FP_CODE[x1.dtype], _ptr(q2), _ptr(s2), R, Cc, code, rounding, seed, offset,
                        _ptr(y1), _ptr(q), _ptr(s), _ptr(rs), _ptr(rq), _stream()))
     return (y1, q, s, rs, rq) if with_stats else (y1, q, s)
 
 
 def rowstats_finish(rowsum, rowsq, n_cols):
-    """(mean, rstd) per row from add(..., with_stats=True)'s partial sums [R, parts]: partials added in ascending order,
+    """(mean, rstd) per row from add(..., with_stats=True)'s partial sums [parts, R]: partials added in ascending order,
     var = E[y^2] - mean^2, rstd = 1/sqrt(var), no epsilon."""
     _need(rowsum, torch.float32, "rowsum", 2)
     _need(rowsq, torch.float32, "rowsq", 2)
     if rowsum.shape != rowsq.shape:
         raise RuntimeError("rowsum and rowsq must have the same shape")
-    R, parts = rowsum.shape
+    parts, R = rowsum.shape
     mean = torch.empty(R, dtype=torch.float32, device=rowsum.device)
     rstd = torch.empty(R, dtype=torch.float32, device=rowsum.device)
     check(lib().jf_rowstats_finish(_ptr(rowsum), _ptr(rowsq), R, parts, int(n_cols), _ptr(mean), _ptr(rstd), _stream()))

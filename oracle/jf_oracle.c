@@ -588,7 +588,7 @@ void jfo_layernorm_bwd(const int8_t *qx, const float *sx, const int8_t *qg, cons
 /*
  * Residual add: y1 = x1 + q2*s2 (fp32 out) and its block quantisation.
  * add.py:29-162 (stochastic allowed) / add_mean_var.py:28-177 (+ per-row partial
- * sums of y1 and y1^2 per 32-column block: two 16-column add / fmaf chains, added).
+ * sums of y1 and y1^2 per 32-column block, stored [C/32][R]: two 16-column add / fmaf chains, added).
  * truncate=1 reproduces the reference's `.to(int8)` without llrint (add.py:139).
  */
 void jfo_add(const float *x1, const int8_t *q2, const float *s2, int R, int C,
@@ -608,8 +608,8 @@ void jfo_add(const float *x1, const int8_t *q2, const float *s2, int R, int C,
                 y1[o + (size_t)i * C + j] = v;
                 a[j / 16] = a[j / 16] + v; b[j / 16] = fmaf(v, v, b[j / 16]);
             }
-            if (rowsum) rowsum[(size_t)(rb * QB + i) * SC + cb] = a[0] + a[1];
-            if (rowsq) rowsq[(size_t)(rb * QB + i) * SC + cb] = b[0] + b[1];
+            if (rowsum) rowsum[(size_t)cb * R + rb * QB + i] = a[0] + a[1];      /* [C/32][R] */
+            if (rowsq) rowsq[(size_t)cb * R + rb * QB + i] = b[0] + b[1];
         }
         quantize_block(tmp, QB, q + o, C, &s[rb * SC + cb], stochastic, seed, offset, (uint64_t)o, (uint64_t)C, 0.0f, truncate);
     }

@@ -359,8 +359,8 @@ def add(x1, q2, s2, stochastic=False, seed=0, offset=0, truncate=True, with_stat
     y1 = np.empty_like(x1)
     q = np.empty_like(q2)
     s = np.empty_like(s2)
-    rs = np.empty((R, C_ // QB), np.float32) if with_stats else None
-    rq = np.empty((R, C_ // QB), np.float32) if with_stats else None
+    rs = np.empty((C_ // QB, R), np.float32) if with_stats else None       # part-major
+    rq = np.empty((C_ // QB, R), np.float32) if with_stats else None
     lib().jfo_add(_ptr(x1), _ptr(q2), _ptr(s2), R, C_, int(stochastic), seed, offset, int(truncate),
                   _ptr(y1), _ptr(q), _ptr(s), _ptr(rs), _ptr(rq))
     if with_stats:

@@ -200,7 +200,7 @@ def test_add(jf, oracle, dtype, mode):
     mean, rstd = jf.rowstats_finish(rs, rq, C)
     a, b = np.zeros(R, np.float32), np.zeros(R, np.float32)
     for j in range(C // 32):
-        a, b = a + wrs[:, j], b + wrq[:, j]
+        a, b = a + wrs[j], b + wrq[j]
     m = a / np.float32(C)
     var = b / np.float32(C) - m * m
     same(mean, m, "mean")

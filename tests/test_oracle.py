@@ -463,8 +463,10 @@ def test_add_closed_form(oracle):
     _, qn, _ = oracle.add(x1, q2, s2, truncate=False)
     assert np.array_equal(qn, np.rint(want / expand_scales(sw)).astype(np.int8))
     w64 = want.astype(np.float64)
-    assert np.allclose(rs.sum(axis=1), w64.sum(axis=1), rtol=1e-5, atol=1e-4)
-    assert np.allclose(rq.sum(axis=1), (w64 ** 2).sum(axis=1), rtol=1e-5)
-    mean = rs.sum(axis=1) / Cc
-    var = rq.sum(axis=1) / Cc - mean ** 2
+    assert rs.shape == (Cc // 32, R)                              # part-major
+    assert np.allclose(rs.sum(axis=0), w64.sum(axis=1), rtol=1e-5, atol=1e-4)
+    assert np.allclose(rq.sum(axis=0), (w64 ** 2).sum(axis=1), rtol=1e-5)
+    assert np.allclose(rs[1], w64[:, 32:64].sum(axis=1), rtol=1e-5, atol=1e-4)
+    mean = rs.sum(axis=0) / Cc
+    var = rq.sum(axis=0) / Cc - mean ** 2
     assert np.allclose(var, w64.var(axis=1), rtol=1e-4)
