@@ -187,43 +187,59 @@ def deep_k_weight_gradients(jf, torch):
 
 
 def recipe_block(torch):
-    """One GPT-2 XL transformer block (1600 wide, 25 heads) forward + backward on 8 x 1024 tokens: the INT8 data-flow
+    """GPT-2 XL transformer blocks (1600 wide, 25 heads) forward + backward on 8 x 1024 tokens: the INT8 data-flow
     recipe (Jetfire/recipe.py: every linear layer, LayerNorm, GELU and residual add on INT8 block tensors, attention
-    itself in fp16 through torch) next to the same block in plain torch bf16."""
+    itself in fp16 through torch) next to the same blocks in plain torch bf16.  Measured for a stack of one block (which
+    includes the stack's own begin / end: quantising the input, its row statistics, quantising the output gradient) and
+    of three; the difference, halved, is what a block costs inside a stack.  Parameter gradients are reset to None before
+    every step, as an optimizer's zero_grad() does."""
     import torch.nn.functional as F
     sys.path.insert(0, os.path.join(PKG, "Jetfire"))
     from recipe import QStack
     torch.manual_seed(0)
     B, T, C, H = 8, 1024, 1600, 25
-    model = QStack(1, C, H).cuda()
-    blk = model.blocks[0]
     x = torch.randn(B, T, C, device="cuda", requires_grad=True)
     w = torch.randn(B, T, C, device="cuda")
+    xr, wr = x.detach().to(torch.bfloat16).requires_grad_(True), w.to(torch.bfloat16)
 
-    def ref_block(xr, dt):
-        h = F.layer_norm(xr, (C,), blk.ln_1.to(dt), None, 1e-5)
-        qkv = h @ blk.w_qkv.to(dt).t()
-        q, k, v = (t.view(B, T, H, C // H).transpose(1, 2) for t in qkv.split(C, dim=2))
-        y = F.scaled_dot_product_attention(q, k, v, is_causal=True).transpose(1, 2).contiguous().view(B, T, C)
-        xr = xr + y @ blk.w_attn_proj.to(dt).t()
-        h = F.layer_norm(xr, (C,), blk.ln_2.to(dt), None, 1e-5)
-        return xr + F.gelu(h @ blk.w_fc.to(dt).t()) @ blk.w_mlp_proj.to(dt).t()
-
-    def t(fn, n=10):
-        for _ in range(3):
+    def t(fn, params, n=10):
+        def step():
+            for p in params:
+                p.grad = None
             fn()
+        for _ in range(3):
+            step()
         torch.cuda.synchronize()
         e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
         e0.record()
         for _ in range(n):
-            fn()
+            step()
         e1.record()
         torch.cuda.synchronize()
-        return round(e0.elapsed_time(e1) / n, 3)
+        return e0.elapsed_time(e1) / n
 
-    xr, wr = x.detach().to(torch.bfloat16).requires_grad_(True), w.to(torch.bfloat16)
-    return {"tokens": B * T, "int8_recipe_ms": t(lambda: model(x).backward(w)),
-            "torch_bf16_ms": t(lambda: ref_block(xr, torch.bfloat16).backward(wr))}
+    out = {}
+    for layers in (1, 3):
+        model = QStack(layers, C, H).cuda()
+
+        def ref_stack(h0, dt):
+            for blk in model.blocks:
+                h = F.layer_norm(h0, (C,), blk.ln_1.to(dt), None, 1e-5)
+                qkv = h @ blk.w_qkv.to(dt).t()
+                q, k, v = (u.view(B, T, H, C // H).transpose(1, 2) for u in qkv.split(C, dim=2))
+                y = F.scaled_dot_product_attention(q, k, v, is_causal=True).transpose(1, 2).contiguous().view(B, T, C)
+                h0 = h0 + y @ blk.w_attn_proj.to(dt).t()
+                h = F.layer_norm(h0, (C,), blk.ln_2.to(dt), None, 1e-5)
+                h0 = h0 + F.gelu(h @ blk.w_fc.to(dt).t()) @ blk.w_mlp_proj.to(dt).t()
+            return h0
+        params = list(model.parameters())
+        out[layers] = (t(lambda: model(x).backward(w), params + [x]),
+                       t(lambda: ref_stack(xr, torch.bfloat16).backward(wr), params + [xr]))
+        del model
+    return {"tokens": B * T, "int8_recipe_ms": round(out[1][0], 3), "torch_bf16_ms": round(out[1][1], 3),
+            "stack_of_3_blocks": {"int8_recipe_ms": round(out[3][0], 3), "torch_bf16_ms": round(out[3][1], 3)},
+            "per_block_inside_a_stack": {"int8_recipe_ms": round((out[3][0] - out[1][0]) / 2, 3),
+                                         "torch_bf16_ms": round((out[3][1] - out[1][1]) / 2, 3)}}
 
 
 def nonlinear_extras(jf, torch):

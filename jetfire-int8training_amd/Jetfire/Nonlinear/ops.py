@@ -55,6 +55,23 @@ def int8_quantize(x, QB, stochastic=False, scale_dtype=torch.float16):
     return sh.fold(q), sh.fold(s)
 
 
+def int8_quantize_concat(xs, QB, stochastic=False, scale_dtype=torch.float16):
+    """int8_quantize(torch.cat(xs, dim=-1), ...) without the concatenation (no counterpart in the reference, which
+    quantises the concatenated gradient of the attention kernel's inputs, qmodel.py:112-120): every tensor of xs is
+    quantised where it lies into its columns of the result.  Same codes, scales and noise as the two-step form."""
+    _check_qb(QB)
+    sh = _Shape(xs[0])
+    flat = []
+    for x in xs:
+        if x.dim() != xs[0].dim() or x.shape[:-1] != xs[0].shape[:-1]:
+            raise RuntimeError("tensors to concatenate must agree in all but the last dimension")
+        f = x.reshape(-1, x.shape[-1])                             # a view whenever the leading dimensions can be merged
+        flat.append(f if f.stride(1) == 1 and (f.stride(0) * f.element_size()) % 16 == 0 and f.data_ptr() % 16 == 0
+                    else f.contiguous())
+    q, s = _jf.quantize_slabs(flat, _jf.ROUND_STOCHASTIC if stochastic else _jf.ROUND_NEAREST, scale_dtype)
+    return sh.fold(q), sh.fold(s)
+
+
 def int8_quantize_transpose(x, QB, stochastic=False, transpose_output_2d=False, scale_dtype=torch.float16):
     """As int8_quantize, plus the transposed codes [N, M].  Reference: quantize_transpose.py:131-171."""
     _check_qb(QB)

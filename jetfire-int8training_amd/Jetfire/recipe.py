@@ -21,7 +21,7 @@ import torch.nn.functional as F
 
 from Linear import int8_linear_backward, int8_linear_backward_gelu, int8_linear_forward, int8_linear_forward_gelu
 from Nonlinear import (int8_add_Ifp_Ig16_Ofp_Og, int8_add_Ifp_Ig16_Ofp_Og_MeanVar, int8_gelu_backward,
-                       int8_layernorm_backward, int8_layernorm_forward, int8_quantize)
+                       int8_layernorm_backward, int8_layernorm_forward, int8_quantize, int8_quantize_concat)
 
 QB = 32
 _F8 = torch.float8_e4m3fn
@@ -93,7 +93,10 @@ class StreamEnd(torch.autograd.Function):
 
 
 class AttentionIn(torch.autograd.Function):
-    """LayerNorm -> QKV projection, fp16 out for the attention kernel (qmodel.py:86-131)."""
+    """LayerNorm -> QKV projection, fp16 out for the attention kernel (qmodel.py:86-131).  Q, K and V leave as three
+    views of the projection's output, so that their gradients come back as three tensors and are quantised where they
+    lie: the concatenated gradient the reference quantises (autograd's cat behind the split of qkv, 78 MB at GPT-2 XL
+    size) is never made; codes, scales and rounding noise are those of the concatenation."""
 
     @staticmethod
     def forward(ctx, residual, qx, sx, w_qkv, ln_w, mean, rstd):
@@ -103,12 +106,13 @@ class AttentionIn(torch.autograd.Function):
         qn, sn, _ = int8_layernorm_forward(qx, sx, ln_w, mean, rstd, QB)
         qkv = int8_linear_forward(qn, sn, qw, sw, False, QB)
         ctx.save_for_backward(qx, sx, qn, sn, qw, sw, ln_w, mean, rstd)
-        return residual, qkv
+        q, k, v = qkv.split(qkv.shape[-1] // 3, dim=-1)
+        return residual, q, k, v
 
     @staticmethod
-    def backward(ctx, fpg, g):
+    def backward(ctx, fpg, gq, gk, gv):
         qx, sx, qn, sn, qw, sw, ln_w, mean, rstd = ctx.saved_tensors
-        qg, sg = int8_quantize(g.contiguous(), QB, stochastic=True)
+        qg, sg = int8_quantize_concat([gq, gk, gv], QB, stochastic=True)
         qg, sg, gw = int8_linear_backward(qn, sn, qg, sg, None, qw, sw, QB, stochastic=True, wgrad_splitk=0, wgrad_dtype=ctx.wdtype)
         qg, sg, g_ln = int8_layernorm_backward(qx, sx, qg, sg, ln_w, QB, mean, rstd, stochastic=True)
         res_g, qg, sg = int8_add_Ifp_Ig16_Ofp_Og(fpg.contiguous(), qg, sg, QB, stochastic=True)
@@ -122,6 +126,7 @@ class AttentionOut(torch.autograd.Function):
     def forward(ctx, residual, y, w_proj):
         qw, sw = weight_codes.get(w_proj)
         ctx.wdtype = w_proj.dtype
+        ctx.set_materialize_grads(False)  # mean / rstd receive no gradient: None instead of two zero-filled tensors
         qy, sy = int8_quantize(y.contiguous(), QB)
         qo, so = int8_linear_forward(qy, sy, qw, sw, True, QB)
         fp, q, s, mean, rstd = int8_add_Ifp_Ig16_Ofp_Og_MeanVar(residual.contiguous(), qo, so, QB)
@@ -145,6 +150,7 @@ class MLPResidual(torch.autograd.Function):
         qw1, sw1 = weight_codes.get(w_fc)
         qw2, sw2 = weight_codes.get(w_proj)
         ctx.wdtype = w_fc.dtype
+        ctx.set_materialize_grads(False)  # as in AttentionOut
         qn, sn, _ = int8_layernorm_forward(qx, sx, ln_w, mean, rstd, QB)
         qh, sh, qa, sa = int8_linear_forward_gelu(qn, sn, qw1, sw1, QB)      # fc and its GELU in one kernel
         qo, so = int8_linear_forward(qa, sa, qw2, sw2, True, QB)
@@ -181,8 +187,8 @@ class QBlock(nn.Module):
 
     def forward(self, x, qx, sx, mean, rstd):
         B, T, C = x.shape
-        res, qkv = AttentionIn.apply(x, qx, sx, self.w_qkv, self.ln_1, mean, rstd)
-        q, k, v = (t.view(B, T, self.n_head, C // self.n_head).transpose(1, 2) for t in qkv.split(C, dim=2))
+        res, q, k, v = AttentionIn.apply(x, qx, sx, self.w_qkv, self.ln_1, mean, rstd)
+        q, k, v = (t.view(B, T, self.n_head, C // self.n_head).transpose(1, 2) for t in (q, k, v))
         y = F.scaled_dot_product_attention(q, k, v, is_causal=True).transpose(1, 2).contiguous().view(B, T, C)
         x, qx, sx, mean, rstd = AttentionOut.apply(res, y, self.w_attn_proj)
         return MLPResidual.apply(x, qx, sx, self.w_fc, self.w_mlp_proj, self.ln_2, mean, rstd)

@@ -29,7 +29,7 @@ EXPORTS = [
     "jf_igemm_splitk_plan", "jf_igemm_block_fp_workspace_bytes", "jf_igemm_block_q_gelu", "jf_igemm_block_fp_noalloc", "jf_igemm_block_q_gelu_bwd",
     "jf_igemm_block_q", "jf_quantize", "jf_dequantize", "jf_transpose_s8", "jf_rowstats", "jf_layernorm_fwd",
     "jf_layernorm_bwd_workspace_bytes", "jf_layernorm_bwd", "jf_gelu_fwd", "jf_gelu_bwd", "jf_add", "jf_calibrate", "jf_wall_clock_khz", "jf_igemm_phase_record", "jf_rowstats_finish",
-    "jf_igemm_block_q_dequant",
+    "jf_igemm_block_q_dequant", "jf_quantize_slab",
 ]
 
 _lib = None
@@ -61,6 +61,7 @@ def lib():
         L.jf_rowstats_finish.argtypes = [_p, _p, _i, _i, _i, _p, _p, _p]
         L.jf_igemm_block_q.argtypes = [_p, _p, _p, _p, _p, _p, _p, _p, _i, _i, _i, _i, _i, _i, _i, _i, _u64, _u64, _p, _sz, _p]
         L.jf_quantize.argtypes = [_p, _i, _i, _i, _p, _p, _p, _i, _i, _u64, _u64, _f, _p]
+        L.jf_quantize_slab.argtypes = [_p, _i, _i, _i, _i, _p, _p, _i, _i, _i, _i, _u64, _u64, _f, _p]
         L.jf_dequantize.argtypes = [_p, _p, _i, _i, _i, _p, _i, _p]
         L.jf_transpose_s8.argtypes = [_p, _i, _i, _p, _p]
         L.jf_rowstats.argtypes = [_p, _p, _i, _i, _i, _f, _p, _p, _p]
@@ -364,6 +365,30 @@ def _block_tensor(q, s, name):
     if s.device != q.device:
         raise RuntimeError(f"{name}: codes and scales are on different devices")
     return R, Cc, _scale_code(s, name)
+
+
+def quantize_slabs(slabs, rounding=ROUND_NEAREST, scale_dtype=torch.float16, amax_eps=0.0, seed=None, offset=None):
+    """quantize(torch.cat(slabs, dim=1)) without making the concatenation: every slab ([R, C_i], unit column stride, any
+    row stride) is quantised into its columns of one block tensor; same codes, scales and noise counters."""
+    R = slabs[0].shape[0]
+    widths = []
+    for x in slabs:
+        if not isinstance(x, torch.Tensor) or not x.is_cuda or x.dim() != 2 or x.shape[0] != R or x.stride(1) != 1:
+            raise RuntimeError("slabs: expected 2-D GPU tensors with the same number of rows and unit column stride")
+        if x.dtype not in _FP_CODE or x.dtype != slabs[0].dtype:
+            raise RuntimeError("slabs: one floating dtype for all of them")
+        widths.append(x.shape[1])
+    Ct = sum(widths)
+    _mult32(R, Ct, *widths)
+    seed, offset = _rng(rounding, R * Ct, seed, offset, slabs[0].device)
+    q = torch.empty((R, Ct), dtype=torch.int8, device=slabs[0].device)
+    s = torch.empty((R // QB, Ct // QB), dtype=scale_dtype, device=slabs[0].device)
+    col0 = 0
+    for x, w in zip(slabs, widths):
+        check(lib().jf_quantize_slab(_ptr(x), _FP_CODE[x.dtype], x.stride(0), R, w, _ptr(q), _ptr(s), Ct, col0,
+                                     _scale_code(s, "s"), rounding, seed, offset, amax_eps, _stream()))
+        col0 += w
+    return q, s
 
 
 def dequantize(q, s, out_dtype=torch.float32):

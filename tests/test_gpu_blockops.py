@@ -53,6 +53,30 @@ def test_quantize_half_inputs_and_transpose(jf, oracle, dtype):
     same(qT, np.ascontiguousarray(wq.T), "transposed codes")
 
 
+@pytest.mark.parametrize("dtype", [torch.float32, torch.float16, torch.bfloat16])
+@pytest.mark.parametrize("mode", ["nearest", "stochastic"])
+def test_quantize_slabs_equal_the_quantised_concatenation(jf, oracle, dtype, mode):
+    """Column slabs quantised where they lie (jf_quantize_slab: unit column stride, any row stride) give the codes,
+    scales and rounding noise of jf_quantize on their concatenation, and of the oracle on it."""
+    rng = np.random.default_rng(11)
+    R, widths = 96, (64, 160, 32)
+    parts = [torch.from_numpy(rand_x(rng, R, w) * (0.2 + i)).to(dtype).cuda() for i, w in enumerate(widths)]
+    wide = torch.from_numpy(rand_x(rng, R, 224)).to(dtype).cuda()
+    parts[1] = wide[:, 32:192]                                  # a slab with a row stride of its own (224 elements)
+    cat = torch.cat(parts, dim=1)
+    sd = torch.float16
+    q, s = jf.quantize_slabs(parts, ROUND[mode], sd, seed=42, offset=17)
+    q0, s0 = jf.quantize(cat, ROUND[mode], sd, seed=42, offset=17)
+    assert torch.equal(q, q0) and torch.equal(s, s0)
+    wq, ws = oracle.quantize(cat.float().cpu().numpy(), stochastic=mode == "stochastic", seed=42, offset=17, scale_dtype="f16")
+    same(q, wq, "codes")
+    same(s, ws, "scales")
+    with pytest.raises(RuntimeError):
+        jf.quantize_slabs([parts[0], parts[1][:64]])            # rows differ
+    with pytest.raises(RuntimeError):
+        jf.quantize_slabs([parts[0], wide[:, 1:33]])            # a slab that does not start on a 16-byte boundary
+
+
 def test_quantize_amax_eps_and_tiny_scales(jf, oracle):
     rng = np.random.default_rng(4)
     x = (rng.standard_normal((64, 64)) * 1e-25).astype(np.float32)     # scale below the fast-division range
