@@ -175,14 +175,15 @@ int jf_quantize(const void *x, int x_dtype, int R, int C, int8_t *q, void *s, in
                 int scale_dtype, int rounding, uint64_t seed, uint64_t offset, float amax_eps,
                 jf_stream_t stream);
 
-/* jf_quantize of a tensor that exists only as column slabs: x[R,C] (rows ldx elements apart) becomes the columns
- * col0 .. col0+C-1 of the block tensor (q: [R, ldq] codes, s: [R/32, ldq/32] scales; q and s point to the WIDE tensor).
- * Rounding noise is drawn by position in the wide tensor, so quantising every slab with the same (seed, offset) gives the
- * codes jf_quantize gives for the concatenation.  No counterpart in the reference, which quantises the concatenated
- * gradient of the attention kernel's three inputs (INT8_GPT2/qmodel.py:112-120 behind autograd's cat); here the three
- * gradients are quantised where they lie and the 78 MB concatenation is never made. */
-int jf_quantize_slab(const void *x, int x_dtype, int ldx, int R, int C, int8_t *q, void *s, int ldq, int col0,
-                     int scale_dtype, int rounding, uint64_t seed, uint64_t offset, float amax_eps, jf_stream_t stream);
+/* jf_quantize of a tensor that exists only as column slabs lying side by side: slab k is x[k], [R, widths[k]] with rows
+ * ldx[k] elements apart (nslabs <= 4; x, ldx, widths are HOST arrays); (q, s) is the block tensor of the concatenation,
+ * [R, sum of widths].  Rounding noise is drawn by position in the result, so the codes are those jf_quantize gives for
+ * the concatenated tensor.  No counterpart in the reference, which quantises the concatenated gradient of the attention
+ * kernel's three inputs (INT8_GPT2/qmodel.py:112-120 behind autograd's cat); here the three gradients are read where
+ * they lie and the 78 MB concatenation is never made. */
+int jf_quantize_slabs(const void *const *x, const int *ldx, const int *widths, int nslabs, int x_dtype, int R,
+                      int8_t *q, void *s, int scale_dtype, int rounding, uint64_t seed, uint64_t offset, float amax_eps,
+                      jf_stream_t stream);
 
 /* out[R,C] = q*s, the fp32 product rounded to `out_dtype` (JF_FP_F32 / JF_FP_F16 / JF_FP_BF16; for binary16 scales and
  * output this equals the reference's binary16 multiplication).  Replaces int8_dequantize

@@ -90,26 +90,36 @@ struct BlockPos {
 
 // ------------------------------------------------------------------------------------------------
 // quantize.py:33-117 (and quantize_transpose.py:33-129 when qT != nullptr)
-// x: [R, C] with rows ldx elements apart.  The result may be a column slab of a wider block tensor: q has rows of ldq
-// codes, s rows of ldq/32 scales, and the slab starts at column col0 of it (plain case: ldx = ldq = C, col0 = 0).  The
-// rounding noise of an element depends on its position in the WIDE tensor, so quantising a tensor slab by slab gives
-// the same codes as quantising it whole.
+// The input is up to QSRC_MAX column slabs lying side by side in the result: slab k is [R, end[k] - end[k-1]] with rows
+// ldx[k] elements apart (plain case: one slab, ldx = C).  The rounding noise of an element depends on its position in
+// the result, so quantising slabs where they lie gives the codes of quantising their concatenation.
+constexpr int QSRC_MAX = 4;
+struct QuantSrc {
+    const void *x[QSRC_MAX];
+    int ldx[QSRC_MAX];
+    int end[QSRC_MAX];       // first column behind slab k (cumulative widths)
+    int n;
+};
 template <typename T, typename ST>
-__global__ __launch_bounds__(NT) void quantize_kernel(const T *x, int R, int C, int ldx, int8_t *q, ST *s, int ldq, int col0,
-                                                      int8_t *qT, int rounding, uint64_t seed, uint64_t offset,
-                                                      float amax_eps)
+__global__ __launch_bounds__(NT) void quantize_kernel(QuantSrc src, int R, int C, int8_t *q, ST *s, int8_t *qT,
+                                                      int rounding, uint64_t seed, uint64_t offset, float amax_eps)
 {
     __shared__ __attribute__((aligned(16))) unsigned char tpatch[WPB][QB][QB + 16];
     JF_FOR_EACH_BLOCK(R, C)
     {
         BlockPos pos(blk, SC, C, lane);
+        // the slab of this block (uniform over the wave; slabs are whole blocks wide)
+        const T *x = reinterpret_cast<const T *>(src.x[0]);
+        int ldx = src.ldx[0], begin = 0;
+#pragma unroll
+        for (int k = 1; k < QSRC_MAX; ++k)
+            if (k < src.n && pos.cb * QB >= src.end[k - 1]) { x = reinterpret_cast<const T *>(src.x[k]); ldx = src.ldx[k]; begin = src.end[k - 1]; }
         float v[16];
-        Load16<T>::run(x + (size_t)pos.row * ldx + pos.col, v);
-        const size_t eq = (size_t)pos.row * ldq + col0 + pos.col;       // flat index in the wide tensor
+        Load16<T>::run(x + (size_t)pos.row * ldx + (pos.col - begin), v);
         float scale;
-        v4i codes = quantize16(v, amax_eps, rounding, seed, offset, eq, &scale);
-        *reinterpret_cast<v4i *>(q + eq) = codes;
-        if (lane == 0) store_scale(s, pos.rb * (ldq / QB) + col0 / QB + pos.cb, scale);
+        v4i codes = quantize16(v, amax_eps, rounding, seed, offset, pos.e0, &scale);
+        *reinterpret_cast<v4i *>(q + pos.e0) = codes;
+        if (lane == 0) store_scale(s, pos.rb * SC + pos.cb, scale);
         if (qT) {
             unsigned char(*tp)[QB + 16] = tpatch[threadIdx.x >> 6];
             *reinterpret_cast<v4i *>(&tp[lane >> 1][(lane & 1) * 16]) = codes;
@@ -935,8 +945,10 @@ int jf_quantize(const void *x, int x_dtype, int R, int C, int8_t *q, void *s, in
     if (!aligned16(x) || (qT && !aligned16(qT))) return JF_ERR_ALIGN;
     hipStream_t st = (hipStream_t)stream;
     const int grid = grid_for_blocks(R, C);
+    QuantSrc src = {};
+    src.x[0] = x; src.ldx[0] = C; src.end[0] = C; src.n = 1;
 #define JF_Q(T, ST)                                                                                          \
-    JF_LAUNCH((quantize_kernel<T, ST>), grid, 0, st, (const T *)x, R, C, C, q, (ST *)s, C, 0, qT, rounding, seed, offset, amax_eps)
+    JF_LAUNCH((quantize_kernel<T, ST>), grid, 0, st, src, R, C, q, (ST *)s, qT, rounding, seed, offset, amax_eps)
     if (scale_dtype == JF_SCALE_F16) {
         if (x_dtype == JF_FP_F32) JF_Q(float, half_t);
         if (x_dtype == JF_FP_F16) JF_Q(half_t, half_t);
@@ -949,21 +961,30 @@ int jf_quantize(const void *x, int x_dtype, int R, int C, int8_t *q, void *s, in
 #undef JF_Q
 }
 
-int jf_quantize_slab(const void *x, int x_dtype, int ldx, int R, int C, int8_t *q, void *s, int ldq, int col0,
-                     int scale_dtype, int rounding, uint64_t seed, uint64_t offset, float amax_eps, jf_stream_t stream)
+int jf_quantize_slabs(const void *const *x, const int *ldx, const int *widths, int nslabs, int x_dtype, int R,
+                      int8_t *q, void *s, int scale_dtype, int rounding, uint64_t seed, uint64_t offset, float amax_eps,
+                      jf_stream_t stream)
 {
+    if (!x || !ldx || !widths) return JF_ERR_NULL;
+    if (nslabs < 1 || nslabs > QSRC_MAX) return JF_ERR_SHAPE;
+    if (!rounding_ok(rounding) || x_dtype < JF_FP_F16 || x_dtype > JF_FP_BF16) return JF_ERR_ENUM;
+    const size_t xbytes = x_dtype == JF_FP_F32 ? 4 : 2;
+    QuantSrc src = {};
+    int C = 0;
+    for (int k = 0; k < nslabs; ++k) {
+        if (!x[k]) return JF_ERR_NULL;
+        if (!mult32(widths[k]) || ldx[k] < widths[k]) return JF_ERR_SHAPE;
+        if (!aligned16(x[k]) || ((size_t)ldx[k] * xbytes) % 16) return JF_ERR_ALIGN;
+        C += widths[k];
+        src.x[k] = x[k]; src.ldx[k] = ldx[k]; src.end[k] = C;
+    }
+    src.n = nslabs;
     int rc = check_block_tensor(q, s, R, C, scale_dtype);
     if (rc) return rc;
-    if (!x) return JF_ERR_NULL;
-    if (!rounding_ok(rounding) || x_dtype < JF_FP_F16 || x_dtype > JF_FP_BF16) return JF_ERR_ENUM;
-    if (!mult32(ldq) || col0 < 0 || col0 % QB || col0 + C > ldq || ldx < C) return JF_ERR_SHAPE;
-    const size_t xbytes = x_dtype == JF_FP_F32 ? 4 : 2;
-    if (!aligned16(x) || ((size_t)ldx * xbytes) % 16) return JF_ERR_ALIGN;
     hipStream_t st = (hipStream_t)stream;
     const int grid = grid_for_blocks(R, C);
 #define JF_Q(T, ST)                                                                                          \
-    JF_LAUNCH((quantize_kernel<T, ST>), grid, 0, st, (const T *)x, R, C, ldx, q, (ST *)s, ldq, col0, (int8_t *)nullptr, \
-              rounding, seed, offset, amax_eps)
+    JF_LAUNCH((quantize_kernel<T, ST>), grid, 0, st, src, R, C, q, (ST *)s, (int8_t *)nullptr, rounding, seed, offset, amax_eps)
     if (scale_dtype == JF_SCALE_F16) {
         if (x_dtype == JF_FP_F32) JF_Q(float, half_t);
         if (x_dtype == JF_FP_F16) JF_Q(half_t, half_t);

@@ -29,7 +29,7 @@ EXPORTS = [
     "jf_igemm_splitk_plan", "jf_igemm_block_fp_workspace_bytes", "jf_igemm_block_q_gelu", "jf_igemm_block_fp_noalloc", "jf_igemm_block_q_gelu_bwd",
     "jf_igemm_block_q", "jf_quantize", "jf_dequantize", "jf_transpose_s8", "jf_rowstats", "jf_layernorm_fwd",
     "jf_layernorm_bwd_workspace_bytes", "jf_layernorm_bwd", "jf_gelu_fwd", "jf_gelu_bwd", "jf_add", "jf_calibrate", "jf_wall_clock_khz", "jf_igemm_phase_record", "jf_rowstats_finish",
-    "jf_igemm_block_q_dequant", "jf_quantize_slab",
+    "jf_igemm_block_q_dequant", "jf_quantize_slabs",
 ]
 
 _lib = None
@@ -61,7 +61,7 @@ def lib():
         L.jf_rowstats_finish.argtypes = [_p, _p, _i, _i, _i, _p, _p, _p]
         L.jf_igemm_block_q.argtypes = [_p, _p, _p, _p, _p, _p, _p, _p, _i, _i, _i, _i, _i, _i, _i, _i, _u64, _u64, _p, _sz, _p]
         L.jf_quantize.argtypes = [_p, _i, _i, _i, _p, _p, _p, _i, _i, _u64, _u64, _f, _p]
-        L.jf_quantize_slab.argtypes = [_p, _i, _i, _i, _i, _p, _p, _i, _i, _i, _i, _u64, _u64, _f, _p]
+        L.jf_quantize_slabs.argtypes = [_p, _p, _p, _i, _i, _i, _p, _p, _i, _i, _u64, _u64, _f, _p]
         L.jf_dequantize.argtypes = [_p, _p, _i, _i, _i, _p, _i, _p]
         L.jf_transpose_s8.argtypes = [_p, _i, _i, _p, _p]
         L.jf_rowstats.argtypes = [_p, _p, _i, _i, _i, _f, _p, _p, _p]
@@ -381,13 +381,16 @@ def quantize_slabs(slabs, rounding=ROUND_NEAREST, scale_dtype=torch.float16, ama
     Ct = sum(widths)
     _mult32(R, Ct, *widths)
     seed, offset = _rng(rounding, R * Ct, seed, offset, slabs[0].device)
+    if len(slabs) > 4:
+        raise RuntimeError("at most 4 slabs")
     q = torch.empty((R, Ct), dtype=torch.int8, device=slabs[0].device)
     s = torch.empty((R // QB, Ct // QB), dtype=scale_dtype, device=slabs[0].device)
-    col0 = 0
-    for x, w in zip(slabs, widths):
-        check(lib().jf_quantize_slab(_ptr(x), _FP_CODE[x.dtype], x.stride(0), R, w, _ptr(q), _ptr(s), Ct, col0,
-                                     _scale_code(s, "s"), rounding, seed, offset, amax_eps, _stream()))
-        col0 += w
+    n = len(slabs)
+    xs = (C.c_void_p * n)(*[x.data_ptr() for x in slabs])
+    ld = (C.c_int * n)(*[x.stride(0) for x in slabs])
+    wd = (C.c_int * n)(*widths)
+    check(lib().jf_quantize_slabs(xs, ld, wd, n, _FP_CODE[slabs[0].dtype], R, _ptr(q), _ptr(s), _scale_code(s, "s"),
+                                  rounding, seed, offset, amax_eps, _stream()))
     return q, s
 
 

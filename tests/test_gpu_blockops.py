@@ -56,7 +56,7 @@ def test_quantize_half_inputs_and_transpose(jf, oracle, dtype):
 @pytest.mark.parametrize("dtype", [torch.float32, torch.float16, torch.bfloat16])
 @pytest.mark.parametrize("mode", ["nearest", "stochastic"])
 def test_quantize_slabs_equal_the_quantised_concatenation(jf, oracle, dtype, mode):
-    """Column slabs quantised where they lie (jf_quantize_slab: unit column stride, any row stride) give the codes,
+    """Column slabs quantised where they lie (jf_quantize_slabs: unit column stride, any row stride) give the codes,
     scales and rounding noise of jf_quantize on their concatenation, and of the oracle on it."""
     rng = np.random.default_rng(11)
     R, widths = 96, (64, 160, 32)
