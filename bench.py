@@ -186,7 +186,7 @@ def deep_k_weight_gradients(jf, torch):
     return out
 
 
-def recipe_block(torch):
+def recipe_block(torch, only=None):
     """GPT-2 XL transformer blocks (1600 wide, 25 heads) forward + backward on 8 x 1024 tokens: the INT8 data-flow
     recipe (Jetfire/recipe.py: every linear layer, LayerNorm, GELU and residual add on INT8 block tensors, attention
     itself in fp16 through torch) next to the same blocks in plain torch bf16.  Measured for a stack of one block (which
@@ -219,7 +219,7 @@ def recipe_block(torch):
         return e0.elapsed_time(e1) / n
 
     out = {}
-    for layers in (1, 3):
+    for layers in ((3,) if only else (1, 3)):
         model = QStack(layers, C, H).cuda()
 
         def ref_stack(h0, dt):
@@ -233,6 +233,9 @@ def recipe_block(torch):
                 h0 = h0 + F.gelu(h @ blk.w_fc.to(dt).t()) @ blk.w_mlp_proj.to(dt).t()
             return h0
         params = list(model.parameters())
+        if only:                                                   # one of the two, 3 + 10 steps: a kernel trace of it
+            return round(t(lambda: model(x).backward(w), params + [x]) if only == "int8"
+                         else t(lambda: ref_stack(xr, torch.bfloat16).backward(wr), params + [xr]), 3)
         out[layers] = (t(lambda: model(x).backward(w), params + [x]),
                        t(lambda: ref_stack(xr, torch.bfloat16).backward(wr), params + [xr]))
         del model
@@ -509,7 +512,9 @@ def main():
     ap.add_argument("--roofline-only", action="store_true", help="only the dominant-kernel measurement (for rocprofv3 --stats)")
     ap.add_argument("--extras-only", action="store_true", help="only the block-kernel section (for rocprofv3 --pmc)")
     ap.add_argument("--calibration-only", action="store_true", help="only the register-only calibration loops")
-    ap.add_argument("--block-only", action="store_true", help="only the transformer-block comparison (for rocprofv3 --stats)")
+    ap.add_argument("--block-only", action="store_true", help="only the transformer-block comparison")
+    ap.add_argument("--stack-only", choices=["int8", "bf16"], default=None,
+                    help="10 steps of a three-block GPT-2 XL stack through the INT8 recipe or plain torch bf16 (for rocprofv3 --stats)")
     a = ap.parse_args()
     if a.gpus != 1:
         sys.exit("bench.py: this build measures one GPU only (--gpus 1); nothing here uses a second GPU")
@@ -525,6 +530,9 @@ def main():
         return
     if a.block_only:
         print(json.dumps({"xl_block_forward_backward": recipe_block(torch)}))
+        return
+    if a.stack_only:
+        print(json.dumps({"stack_of_3_blocks_ms": recipe_block(torch, only=a.stack_only)}))
         return
     ops = make_inputs(jf, torch)
     if a.pmc_probe:
