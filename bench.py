@@ -233,6 +233,21 @@ def recipe_block(torch, only=None):
                 h0 = h0 + F.gelu(h @ blk.w_fc.to(dt).t()) @ blk.w_mlp_proj.to(dt).t()
             return h0
         params = list(model.parameters())
+
+        def peak_mb(fn):
+            # memory held at the end of the forward pass above what is held before it (saved activations + output)
+            for q in params + [x, xr]:
+                q.grad = None
+            torch.cuda.synchronize()
+            base = torch.cuda.memory_allocated()
+            y = fn()
+            torch.cuda.synchronize()
+            held = torch.cuda.memory_allocated() - base
+            y.backward(w if y.dtype == w.dtype else wr)
+            del y
+            return round(held / 2 ** 20, 1)
+        if layers == 3 and not only:
+            out["mem"] = (peak_mb(lambda: model(x)), peak_mb(lambda: ref_stack(xr, torch.bfloat16)))
         if only:                                                   # one of the two, 3 + 10 steps: a kernel trace of it
             return round(t(lambda: model(x).backward(w), params + [x]) if only == "int8"
                          else t(lambda: ref_stack(xr, torch.bfloat16).backward(wr), params + [xr]), 3)
@@ -240,7 +255,8 @@ def recipe_block(torch, only=None):
                        t(lambda: ref_stack(xr, torch.bfloat16).backward(wr), params + [xr]))
         del model
     return {"tokens": B * T, "int8_recipe_ms": round(out[1][0], 3), "torch_bf16_ms": round(out[1][1], 3),
-            "stack_of_3_blocks": {"int8_recipe_ms": round(out[3][0], 3), "torch_bf16_ms": round(out[3][1], 3)},
+            "stack_of_3_blocks": {"int8_recipe_ms": round(out[3][0], 3), "torch_bf16_ms": round(out[3][1], 3),
+                                  "held_after_forward_MiB": {"int8_recipe": out["mem"][0], "torch_bf16": out["mem"][1]}},
             "per_block_inside_a_stack": {"int8_recipe_ms": round((out[3][0] - out[1][0]) / 2, 3),
                                          "torch_bf16_ms": round((out[3][1] - out[1][1]) / 2, 3)}}
 
