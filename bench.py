@@ -312,6 +312,11 @@ def nonlinear_extras(jf, torch):
     put("transpose_8192x1600", t(lambda: jf.transpose_s8(qx)), 2 * n)
     put("layernorm_fwd_8192x1600", t(lambda: jf.layernorm_fwd(qx, sx, gamma, beta, mean, rstd)), 2 * n)
     put("layernorm_bwd_sr_8192x1600", t(lambda: jf.layernorm_bwd(qx, sx, qg, sg, gamma, mean, rstd, jf.ROUND_STOCHASTIC, seed=1, offset=0)), 3 * n)
+    # residual add: fp32 in + codes in, fp32 out + codes out (the reference's default truncation; the backward's stochastic
+    # form; the forward's form with the row partial sums and their finishing launch)
+    put("add_8192x1600", t(lambda: jf.add(x, qx, sx, jf.ROUND_TRUNC)), 10 * n)
+    put("add_sr_8192x1600", t(lambda: jf.add(x, qx, sx, jf.ROUND_STOCHASTIC_TRUNC, seed=1, offset=0)), 10 * n)
+    put("add_meanvar_8192x1600", t(lambda: jf.rowstats_finish(*jf.add(x, qx, sx, jf.ROUND_TRUNC, with_stats=True)[3:], C)), 10 * n)
     R, C = TOKENS, 6400
     x = torch.randn(R, C, generator=g).cuda()
     dy = (torch.randn(R, C, generator=g) * 1e-3).cuda()
