@@ -1080,11 +1080,11 @@ int jf_layernorm_bwd(const int8_t *qx, const void *sx, const int8_t *qg, const v
         float *sdg = (float *)workspace, *sdb = sdg + (size_t)(R / QB) * C;      // [R/32][C] each: fits the size above
         const size_t lds = ((size_t)C + 2 * SC * QB + 2 * 8 * QB + 2 * QB + (want_dw ? LNS_WAVES * COLSUM_PATCH : 0)) * sizeof(float);
         int dev = 0;
-        if (hipGetDevice(&dev) != hipSuccess || dev < 0 || dev >= 64) return JF_ERR_DEVICE;
+        if (hipGetDevice(&dev) != hipSuccess || dev < 0 || dev >= MAX_DEVICES) return JF_ERR_DEVICE;
 #define JF_LNS(ST, DW)                                                                                                 \
         do {                                                                                                           \
             auto kern = layernorm_bwd_strip_kernel<ST, DW>;                                                            \
-            static std::atomic<bool> opted_in[64] = {};           /* more than 64 KiB of LDS: once per device */        \
+            static std::atomic<bool> opted_in[MAX_DEVICES] = {};  /* more than 64 KiB of LDS: once per device */        \
             if (lds > 64 * 1024 && !opted_in[dev].load(std::memory_order_acquire)) {                                   \
                 hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void *>(kern),                               \
                                                    hipFuncAttributeMaxDynamicSharedMemorySize, 160 * 1024);            \

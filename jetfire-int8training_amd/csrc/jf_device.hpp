@@ -458,11 +458,12 @@ __device__ __forceinline__ v4i gelu_bwd_block(v4i cx, float scx, v4i cg, float s
 // host-side argument checks shared by the entry points
 // The kernels exist as gfx950 code objects only: say so instead of failing at launch with "no binary for GPU".
 // (One property query per device and process; afterwards a table look-up.)
+constexpr int MAX_DEVICES = 64;                     // devices a process may use (per-device host state)
 static inline bool device_is_gfx950()
 {
-    static signed char known[64] = {};           // 0: not asked yet, 1: gfx950, -1: something else
+    static signed char known[MAX_DEVICES] = {};           // 0: not asked yet, 1: gfx950, -1: something else
     int dev = 0;
-    if (hipGetDevice(&dev) != hipSuccess || dev < 0 || dev >= 64) return false;
+    if (hipGetDevice(&dev) != hipSuccess || dev < 0 || dev >= MAX_DEVICES) return false;
     if (known[dev] == 0) {
         hipDeviceProp_t prop;
         bool ok = hipGetDeviceProperties(&prop, dev) == hipSuccess;

@@ -35,7 +35,6 @@ namespace jf {
 
 constexpr int KB_STAGE = 4;                         // 32-deep K blocks per LDS stage (128 bytes of K per row)
 constexpr int ROW_BYTES = KB_STAGE * QB;            // 128: one LDS row = one 128-byte global segment
-constexpr int MAX_DEVICES = 64;                    // devices a process may use (per-device host state below)
 constexpr int EPI_LD = 36;                          // floats per staged row (32 + pad, keeps 16B alignment)
 
 // EPI_QG: EPI_Q (deterministic) followed by the GELU forward of the block just requantised: two block tensors leave
