@@ -93,6 +93,15 @@ struct BlockPos {
 // The input is up to QSRC_MAX column slabs lying side by side in the result: slab k is [R, end[k] - end[k-1]] with rows
 // ldx[k] elements apart (plain case: one slab, ldx = C).  The rounding noise of an element depends on its position in
 // the result, so quantising slabs where they lie gives the codes of quantising their concatenation.
+// workgroups of the quantize kernel (4 waves = 4 adjacent column blocks of one row block); with a transposed copy: 32 per
+// 8 (quad of row blocks, group of 4 column blocks) pairs, see the kernel
+__host__ __device__ static inline int quantize_groups(int R, int C, bool transposed)
+{
+    const int RB = R / QB, SC = C / QB, G4 = (SC + WPB - 1) / WPB;
+    if (!transposed) return (RB * SC + WPB - 1) / WPB;
+    const int pairs = ((RB + 3) / 4) * G4;
+    return 32 * ((pairs + 7) / 8);
+}
 constexpr int QSRC_MAX = 4;
 struct QuantSrc {
     const void *x[QSRC_MAX];
@@ -105,8 +114,26 @@ __global__ __launch_bounds__(NT) void quantize_kernel(QuantSrc src, int R, int C
                                                       int rounding, uint64_t seed, uint64_t offset, float amax_eps)
 {
     __shared__ __attribute__((aligned(16))) unsigned char tpatch[WPB][QB][QB + 16];
-    JF_FOR_EACH_BLOCK(R, C)
+    const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+    const int SC = C / QB, RB = R / QB, G4 = (SC + WPB - 1) / WPB;
+    // Which blocks a workgroup takes: four adjacent column blocks of one row block (whole 128-byte lines of q).  Without
+    // a transposed copy workgroups walk the tensor row block by row block.  With one, the 128-byte lines of qT are
+    // written 32 bytes at a time by the workgroups of four consecutive row blocks: those four are made the workgroups
+    // b, b+8, b+16, b+24, which the dispatcher deals to the same XCD one after the other, so that the four pieces of a
+    // line meet in that XCD's L2 before the line leaves for memory (see quantize_groups() for the count).
+    const int nwg = qT ? quantize_groups(R, C, true) : (RB * SC + WPB - 1) / WPB;
+    for (int wg = blockIdx.x; wg < nwg; wg += gridDim.x)
     {
+        int blk;
+        if (qT) {
+            const int idx = (wg >> 5) * 8 + (wg & 7), j = (wg >> 3) & 3;     // (row-block quad, column group) and the row block of the quad
+            const int rbq = (idx / G4) * 4 + j, cbq = (idx % G4) * WPB + wave;
+            if (rbq >= RB || cbq >= SC) continue;                           // wave-uniform
+            blk = rbq * SC + cbq;
+        } else {
+            blk = wg * WPB + wave;
+            if (blk >= RB * SC) continue;
+        }
         BlockPos pos(blk, SC, C, lane);
         // the slab of this block (uniform over the wave; slabs are whole blocks wide)
         const T *x = reinterpret_cast<const T *>(src.x[0]);
@@ -126,12 +153,19 @@ __global__ __launch_bounds__(NT) void quantize_kernel(QuantSrc src, int R, int C
             __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
             __builtin_amdgcn_wave_barrier();
             __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
-            unsigned char b[16];
-            const int ocol = lane >> 1, orow0 = (lane & 1) * 16;     // output row = input column
-#pragma unroll
-            for (int k = 0; k < 16; ++k) b[k] = tp[orow0 + k][ocol];
-            *reinterpret_cast<v4i *>(qT + (size_t)(pos.cb * QB + ocol) * R + pos.rb * QB + orow0) =
-                *reinterpret_cast<v4i *>(b);
+            // The transposing LDS read of gfx950 (groups of 16 lanes; lanes 2k, 2k+1 address the two 8-byte pieces of
+            // patch row k, lane i receives byte i%8 of the pieces addressed by lanes i/8, i/8+2, ..: one column, 8 rows).
+            // Lane group g takes the 16-column window g%2 and the 16-row half g/2 of the block; two reads (rows +0..7,
+            // +8..15) leave a lane with 16 consecutive bytes of one output row.
+            typedef __attribute__((address_space(3))) unsigned char lds_u8;
+            const int g = lane >> 4, i = lane & 15, cw = g & 1, rh = g >> 1;
+            const unsigned addr = (unsigned)(uintptr_t)(lds_u8 *)&tp[16 * rh + (i >> 1)][16 * cw + 8 * (i & 1)];
+            v2i lo, hi;
+            asm volatile("ds_read_b64_tr_b8 %0, %1" : "=v"(lo) : "v"(addr));
+            asm volatile("ds_read_b64_tr_b8 %0, %1 offset:%2" : "=v"(hi) : "v"(addr), "n"(8 * (QB + 16)));
+            asm volatile("s_waitcnt lgkmcnt(0)" : "+v"(lo), "+v"(hi));
+            const int ocol = 16 * cw + (i & 7) + 8 * (i >> 3);           // output row = input column
+            *reinterpret_cast<v4i *>(qT + (size_t)(pos.cb * QB + ocol) * R + pos.rb * QB + 16 * rh) = v4i{lo.x, lo.y, hi.x, hi.y};
             __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
             __builtin_amdgcn_wave_barrier();
         }
@@ -944,7 +978,8 @@ int jf_quantize(const void *x, int x_dtype, int R, int C, int8_t *q, void *s, in
     if (!rounding_ok(rounding) || x_dtype < JF_FP_F16 || x_dtype > JF_FP_BF16) return JF_ERR_ENUM;
     if (!aligned16(x) || (qT && !aligned16(qT))) return JF_ERR_ALIGN;
     hipStream_t st = (hipStream_t)stream;
-    const int grid = grid_for_blocks(R, C);
+    const int groups = quantize_groups(R, C, qT != nullptr);
+    const int grid = groups < 256 * 32 ? groups : 256 * 32;       // (a multiple of 32, which the transposed walk needs)
     QuantSrc src = {};
     src.x[0] = x; src.ldx[0] = C; src.end[0] = C; src.n = 1;
 #define JF_Q(T, ST)                                                                                          \

@@ -810,35 +810,56 @@ __global__ __launch_bounds__(64 * WGM * WGN, WGPC * WGM * WGN / 4) void igemm_nt
 }
 
 // -------------------------------------------------------------------------------------------------
-// int8 transpose: out[C,R] = in[R,C].  64x64 tiles through LDS; 16-byte loads and stores.
+// int8 transpose: out[C,R] = in[R,C].  TR_ROWS x 64 tiles through LDS: 16-byte loads, the transposing LDS read of gfx950
+// (ds_read_b64_tr_b8, as for the GEMM's [K,N] operands) and 16-byte stores.  The instruction works on groups of 16 lanes:
+// lanes 2k and 2k+1 of a group address the 8-byte pieces [8 columns] x 2 of tile row k (k = 0..7), and lane i receives
+// byte i%8 of the pieces addressed by lanes i/8, i/8 + 2, ..., i/8 + 14: column i of the 16, rows 0..7.  Two reads (rows
+// +0..7, +8..15) give a lane 16 consecutive bytes of one output row.  Wave w of the workgroup takes tile columns 16w ..
+// 16w+15 (16 output rows); its four lane groups take 16 tile rows each, so a store instruction writes 64 contiguous bytes
+// of each of its 16 output rows, and the passes of a tall tile continue those runs.
+constexpr int TR_ROWS = 64;                        // tile rows (input rows = bytes per output-row run)
 __global__ __launch_bounds__(256) void transpose_s8_kernel(const int8_t *in, int8_t *out, int R, int C)
 {
-    __shared__ __attribute__((aligned(16))) unsigned char tile[64][64 + 16];
+    __shared__ __attribute__((aligned(16))) unsigned char tile[TR_ROWS][64 + 16];
+    typedef __attribute__((address_space(3))) unsigned char lds_u8;
     const int tiles_c = (C + 63) / 64;
-    const int tr = blockIdx.x / tiles_c, tc = blockIdx.x % tiles_c;
-    const int r0 = tr * 64, c0 = tc * 64;
+    // Workgroups are dealt round-robin to the 8 XCDs: with 8 consecutive workgroups on 8 consecutive row tiles of one
+    // column tile, every XCD walks along the columns of its own rows, so the two 64-byte halves of a 128-byte line meet
+    // in one L2 (measured at 8192x6400: 17.8 us against 24.4 us with the column tile running fastest).
+    const int tiles_r = (R + TR_ROWS - 1) / TR_ROWS;
+    const int per = 8 * tiles_c, grp = blockIdx.x / per, rem = blockIdx.x % per;
+    const int nr = (tiles_r - grp * 8) < 8 ? (tiles_r - grp * 8) : 8;
+    const int tr = grp * 8 + rem % nr, tc = rem / nr;
+    const int r0 = tr * TR_ROWS, c0 = tc * 64;
     const int tid = threadIdx.x;
-    {
-        const int row = tid >> 2, ch = tid & 3;                 // 64 rows x 4 chunks of 16 bytes
+#pragma unroll
+    for (int pass = 0; pass < TR_ROWS / 64; ++pass) {
+        const int row = pass * 64 + (tid >> 2), ch = tid & 3;   // 64 rows x 4 chunks of 16 bytes per pass
         v4i v = {0, 0, 0, 0};
         if (r0 + row < R && c0 + ch * 16 < C)
             v = *reinterpret_cast<const v4i *>(in + (size_t)(r0 + row) * C + c0 + ch * 16);
         *reinterpret_cast<v4i *>(&tile[row][ch * 16]) = v;
     }
     __syncthreads();
-    {
-        const int orow = tid >> 2, och = tid & 3;               // output row = input column
-        unsigned char b[16];
+    const int lane = tid & 63, wave = tid >> 6;
+    const int g = lane >> 4, i = lane & 15;
+    const int ocol = 16 * wave + (i & 7) + 8 * (i >> 3);        // tile column this lane receives = output row
 #pragma unroll
-        for (int k = 0; k < 16; ++k) b[k] = tile[och * 16 + k][orow];
-        if (c0 + orow < C && r0 + och * 16 < R)
-            *reinterpret_cast<v4i *>(out + (size_t)(c0 + orow) * R + r0 + och * 16) = *reinterpret_cast<v4i *>(b);
+    for (int pass = 0; pass < TR_ROWS / 64; ++pass) {
+        const int trow = pass * 64 + 16 * g;                    // first of the 16 tile rows of this lane group
+        const unsigned addr = (unsigned)(uintptr_t)(lds_u8 *)&tile[trow + (i >> 1)][16 * wave + 8 * (i & 1)];
+        v2i lo, hi;
+        asm volatile("ds_read_b64_tr_b8 %0, %1" : "=v"(lo) : "v"(addr));
+        asm volatile("ds_read_b64_tr_b8 %0, %1 offset:%2" : "=v"(hi) : "v"(addr), "n"(8 * (64 + 16)));
+        asm volatile("s_waitcnt lgkmcnt(0)" : "+v"(lo), "+v"(hi));
+        if (c0 + ocol < C && r0 + trow < R)
+            *reinterpret_cast<v4i *>(out + (size_t)(c0 + ocol) * R + r0 + trow) = v4i{lo.x, lo.y, hi.x, hi.y};
     }
 }
 
 static int launch_transpose(const int8_t *in, int R, int C, int8_t *out, hipStream_t st)
 {
-    const int tiles = ((R + 63) / 64) * ((C + 63) / 64);
+    const int tiles = ((R + TR_ROWS - 1) / TR_ROWS) * ((C + 63) / 64);
     hipLaunchKernelGGL(transpose_s8_kernel, dim3(tiles), dim3(256), 0, st, in, out, R, C);
     return (int)hipGetLastError();
 }
