@@ -42,10 +42,13 @@ def test_quantize(jf, oracle, R, C, mode, f16):
     same(s, ws, "scales")
 
 
+@pytest.mark.parametrize("R,C", [(96, 160), (32, 32), (160, 96), (288, 1056), (1056, 288)])
 @pytest.mark.parametrize("dtype", [torch.float16, torch.bfloat16])
-def test_quantize_half_inputs_and_transpose(jf, oracle, dtype):
+def test_quantize_half_inputs_and_transpose(jf, oracle, dtype, R, C):
+    """(shapes: row-block counts that are not multiples of 4 and column-block counts that are not multiples of 4: the
+    kernel's walk with a transposed copy takes quads of row blocks and groups of four column blocks)"""
     rng = np.random.default_rng(3)
-    x = torch.from_numpy(rand_x(rng, 96, 160)).to(dtype)
+    x = torch.from_numpy(rand_x(rng, R, C)).to(dtype)
     q, s, qT = jf.quantize(x.cuda(), rounding=jf.ROUND_STOCHASTIC, transpose=True, seed=5, offset=0)
     wq, ws = oracle.quantize(x.float().numpy(), stochastic=True, seed=5, offset=0, scale_dtype="f16")
     same(q, wq, "codes")
@@ -91,7 +94,7 @@ def test_quantize_amax_eps_and_tiny_scales(jf, oracle):
     same(s, ws, "scales eps")
 
 
-@pytest.mark.parametrize("R,C", [(32, 32), (96, 160), (16, 48), (1600, 8192)])
+@pytest.mark.parametrize("R,C", [(32, 32), (96, 160), (16, 48), (48, 80), (80, 16), (208, 1040), (1040, 528), (1600, 8192)])
 def test_transpose(jf, R, C):
     rng = np.random.default_rng(R)
     q = rand_codes(rng, (R, C))
