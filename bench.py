@@ -192,7 +192,9 @@ def recipe_block(torch, only=None):
     itself in fp16 through torch) next to the same blocks in plain torch bf16.  Measured for a stack of one block (which
     includes the stack's own begin / end: quantising the input, its row statistics, quantising the output gradient) and
     of three; the difference, halved, is what a block costs inside a stack.  Parameter gradients are reset to None before
-    every step, as an optimizer's zero_grad() does."""
+    every step, as an optimizer's zero_grad() does.  The INT8 stack takes a float32 input (an embedding's output) and
+    carries a bfloat16 residual between blocks, as the reference does (INT8_GPT2/qmodel.py:228); the sum inside a block
+    stays float32."""
     import torch.nn.functional as F
     sys.path.insert(0, os.path.join(PKG, "Jetfire"))
     from recipe import QStack
@@ -220,7 +222,7 @@ def recipe_block(torch, only=None):
 
     out = {}
     for layers in ((3,) if only else (1, 3)):
-        model = QStack(layers, C, H).cuda()
+        model = QStack(layers, C, H, stream_dtype=torch.bfloat16).cuda()    # fp32 in, bfloat16 between blocks and out
 
         def ref_stack(h0, dt):
             for blk in model.blocks:
@@ -249,9 +251,9 @@ def recipe_block(torch, only=None):
         if layers == 3 and not only:
             out["mem"] = (peak_mb(lambda: model(x)), peak_mb(lambda: ref_stack(xr, torch.bfloat16)))
         if only:                                                   # one of the two, 3 + 10 steps: a kernel trace of it
-            return round(t(lambda: model(x).backward(w), params + [x]) if only == "int8"
+            return round(t(lambda: model(x).backward(wr), params + [x]) if only == "int8"
                          else t(lambda: ref_stack(xr, torch.bfloat16).backward(wr), params + [xr]), 3)
-        out[layers] = (t(lambda: model(x).backward(w), params + [x]),
+        out[layers] = (t(lambda: model(x).backward(wr), params + [x]),
                        t(lambda: ref_stack(xr, torch.bfloat16).backward(wr), params + [xr]))
         del model
     return {"tokens": B * T, "int8_recipe_ms": round(out[1][0], 3), "torch_bf16_ms": round(out[1][1], 3),

@@ -228,14 +228,17 @@ int jf_gelu_bwd(const int8_t *qx, const void *sx, const int8_t *qg, const void *
                 int scale_dtype, int approx, int rounding, uint64_t seed, uint64_t offset,
                 int8_t *qy, void *sy, jf_stream_t stream);
 
-/* y1_f32 = x1 + q2*s2, (q, s) = block quantisation of y1; optional per-row, per-32-column partial
- * sums of y1 and y1^2 (rowsum, rowsq: [C/32, R] fp32 -- part-major, so that a block's 32 rows are one contiguous store;
- * may be NULL).
+/* y = x1 + q2*s2 in fp32, (q, s) = block quantisation of y; optional per-row, per-32-column partial
+ * sums of y and y^2 (rowsum, rowsq: [C/32, R] fp32 -- part-major, so that a block's 32 rows are one contiguous store;
+ * may be NULL).  y1 receives y in y1_dtype (JF_FP_F32: as the reference's kernels write it; JF_FP_F16 / JF_FP_BF16: y
+ * rounded to nearest even, i.e. the kernel followed by the cast the reference's recipe applies to it,
+ * INT8_GPT2/qmodel.py:228, without the fp32 tensor in between).  The quantisation and the partial sums always use the
+ * fp32 y.
  * Replaces int8_add_Ifp_Ig16_Ofp_Og (Jetfire/Nonlinear/add.py:164-211) and
  * int8_add_Ifp_Ig16_Ofp_Og_MeanVar (Jetfire/Nonlinear/add_mean_var.py:179-230). */
 int jf_add(const void *x1, int x1_dtype, const int8_t *q2, const void *s2, int R, int C,
            int scale_dtype, int rounding, uint64_t seed, uint64_t offset,
-           float *y1, int8_t *q, void *s, float *rowsum, float *rowsq, jf_stream_t stream);
+           void *y1, int y1_dtype, int8_t *q, void *s, float *rowsum, float *rowsq, jf_stream_t stream);
 
 /* mean[r] = (sum of rowsum[0..parts-1, r], ascending) / C;  rstd[r] = 1 / sqrt((sum of rowsq[:, r]) / C - mean[r]^2)
  * (no epsilon): the finishing step of int8_add_Ifp_Ig16_Ofp_Og_MeanVar (Jetfire/Nonlinear/add_mean_var.py:219-221), which

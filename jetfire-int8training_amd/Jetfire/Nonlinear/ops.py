@@ -168,20 +168,22 @@ def _add_rounding(stochastic, rounding):
     raise RuntimeError("rounding must be 'trunc' or 'nearest'")
 
 
-def int8_add_Ifp_Ig16_Ofp_Og(x1, x2, s_x2, QB, stochastic=False, rounding="trunc"):
-    """y1 = x1 + dequant(x2) as float32, and its block quantisation (y2, s_y2).  Reference: add.py:164-211."""
+def int8_add_Ifp_Ig16_Ofp_Og(x1, x2, s_x2, QB, stochastic=False, rounding="trunc", out_dtype=torch.float32):
+    """y1 = x1 + dequant(x2) as float32, and its block quantisation (y2, s_y2).  Reference: add.py:164-211.
+    out_dtype = float16 / bfloat16: y1 leaves the kernel already cast (what the reference's recipe does with a separate
+    `.to()`, qmodel.py:228); y2, s_y2 are those of the fp32 sum either way."""
     _check_qb(QB)
     sh = _Shape(x1)
-    y1, q, s = _jf.add(sh.flat(x1), sh.flat(x2), sh.flat(s_x2), _add_rounding(stochastic, rounding))
+    y1, q, s = _jf.add(sh.flat(x1), sh.flat(x2), sh.flat(s_x2), _add_rounding(stochastic, rounding), out_dtype=out_dtype)
     return sh.fold(y1), sh.fold(q), sh.fold(s)
 
 
-def int8_add_Ifp_Ig16_Ofp_Og_MeanVar(x1, x2, s_x2, QB, rounding="trunc"):
-    """As above plus per-row (mean, rstd) of y1 for the next LayerNorm: var = E[y^2] - mean^2, rstd = 1/sqrt(var),
-    no epsilon (reference: add_mean_var.py:179-230, finishing step :219-221)."""
+def int8_add_Ifp_Ig16_Ofp_Og_MeanVar(x1, x2, s_x2, QB, rounding="trunc", out_dtype=torch.float32):
+    """As above plus per-row (mean, rstd) of the fp32 y1 for the next LayerNorm: var = E[y^2] - mean^2,
+    rstd = 1/sqrt(var), no epsilon (reference: add_mean_var.py:179-230, finishing step :219-221)."""
     _check_qb(QB)
     sh = _Shape(x1)
     y1, q, s, rowsum, rowsq = _jf.add(sh.flat(x1), sh.flat(x2), sh.flat(s_x2), _add_rounding(False, rounding),
-                                      with_stats=True)
+                                      with_stats=True, out_dtype=out_dtype)
     mean, rstd = _jf.rowstats_finish(rowsum, rowsq, y1.shape[-1])     # one launch instead of eight torch operators
     return sh.fold(y1), sh.fold(q), sh.fold(s), sh.fold_vec(mean), sh.fold_vec(rstd)

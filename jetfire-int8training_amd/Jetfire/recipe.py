@@ -102,6 +102,7 @@ class AttentionIn(torch.autograd.Function):
     def forward(ctx, residual, qx, sx, w_qkv, ln_w, mean, rstd):
         qw, sw = weight_codes.get(w_qkv)
         ctx.wdtype = w_qkv.dtype          # the weight gradient leaves its GEMM in the parameter's type: no conversion kernel
+        ctx.res_dtype = residual.dtype    # and the residual's gradient leaves the add in the residual's type
         qx = _as_s8(qx)
         qn, sn, _ = int8_layernorm_forward(qx, sx, ln_w, mean, rstd, QB)
         qkv = int8_linear_forward(qn, sn, qw, sw, False, QB)
@@ -115,8 +116,50 @@ class AttentionIn(torch.autograd.Function):
         qg, sg = int8_quantize_concat([gq, gk, gv], QB, stochastic=True)
         qg, sg, gw = int8_linear_backward(qn, sn, qg, sg, None, qw, sw, QB, stochastic=True, wgrad_splitk=0, wgrad_dtype=ctx.wdtype)
         qg, sg, g_ln = int8_layernorm_backward(qx, sx, qg, sg, ln_w, QB, mean, rstd, stochastic=True)
-        res_g, qg, sg = int8_add_Ifp_Ig16_Ofp_Og(fpg.contiguous(), qg, sg, QB, stochastic=True)
+        res_g, qg, sg = int8_add_Ifp_Ig16_Ofp_Og(fpg.contiguous(), qg, sg, QB, stochastic=True, out_dtype=ctx.res_dtype)
         return res_g, _as_f8(qg), sg, gw, g_ln, None, None
+
+
+def _attention_out_forward(residual, y, w_proj):
+    """quantise -> output projection -> residual add with the next LayerNorm's statistics (qmodel.py:134-153); the sum is
+    float32 as in the reference.  Returns the outputs and what the backward needs."""
+    qw, sw = weight_codes.get(w_proj)
+    qy, sy = int8_quantize(y.contiguous(), QB)
+    qo, so = int8_linear_forward(qy, sy, qw, sw, True, QB)
+    fp, q, s, mean, rstd = int8_add_Ifp_Ig16_Ofp_Og_MeanVar(residual.contiguous(), qo, so, QB)
+    return (fp, q, s, mean, rstd), (qy, sy, qw, sw)
+
+
+def _attention_out_backward(saved, qg, sg, wdtype):
+    """gradient of the attention output (fp16 / bf16 for the attention kernel's backward) and of the projection's
+    weight (qmodel.py:155-171)"""
+    qy, sy, qw, sw = saved
+    return int8_linear_backward(qy, sy, qg, sg, None, qw, sw, QB, stochastic=True, dgrad_quantize=False, wgrad_splitk=0,
+                                wgrad_dtype=wdtype)
+
+
+def _mlp_forward(residual, qx, sx, w_fc, w_proj, ln_w, mean, rstd, out_dtype):
+    """LayerNorm -> fc + GELU -> proj -> residual add (qmodel.py:193-231).  out_dtype: type of the fp sum that leaves the
+    block (the reference casts it to bfloat16, qmodel.py:228; here the add kernel writes it in that type)."""
+    qw1, sw1 = weight_codes.get(w_fc)
+    qw2, sw2 = weight_codes.get(w_proj)
+    qn, sn, _ = int8_layernorm_forward(qx, sx, ln_w, mean, rstd, QB)
+    qh, sh, qa, sa = int8_linear_forward_gelu(qn, sn, qw1, sw1, QB)      # fc and its GELU in one kernel
+    qo, so = int8_linear_forward(qa, sa, qw2, sw2, True, QB)
+    outs = int8_add_Ifp_Ig16_Ofp_Og_MeanVar(residual.contiguous(), qo, so, QB, out_dtype=out_dtype)
+    return outs, (qx, sx, qn, sn, qh, sh, qa, sa, qw1, sw1, qw2, sw2, ln_w, mean, rstd)
+
+
+def _mlp_backward(saved, fpg, qg, sg, wdtype, res_dtype):
+    """(qmodel.py:233-267); the residual's gradient leaves the add in res_dtype"""
+    qx, sx, qn, sn, qh, sh, qa, sa, qw1, sw1, qw2, sw2, ln_w, mean, rstd = saved
+    # proj's backward with the GELU backward in the epilogue of its activation-gradient GEMM (one kernel for
+    # int8_linear_backward's dgrad + int8_gelu_backward, same bits)
+    qg, sg, gw2 = int8_linear_backward_gelu(qa, sa, qg, sg, qw2, sw2, qh, sh, QB, stochastic=True, wgrad_splitk=0, wgrad_dtype=wdtype)
+    qg, sg, gw1 = int8_linear_backward(qn, sn, qg, sg, None, qw1, sw1, QB, stochastic=True, wgrad_splitk=0, wgrad_dtype=wdtype)
+    qg, sg, g_ln = int8_layernorm_backward(qx, sx, qg, sg, ln_w, QB, mean, rstd, stochastic=True)
+    res_g, qg, sg = int8_add_Ifp_Ig16_Ofp_Og(fpg.contiguous(), qg, sg, QB, stochastic=True, out_dtype=res_dtype)
+    return res_g, qg, sg, gw1, gw2, g_ln
 
 
 class AttentionOut(torch.autograd.Function):
@@ -124,20 +167,15 @@ class AttentionOut(torch.autograd.Function):
 
     @staticmethod
     def forward(ctx, residual, y, w_proj):
-        qw, sw = weight_codes.get(w_proj)
         ctx.wdtype = w_proj.dtype
         ctx.set_materialize_grads(False)  # mean / rstd receive no gradient: None instead of two zero-filled tensors
-        qy, sy = int8_quantize(y.contiguous(), QB)
-        qo, so = int8_linear_forward(qy, sy, qw, sw, True, QB)
-        fp, q, s, mean, rstd = int8_add_Ifp_Ig16_Ofp_Og_MeanVar(residual.contiguous(), qo, so, QB)
-        ctx.save_for_backward(qy, sy, qw, sw)
+        (fp, q, s, mean, rstd), saved = _attention_out_forward(residual, y, w_proj)
+        ctx.save_for_backward(*saved)
         return fp, _as_f8(q), s, mean, rstd
 
     @staticmethod
     def backward(ctx, fpg, qg, sg, _m, _r):
-        qy, sy, qw, sw = ctx.saved_tensors
-        qg = _as_s8(qg)
-        g, gw = int8_linear_backward(qy, sy, qg, sg, None, qw, sw, QB, stochastic=True, dgrad_quantize=False, wgrad_splitk=0, wgrad_dtype=ctx.wdtype)
+        g, gw = _attention_out_backward(ctx.saved_tensors, _as_s8(qg), sg, ctx.wdtype)
         return fpg, g, gw
 
 
@@ -145,39 +183,53 @@ class MLPResidual(torch.autograd.Function):
     """LayerNorm -> fc -> GELU -> proj -> residual add, all on INT8 block tensors (qmodel.py:190-268)."""
 
     @staticmethod
-    def forward(ctx, residual, qx, sx, w_fc, w_proj, ln_w, mean, rstd):
-        qx = _as_s8(qx)
-        qw1, sw1 = weight_codes.get(w_fc)
-        qw2, sw2 = weight_codes.get(w_proj)
+    def forward(ctx, residual, qx, sx, w_fc, w_proj, ln_w, mean, rstd, out_dtype=torch.float32):
         ctx.wdtype = w_fc.dtype
+        ctx.res_dtype = residual.dtype
         ctx.set_materialize_grads(False)  # as in AttentionOut
-        qn, sn, _ = int8_layernorm_forward(qx, sx, ln_w, mean, rstd, QB)
-        qh, sh, qa, sa = int8_linear_forward_gelu(qn, sn, qw1, sw1, QB)      # fc and its GELU in one kernel
-        qo, so = int8_linear_forward(qa, sa, qw2, sw2, True, QB)
-        fp, q, s, mean2, rstd2 = int8_add_Ifp_Ig16_Ofp_Og_MeanVar(residual.contiguous(), qo, so, QB)
-        ctx.save_for_backward(qx, sx, qn, sn, qh, sh, qa, sa, qw1, sw1, qw2, sw2, ln_w, mean, rstd)
+        (fp, q, s, mean2, rstd2), saved = _mlp_forward(residual, _as_s8(qx), sx, w_fc, w_proj, ln_w, mean, rstd, out_dtype)
+        ctx.save_for_backward(*saved)
         return fp, _as_f8(q), s, mean2, rstd2
 
     @staticmethod
     def backward(ctx, fpg, qg, sg, _m, _r):
-        qx, sx, qn, sn, qh, sh, qa, sa, qw1, sw1, qw2, sw2, ln_w, mean, rstd = ctx.saved_tensors
-        qg = _as_s8(qg)
-        # proj's backward with the GELU backward in the epilogue of its activation-gradient GEMM (one kernel for
-        # int8_linear_backward's dgrad + int8_gelu_backward, same bits)
-        qg, sg, gw2 = int8_linear_backward_gelu(qa, sa, qg, sg, qw2, sw2, qh, sh, QB, stochastic=True, wgrad_splitk=0, wgrad_dtype=ctx.wdtype)
-        qg, sg, gw1 = int8_linear_backward(qn, sn, qg, sg, None, qw1, sw1, QB, stochastic=True, wgrad_splitk=0, wgrad_dtype=ctx.wdtype)
-        qg, sg, g_ln = int8_layernorm_backward(qx, sx, qg, sg, ln_w, QB, mean, rstd, stochastic=True)
-        res_g, qg, sg = int8_add_Ifp_Ig16_Ofp_Og(fpg.contiguous(), qg, sg, QB, stochastic=True)
-        return res_g, _as_f8(qg), sg, gw1, gw2, g_ln, None, None
+        res_g, qg, sg, gw1, gw2, g_ln = _mlp_backward(ctx.saved_tensors, fpg, _as_s8(qg), sg, ctx.wdtype, ctx.res_dtype)
+        return res_g, _as_f8(qg), sg, gw1, gw2, g_ln, None, None, None
+
+
+class AttentionOutMLP(torch.autograd.Function):
+    """AttentionOut followed by MLPResidual as ONE autograd node, same kernels and same bits.  The float32 sum between
+    the two halves and its gradient then never cross an autograd edge, so the gradient can leave its add kernel in the
+    type of the residual that receives it: with a bfloat16 stream between blocks (qmodel.py:228) the reference's
+    float32 gradient of that sum is cast by autograd when it reaches the bfloat16 residual, a pass of its own."""
+
+    @staticmethod
+    def forward(ctx, residual, y, w_attn_proj, w_fc, w_mlp_proj, ln_w, out_dtype):
+        ctx.wdtype = w_fc.dtype
+        ctx.res_dtype = residual.dtype
+        ctx.set_materialize_grads(False)
+        (mid, q, s, mean, rstd), saved_a = _attention_out_forward(residual, y, w_attn_proj)
+        (fp, q, s, mean2, rstd2), saved_m = _mlp_forward(mid, q, s, w_fc, w_mlp_proj, ln_w, mean, rstd, out_dtype)
+        ctx.n_a = len(saved_a)
+        ctx.save_for_backward(*saved_a, *saved_m)
+        return fp, _as_f8(q), s, mean2, rstd2
+
+    @staticmethod
+    def backward(ctx, fpg, qg, sg, _m, _r):
+        saved = ctx.saved_tensors
+        res_g, qg, sg, gw1, gw2, g_ln = _mlp_backward(saved[ctx.n_a:], fpg, _as_s8(qg), sg, ctx.wdtype, ctx.res_dtype)
+        g, gwp = _attention_out_backward(saved[:ctx.n_a], qg, sg, ctx.wdtype)
+        return res_g, g, gwp, gw1, gw2, g_ln, None
 
 
 class QBlock(nn.Module):
-    """One pre-LayerNorm transformer block (causal self-attention + MLP) on the INT8 data flow."""
+    """One pre-LayerNorm transformer block (causal self-attention + MLP) on the INT8 data flow.  out_dtype: type of the
+    fp residual that leaves the block (float32, or the reference's bfloat16, qmodel.py:228)."""
 
-    def __init__(self, n_embd, n_head):
+    def __init__(self, n_embd, n_head, out_dtype=torch.float32):
         super().__init__()
         assert n_embd % n_head == 0 and n_embd % QB == 0
-        self.n_embd, self.n_head = n_embd, n_head
+        self.n_embd, self.n_head, self.out_dtype = n_embd, n_head, out_dtype
         self.ln_1 = nn.Parameter(torch.ones(n_embd))
         self.ln_2 = nn.Parameter(torch.ones(n_embd))
         self.w_qkv = nn.Parameter(torch.randn(3 * n_embd, n_embd) * 0.02)
@@ -190,17 +242,17 @@ class QBlock(nn.Module):
         res, q, k, v = AttentionIn.apply(x, qx, sx, self.w_qkv, self.ln_1, mean, rstd)
         q, k, v = (t.view(B, T, self.n_head, C // self.n_head).transpose(1, 2) for t in (q, k, v))
         y = F.scaled_dot_product_attention(q, k, v, is_causal=True).transpose(1, 2).contiguous().view(B, T, C)
-        x, qx, sx, mean, rstd = AttentionOut.apply(res, y, self.w_attn_proj)
-        return MLPResidual.apply(x, qx, sx, self.w_fc, self.w_mlp_proj, self.ln_2, mean, rstd)
+        return AttentionOutMLP.apply(res, y, self.w_attn_proj, self.w_fc, self.w_mlp_proj, self.ln_2, self.out_dtype)
 
 
 class QStack(nn.Module):
     """A stack of QBlocks between StreamBegin and StreamEnd: fp in, fp out (qmodel.py:418-446 without the
-    embedding and the language-model head)."""
+    embedding and the language-model head).  stream_dtype: type of the fp residual between blocks and of the output
+    (the reference: bfloat16, qmodel.py:228); the input keeps its own type."""
 
-    def __init__(self, n_layer, n_embd, n_head):
+    def __init__(self, n_layer, n_embd, n_head, stream_dtype=torch.float32):
         super().__init__()
-        self.blocks = nn.ModuleList(QBlock(n_embd, n_head) for _ in range(n_layer))
+        self.blocks = nn.ModuleList(QBlock(n_embd, n_head, stream_dtype) for _ in range(n_layer))
 
     def forward(self, x):
         x, qx, sx = StreamBegin.apply(x)

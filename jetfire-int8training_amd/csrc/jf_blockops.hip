@@ -839,9 +839,9 @@ __global__ __launch_bounds__(1024) void layernorm_bwd_colsum_finish_kernel(const
 // 17.0 against 22.9 us; the mapping of the loads makes no difference).
 // rowsum / rowsq: [C/32][R] (a wave stores the 32 consecutive rows of its block).
 constexpr int ADD_PITCH = QB + 4;                  // floats per patch row (16-byte aligned rows, rotated over the banks)
-template <typename T, typename ST>
+template <typename T, typename ST, typename OT>
 __global__ __launch_bounds__(NT) void add_kernel(const T *x1, const int8_t *q2, const ST *s2, int R, int C,
-                                                 int rounding, uint64_t seed, uint64_t offset, float *y1, int8_t *q,
+                                                 int rounding, uint64_t seed, uint64_t offset, OT *y1, int8_t *q,
                                                  ST *s, float *rowsum, float *rowsq)
 {
     __shared__ __attribute__((aligned(16))) float ypatch_all[WPB][QB * ADD_PITCH];
@@ -861,11 +861,24 @@ __global__ __launch_bounds__(NT) void add_kernel(const T *x1, const int8_t *q2, 
             __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
             __builtin_amdgcn_wave_barrier();
             __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
-            float *dst = y1 + (size_t)(pos.rb * QB + (lane >> 3)) * C + pos.cb * QB + (lane & 7) * 4;
+            if (sizeof(OT) == 4) {
+                float *dst = reinterpret_cast<float *>(y1) + (size_t)(pos.rb * QB + (lane >> 3)) * C + pos.cb * QB + (lane & 7) * 4;
 #pragma unroll
-            for (int i = 0; i < 4; ++i)
-                *reinterpret_cast<v4f *>(dst + (size_t)(8 * i) * C) =
-                    *reinterpret_cast<const v4f *>(ypatch + (8 * i + (lane >> 3)) * ADD_PITCH + (lane & 7) * 4);
+                for (int i = 0; i < 4; ++i)
+                    *reinterpret_cast<v4f *>(dst + (size_t)(8 * i) * C) =
+                        *reinterpret_cast<const v4f *>(ypatch + (8 * i + (lane >> 3)) * ADD_PITCH + (lane & 7) * 4);
+            } else {
+                // 16-bit sum (rounded to nearest even from the fp32 sum): a row of the block is 64 bytes, a store
+                // instruction writes 16 whole rows (lane l: row 16i + l/4, columns 8*(l%4) .. +7)
+                OT *dst = y1 + (size_t)(pos.rb * QB + (lane >> 2)) * C + pos.cb * QB + (lane & 3) * 8;
+#pragma unroll
+                for (int i = 0; i < 2; ++i) {
+                    const float *r = ypatch + (16 * i + (lane >> 2)) * ADD_PITCH + (lane & 3) * 8;
+                    const v4f lo = *reinterpret_cast<const v4f *>(r), hi = *reinterpret_cast<const v4f *>(r + 4);
+                    OT h[8] = {(OT)lo.x, (OT)lo.y, (OT)lo.z, (OT)lo.w, (OT)hi.x, (OT)hi.y, (OT)hi.z, (OT)hi.w};
+                    *reinterpret_cast<v4i *>(dst + (size_t)(16 * i) * C) = *reinterpret_cast<v4i *>(h);
+                }
+            }
             __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
             __builtin_amdgcn_wave_barrier();                       // the patch may be rewritten
         }
@@ -1201,7 +1214,7 @@ int jf_gelu_bwd(const int8_t *qx, const void *sx, const int8_t *qg, const void *
 }
 
 int jf_add(const void *x1, int x1_dtype, const int8_t *q2, const void *s2, int R, int C, int scale_dtype, int rounding,
-           uint64_t seed, uint64_t offset, float *y1, int8_t *q, void *s, float *rowsum, float *rowsq,
+           uint64_t seed, uint64_t offset, void *y1, int y1_dtype, int8_t *q, void *s, float *rowsum, float *rowsq,
            jf_stream_t stream)
 {
     int rc = check_block_tensor(q2, s2, R, C, scale_dtype);
@@ -1209,21 +1222,29 @@ int jf_add(const void *x1, int x1_dtype, const int8_t *q2, const void *s2, int R
     if (!x1 || !y1 || !q || !s) return JF_ERR_NULL;
     if ((rowsum == nullptr) != (rowsq == nullptr)) return JF_ERR_NULL;
     if (!rounding_ok(rounding) || x1_dtype < JF_FP_F16 || x1_dtype > JF_FP_BF16) return JF_ERR_ENUM;
+    if (y1_dtype < JF_FP_F16 || y1_dtype > JF_FP_BF16) return JF_ERR_ENUM;
     if (!aligned16(x1) || !aligned16(y1) || !aligned16(q)) return JF_ERR_ALIGN;
     hipStream_t st = (hipStream_t)stream;
     const int grid = grid_for_blocks(R, C);
-#define JF_ADD(T, ST)                                                                                             \
-    JF_LAUNCH((add_kernel<T, ST>), grid, 0, st, (const T *)x1, q2, (const ST *)s2, R, C, rounding, seed, offset, y1, q, \
-              (ST *)s, rowsum, rowsq)
+#define JF_ADD(T, ST, OT)                                                                                         \
+    JF_LAUNCH((add_kernel<T, ST, OT>), grid, 0, st, (const T *)x1, q2, (const ST *)s2, R, C, rounding, seed, offset, \
+              (OT *)y1, q, (ST *)s, rowsum, rowsq)
+#define JF_ADD_OUT(T, ST)                                                                                         \
+    do {                                                                                                          \
+        if (y1_dtype == JF_FP_F32) JF_ADD(T, ST, float);                                                          \
+        if (y1_dtype == JF_FP_F16) JF_ADD(T, ST, half_t);                                                         \
+        JF_ADD(T, ST, __bf16);                                                                                    \
+    } while (0)
     if (scale_dtype == JF_SCALE_F16) {
-        if (x1_dtype == JF_FP_F32) JF_ADD(float, half_t);
-        if (x1_dtype == JF_FP_F16) JF_ADD(half_t, half_t);
-        JF_ADD(__bf16, half_t);
+        if (x1_dtype == JF_FP_F32) JF_ADD_OUT(float, half_t);
+        if (x1_dtype == JF_FP_F16) JF_ADD_OUT(half_t, half_t);
+        JF_ADD_OUT(__bf16, half_t);
     } else {
-        if (x1_dtype == JF_FP_F32) JF_ADD(float, float);
-        if (x1_dtype == JF_FP_F16) JF_ADD(half_t, float);
-        JF_ADD(__bf16, float);
+        if (x1_dtype == JF_FP_F32) JF_ADD_OUT(float, float);
+        if (x1_dtype == JF_FP_F16) JF_ADD_OUT(half_t, float);
+        JF_ADD_OUT(__bf16, float);
     }
+#undef JF_ADD_OUT
 #undef JF_ADD
 }
 

@@ -71,7 +71,7 @@ def lib():
         L.jf_layernorm_bwd.argtypes = [_p, _p, _p, _p, _p, _p, _p, _i, _i, _i, _i, _u64, _u64, _p, _p, _p, _p, _p, _sz, _p]
         L.jf_gelu_fwd.argtypes = [_p, _p, _i, _i, _i, _i, _f, _p, _p, _p]
         L.jf_gelu_bwd.argtypes = [_p, _p, _p, _p, _i, _i, _i, _i, _i, _u64, _u64, _p, _p, _p]
-        L.jf_add.argtypes = [_p, _i, _p, _p, _i, _i, _i, _i, _u64, _u64, _p, _p, _p, _p, _p, _p]
+        L.jf_add.argtypes = [_p, _i, _p, _p, _i, _i, _i, _i, _u64, _u64, _p, _i, _p, _p, _p, _p, _p]
         L.jf_wall_clock_khz.argtypes = []
         L.jf_calibrate.argtypes = [_i, _i, _i, _i, _i, _i, _p, _p, _p]
         missing = [name for name in EXPORTS if not hasattr(L, name)]
@@ -485,19 +485,23 @@ def gelu_bwd(qx, sx, qg, sg, approx=GELU_ERF, rounding=ROUND_NEAREST, seed=None,
     return qy, sy
 
 
-def add(x1, q2, s2, rounding=ROUND_TRUNC, with_stats=False, seed=None, offset=None):
+def add(x1, q2, s2, rounding=ROUND_TRUNC, with_stats=False, seed=None, offset=None, out_dtype=torch.float32):
+    """y = x1 + q2*s2 (fp32), returned in `out_dtype`, and its block quantisation; the quantisation and the row
+    statistics are taken from the fp32 sum whatever `out_dtype` is."""
     R, Cc, code = _block_tensor(q2, s2, "x2")
     _need(x1, None, "x1")
     if x1.dtype not in _FP_CODE or tuple(x1.shape) != (R, Cc):
         raise RuntimeError("x1 must be a float tensor of the same shape as x2")
+    if out_dtype not in _FP_CODE:
+        raise RuntimeError("out_dtype must be float32, float16 or bfloat16")
     seed, offset = _rng(rounding, R * Cc, seed, offset, x1.device)
-    y1 = torch.empty((R, Cc), dtype=torch.float32, device=x1.device)
+    y1 = torch.empty((R, Cc), dtype=out_dtype, device=x1.device)
     q = torch.empty_like(q2)
     s = torch.empty_like(s2)
     rs = torch.empty((Cc // QB, R), dtype=torch.float32, device=x1.device) if with_stats else None   # part-major
     rq = torch.empty((Cc // QB, R), dtype=torch.float32, device=x1.device) if with_stats else None
     check(lib().jf_add(_ptr(x1), _FP_CODE[x1.dtype], _ptr(q2), _ptr(s2), R, Cc, code, rounding, seed, offset,
-                       _ptr(y1), _ptr(q), _ptr(s), _ptr(rs), _ptr(rq), _stream()))
+                       _ptr(y1), _FP_CODE[out_dtype], _ptr(q), _ptr(s), _ptr(rs), _ptr(rq), _stream()))
     return (y1, q, s, rs, rq) if with_stats else (y1, q, s)
 
 

@@ -235,6 +235,30 @@ def test_add(jf, oracle, dtype, mode):
     assert np.allclose(m, wy.mean(-1), atol=1e-5) and np.allclose(rstd.cpu().numpy(), 1 / np.sqrt(wy.var(-1)), rtol=1e-4)
 
 
+@pytest.mark.parametrize("out_dtype", [torch.bfloat16, torch.float16])
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
+def test_add_with_a_16_bit_sum(jf, oracle, dtype, out_dtype):
+    """The sum may leave the kernel already cast (the reference casts it afterwards, qmodel.py:228): it is the fp32 sum
+    rounded to nearest even, and codes, scales and row statistics are those of the fp32 sum."""
+    rng = np.random.default_rng(32)
+    R, C = 64, 224
+    x1 = torch.from_numpy(rng.standard_normal((R, C)).astype(np.float32) * 3).to(dtype)
+    q2, s2 = block_tensor(oracle, rng, R, C, 0.5)
+    y32, q32, s32, rs32, rq32 = jf.add(x1.cuda(), dev(q2), dev(s2), ROUND["stochastic"], with_stats=True, seed=9, offset=2)
+    y16, q, s, rs, rq = jf.add(x1.cuda(), dev(q2), dev(s2), ROUND["stochastic"], with_stats=True, seed=9, offset=2,
+                               out_dtype=out_dtype)
+    wy, wq, ws, wrs, wrq = oracle.add(x1.float().numpy(), q2, s2.astype(np.float32), True, 9, 2, False, True, "f16")
+    assert y16.dtype == out_dtype
+    assert torch.equal(y16.cpu(), torch.from_numpy(wy).to(out_dtype))      # torch's cast rounds to nearest even
+    assert torch.equal(y16, y32.to(out_dtype))
+    same(q, wq, "codes")
+    same(s, ws, "scales")
+    same(rs, wrs, "row sums")
+    same(rq, wrq, "row square sums")
+    with pytest.raises(RuntimeError):
+        jf.add(x1.cuda(), dev(q2), dev(s2), out_dtype=torch.float64)
+
+
 def test_full_size_nonlinear_properties(jf, oracle):
     """benchmark configuration 4 sizes.  Checked bit-exactly against the oracle on row slabs (the kernels are
     block-local, so a slab of the input is a complete problem), and by size-independent properties."""

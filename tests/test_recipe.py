@@ -131,6 +131,67 @@ def test_twelve_layer_stack_matches_fp32_reference():
         assert c > 0.997 - 0.0003 * (L - 1 - layer), (layer, c)
 
 
+def test_bfloat16_stream_between_blocks():
+    """The reference casts the fp sum that leaves a block to bfloat16 (qmodel.py:228); here the add kernels write it (and
+    the gradient that flows back into a bfloat16 residual) in that type.  Input and its gradient keep float32; the INT8
+    stream is quantised from the float32 sums, so the result is as close to the fp32 stack as with a float32 stream up to
+    the rounding of the residual."""
+    from recipe import QStack
+    torch.manual_seed(11)
+    L, B, T, C, H = 3, 2, 128, 256, 4
+    model = QStack(L, C, H, stream_dtype=torch.bfloat16).cuda()
+    x = torch.randn(B, T, C, device="cuda", requires_grad=True)
+    w = torch.randn(B, T, C, device="cuda")
+    out = model(x)
+    assert out.dtype == torch.bfloat16
+    out.backward(w.to(torch.bfloat16))
+    assert x.grad.dtype == torch.float32
+    got = {n: p.grad.clone() for n, p in model.named_parameters()}
+    gx = x.grad.clone()
+    for p in model.parameters():
+        p.grad = None
+    x2 = x.detach().clone().requires_grad_(True)
+    h = x2
+    for blk in model.blocks:
+        h = ref_block(h, blk)
+    (h * w).sum().backward()
+    print("bf16 stream: output / input-gradient cosine:", round(cos(out, h), 5), round(cos(gx, x2.grad), 5), flush=True)
+    assert cos(out, h) > 0.9995
+    assert cos(gx, x2.grad) > 0.99
+    for n, p in model.named_parameters():
+        assert got[n].dtype == p.dtype and torch.isfinite(got[n]).all()
+        assert cos(got[n], p.grad) > 0.99, (n, cos(got[n], p.grad))
+
+
+def test_merged_node_equals_the_two_functions():
+    """AttentionOutMLP is AttentionOut followed by MLPResidual: same kernels in the same order, so with the same noise
+    offsets the outputs and every gradient are the same bits."""
+    import recipe
+    torch.manual_seed(5)
+    B, T, C = 2, 64, 128
+    blk = recipe.QBlock(C, 4).cuda()
+    res = torch.randn(B, T, C, device="cuda")
+    y = torch.randn(B, T, C, device="cuda").half()
+    gout = torch.randn(B, T, C, device="cuda")
+
+    def run(merged):
+        torch.manual_seed(123)                                    # rewinds the stochastic-rounding stream
+        r, yy = res.clone().requires_grad_(True), y.clone().requires_grad_(True)
+        for p in blk.parameters():
+            p.grad = None
+        if merged:
+            fp, q, s, m, rs = recipe.AttentionOutMLP.apply(r, yy, blk.w_attn_proj, blk.w_fc, blk.w_mlp_proj, blk.ln_2, torch.float32)
+        else:
+            a = recipe.AttentionOut.apply(r, yy, blk.w_attn_proj)
+            fp, q, s, m, rs = recipe.MLPResidual.apply(*a[:3], blk.w_fc, blk.w_mlp_proj, blk.ln_2, a[3], a[4])
+        out = recipe.StreamEnd.apply(fp, q, s)
+        out.backward(gout)
+        return [fp.detach(), q.view(torch.int8), s, m, rs, r.grad, yy.grad, blk.w_attn_proj.grad, blk.w_fc.grad,
+                blk.w_mlp_proj.grad, blk.ln_2.grad]
+    for i, (a, b) in enumerate(zip(run(True), run(False))):
+        assert torch.equal(a, b), i
+
+
 def test_small_stack_trains():
     from recipe import QStack
     torch.manual_seed(1)
