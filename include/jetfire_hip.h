@@ -217,6 +217,20 @@ int jf_layernorm_bwd(const int8_t *qx, const void *sx, const int8_t *qg, const v
                      int8_t *qdx, void *sdx, float *dgamma, float *dbeta,
                      void *workspace, size_t workspace_bytes, jf_stream_t stream);
 
+/* jf_layernorm_bwd followed by jf_add(x1, dx codes, dx scales) in one kernel, for rows of up to 2048 columns
+ * (JF_ERR_SHAPE beyond: make the two calls): dx is requantised with (rounding, seed, offset) exactly as jf_layernorm_bwd
+ * does, read back as codes x the stored scale, added to x1, and the sum (y1, in y1_dtype) and its block quantisation
+ * (q, s; add_rounding, add_seed, add_offset) are what is written -- bit for bit what the two calls write, without dx's
+ * round trip through memory.  dx itself is not stored.  Workspace as for jf_layernorm_bwd.
+ * Replaces the pair int8_layernorm_backward + int8_add_Ifp_Ig16_Ofp_Og of the reference's recipe
+ * (INT8_GPT2/qmodel.py:125-128 and :258-261; Jetfire/Nonlinear/layernorm.py:467-526, add.py:164-211). */
+int jf_layernorm_bwd_add(const int8_t *qx, const void *sx, const int8_t *qg, const void *sg,
+                         const float *gamma, const float *mean, const float *rstd, int R, int C,
+                         int scale_dtype, int rounding, uint64_t seed, uint64_t offset,
+                         const void *x1, int x1_dtype, int add_rounding, uint64_t add_seed, uint64_t add_offset,
+                         void *y1, int y1_dtype, int8_t *q, void *s, float *dgamma, float *dbeta,
+                         void *workspace, size_t workspace_bytes, jf_stream_t stream);
+
 /* dequant -> GELU -> requant (amax_eps is added to the block amax: 5e-5 in the reference).
  * Replaces int8_gelu_forward (Jetfire/Nonlinear/gelu_fwd.py:128-162). */
 int jf_gelu_fwd(const int8_t *q, const void *s, int R, int C, int scale_dtype, int approx,

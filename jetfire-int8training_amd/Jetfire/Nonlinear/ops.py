@@ -134,6 +134,21 @@ def int8_layernorm_backward(x, sx, g, sg, w, QB, m, v, stochastic=False, eps=1e-
     return out + (db.to(w.dtype),) if return_dbias else out
 
 
+def int8_layernorm_backward_add(x, sx, g, sg, w, QB, m, v, x1, stochastic=False, add_stochastic=False, add_rounding="trunc",
+                                out_dtype=torch.float32, return_dbias=False):
+    """int8_layernorm_backward followed by int8_add_Ifp_Ig16_Ofp_Og(x1, dx, s_dx, ...) (the pair the reference's recipe
+    calls back to back, qmodel.py:125-128, 258-261) as one kernel for rows of up to 2048 columns, same bits.
+    Returns (y1, y2, s_y2, dweight[, dbias])."""
+    _check_qb(QB)
+    sh = _Shape(x)
+    rounding = _jf.ROUND_STOCHASTIC if stochastic else _jf.ROUND_NEAREST
+    y1, q, s, dg, db = _jf.layernorm_bwd_add(sh.flat(x), sh.flat(sx), sh.flat(g), sh.flat(sg), _f32(w), _f32(m), _f32(v),
+                                             sh.flat(x1), rounding, _add_rounding(add_stochastic, add_rounding),
+                                             want_dbeta=return_dbias, out_dtype=out_dtype)
+    out = (sh.fold(y1), sh.fold(q), sh.fold(s), dg.to(w.dtype))
+    return out + (db.to(w.dtype),) if return_dbias else out
+
+
 def int8_gelu_forward(x, s_x, QB, approximate="none"):
     """dequant -> GELU -> requant.  'none' = erf form with SCALE_MIN_THRES added to the block absmax
     (reference: gelu_fwd.py:81,90); 'tanh' = tanh approximation, no threshold."""

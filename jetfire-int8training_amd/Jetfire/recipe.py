@@ -20,8 +20,8 @@ import torch.nn as nn
 import torch.nn.functional as F
 
 from Linear import int8_linear_backward, int8_linear_backward_gelu, int8_linear_forward, int8_linear_forward_gelu
-from Nonlinear import (int8_add_Ifp_Ig16_Ofp_Og, int8_add_Ifp_Ig16_Ofp_Og_MeanVar, int8_gelu_backward,
-                       int8_layernorm_backward, int8_layernorm_forward, int8_quantize, int8_quantize_concat)
+from Nonlinear import (int8_add_Ifp_Ig16_Ofp_Og_MeanVar, int8_layernorm_backward_add, int8_layernorm_forward, int8_quantize,
+                       int8_quantize_concat)
 
 QB = 32
 _F8 = torch.float8_e4m3fn
@@ -115,8 +115,9 @@ class AttentionIn(torch.autograd.Function):
         qx, sx, qn, sn, qw, sw, ln_w, mean, rstd = ctx.saved_tensors
         qg, sg = int8_quantize_concat([gq, gk, gv], QB, stochastic=True)
         qg, sg, gw = int8_linear_backward(qn, sn, qg, sg, None, qw, sw, QB, stochastic=True, wgrad_splitk=0, wgrad_dtype=ctx.wdtype)
-        qg, sg, g_ln = int8_layernorm_backward(qx, sx, qg, sg, ln_w, QB, mean, rstd, stochastic=True)
-        res_g, qg, sg = int8_add_Ifp_Ig16_Ofp_Og(fpg.contiguous(), qg, sg, QB, stochastic=True, out_dtype=ctx.res_dtype)
+        # LayerNorm backward and the residual add behind it (qmodel.py:125-128) as one kernel, same bits
+        res_g, qg, sg, g_ln = int8_layernorm_backward_add(qx, sx, qg, sg, ln_w, QB, mean, rstd, fpg.contiguous(), stochastic=True,
+                                                          add_stochastic=True, out_dtype=ctx.res_dtype)
         return res_g, _as_f8(qg), sg, gw, g_ln, None, None
 
 
@@ -157,8 +158,9 @@ def _mlp_backward(saved, fpg, qg, sg, wdtype, res_dtype):
     # int8_linear_backward's dgrad + int8_gelu_backward, same bits)
     qg, sg, gw2 = int8_linear_backward_gelu(qa, sa, qg, sg, qw2, sw2, qh, sh, QB, stochastic=True, wgrad_splitk=0, wgrad_dtype=wdtype)
     qg, sg, gw1 = int8_linear_backward(qn, sn, qg, sg, None, qw1, sw1, QB, stochastic=True, wgrad_splitk=0, wgrad_dtype=wdtype)
-    qg, sg, g_ln = int8_layernorm_backward(qx, sx, qg, sg, ln_w, QB, mean, rstd, stochastic=True)
-    res_g, qg, sg = int8_add_Ifp_Ig16_Ofp_Og(fpg.contiguous(), qg, sg, QB, stochastic=True, out_dtype=res_dtype)
+    # LayerNorm backward and the residual add behind it (qmodel.py:258-261) as one kernel, same bits
+    res_g, qg, sg, g_ln = int8_layernorm_backward_add(qx, sx, qg, sg, ln_w, QB, mean, rstd, fpg.contiguous(), stochastic=True,
+                                                      add_stochastic=True, out_dtype=res_dtype)
     return res_g, qg, sg, gw1, gw2, g_ln
 
 

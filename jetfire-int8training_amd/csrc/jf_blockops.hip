@@ -460,6 +460,53 @@ __device__ __forceinline__ float colsum16_over_rows(const float (&v)[16], int la
     return t;
 }
 
+// A block's fp32 values leave through a wave-private LDS patch: in the layout the arithmetic uses (lane l: row l/2, 16
+// columns) a store instruction would write 64 separate 16-byte pieces; read back as "lane l: row 8i + l/8, columns
+// 4*(l%8) .. +3" each of the four store instructions writes 8 whole 128-byte rows of the block (measured on an fp32 copy
+// of 8192x1600: 17.0 against 22.9 us; the mapping of the loads makes no difference).  16-bit outputs (rounded to nearest
+// even): a row of the block is 64 bytes and a store instruction writes 16 whole rows (lane l: row 16i + l/4, columns
+// 8*(l%4) .. +7).  `out` points at the block's first element, ld = elements per row.
+constexpr int ADD_PITCH = QB + 4;                  // floats per patch row (16-byte aligned rows, rotated over the banks)
+template <typename OT>
+__device__ __forceinline__ void store_block_rows(float *ypatch, const float (&a)[16], OT *out, int ld, int lane)
+{
+    float *w = ypatch + (lane >> 1) * ADD_PITCH + (lane & 1) * 16;
+#pragma unroll
+    for (int k = 0; k < 4; ++k) *reinterpret_cast<v4f *>(w + 4 * k) = v4f{a[4 * k], a[4 * k + 1], a[4 * k + 2], a[4 * k + 3]};
+    __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
+    __builtin_amdgcn_wave_barrier();
+    __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
+    if (sizeof(OT) == 4) {
+        float *dst = reinterpret_cast<float *>(out) + (size_t)(lane >> 3) * ld + (lane & 7) * 4;
+#pragma unroll
+        for (int i = 0; i < 4; ++i)
+            *reinterpret_cast<v4f *>(dst + (size_t)(8 * i) * ld) =
+                *reinterpret_cast<const v4f *>(ypatch + (8 * i + (lane >> 3)) * ADD_PITCH + (lane & 7) * 4);
+    } else {
+        OT *dst = out + (size_t)(lane >> 2) * ld + (lane & 3) * 8;
+#pragma unroll
+        for (int i = 0; i < 2; ++i) {
+            const float *r = ypatch + (16 * i + (lane >> 2)) * ADD_PITCH + (lane & 3) * 8;
+            const v4f lo = *reinterpret_cast<const v4f *>(r), hi = *reinterpret_cast<const v4f *>(r + 4);
+            OT h[8] = {(OT)lo.x, (OT)lo.y, (OT)lo.z, (OT)lo.w, (OT)hi.x, (OT)hi.y, (OT)hi.z, (OT)hi.w};
+            *reinterpret_cast<v4i *>(dst + (size_t)(16 * i) * ld) = *reinterpret_cast<v4i *>(h);
+        }
+    }
+    __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
+    __builtin_amdgcn_wave_barrier();                               // the patch may be rewritten
+}
+
+// The residual add that follows a LayerNorm backward in the recipe, for the kernel that does both (ADD instantiations of
+// layernorm_bwd_strip_kernel): y = x1 + dx as a reader of the stored dx would form it, and y's block quantisation.
+struct LnAddArgs {
+    const void *x1;       // [R, C] x1_dtype
+    void *y1;             // [R, C] y1_dtype
+    int8_t *q;            // [R, C]
+    void *s;              // [R/32, C/32] ST
+    int x1_dtype, y1_dtype, rounding;
+    uint64_t seed, offset;
+};
+
 // ------------------------------------------------------------------------------------------------
 // LayerNorm backward over full rows (layernorm.py:197-428; the reference reduces over its 128-column tile only).
 // Arithmetic (this library's definition, restated by the CPU checker):
@@ -686,18 +733,24 @@ __global__ __launch_bounds__(WAVE * LNB_DX_WAVES) void layernorm_bwd_dx_kernel(
 // j + 8, ..., the tree over T_0..T_7), and phase 2 converts the codes again (cheaper than keeping 32 floats per block
 // alive), forms dx and requantises it.  Same arithmetic, bit for bit, as the two-launch form above, which stays for
 // wider rows.
+// ADD: the residual add that follows in the recipe (add.py:164-211) happens here as well: dx is requantised exactly as
+// without ADD, but instead of being stored it is dequantised again as a reader of the stored tensor would (codes x the
+// scale rounded to ST), added to x1, and the sum and its own block quantisation are what leaves -- the same bits as this
+// kernel without ADD followed by add_kernel, without dx's round trip through memory and the second launch.
 constexpr int LNS_WAVES = 16, LNS_BPW = 4;
-template <typename ST, bool WANT_DW>
+constexpr int LNS_PATCH_ADD = QB * ADD_PITCH;      // floats per wave: the sum's patch, also used for the column sums
+static_assert(LNS_PATCH_ADD >= COLSUM_PATCH, "one patch per wave serves both");
+template <typename ST, bool WANT_DW, bool ADD>
 __global__ __launch_bounds__(WAVE * LNS_WAVES) void layernorm_bwd_strip_kernel(
     const int8_t *qx, const ST *sx, const int8_t *qg, const ST *sg, const float *gamma, const float *mean,
     const float *rstd, int R, int C, int rounding, uint64_t seed, uint64_t offset, int8_t *qdx, ST *sdx, float *pdg,
-    float *pdb)
+    float *pdb, LnAddArgs ad)
 {
     extern __shared__ __attribute__((aligned(16))) float lds_f[];  // gamma[C], part[2][C/32][32], T[2][8][32], c[2][32], patches
     const int lane = threadIdx.x & 63, wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
     const int SC = C / QB, rb = blockIdx.x;
     float *gl = lds_f, *part = gl + C, *tj = part + 2 * SC * QB, *cs = tj + 2 * 8 * QB;
-    float *cpatch = cs + 2 * QB + wave * COLSUM_PATCH;             // (only with WANT_DW)
+    float *cpatch = cs + 2 * QB + wave * (ADD ? LNS_PATCH_ADD : COLSUM_PATCH);   // (only with WANT_DW or ADD)
     const int row = rb * QB + (lane >> 1);
     v4i cx[LNS_BPW], cg[LNS_BPW];
     float scx[LNS_BPW], scg[LNS_BPW];
@@ -782,6 +835,16 @@ __global__ __launch_bounds__(WAVE * LNS_WAVES) void layernorm_bwd_strip_kernel(
         const size_t e0 = (size_t)row * C + col;
         const float a = scx[I] * rs, sgk = scg[I];
         float x[16], g[16], w[16];
+        v4i raw[4];                                                // (ADD) the lane's 16 values of x1 as they lie in memory
+        if (ADD) {
+            if (ad.x1_dtype == JF_FP_F32) {
+#pragma unroll
+                for (int k = 0; k < 4; ++k) raw[k] = reinterpret_cast<const v4i *>(reinterpret_cast<const float *>(ad.x1) + e0)[k];
+            } else {
+#pragma unroll
+                for (int k = 0; k < 2; ++k) raw[k] = reinterpret_cast<const v4i *>(reinterpret_cast<const uint16_t *>(ad.x1) + e0)[k];
+            }
+        }
         Load16<float>::run(gl + col, w);
         // (opaque copies: otherwise the optimiser keeps phase 1's 32 converted values per block alive across the barriers,
         // in registers this kernel does not have)
@@ -797,8 +860,35 @@ __global__ __launch_bounds__(WAVE * LNS_WAVES) void layernorm_bwd_strip_kernel(
         }
         float so;
         const v4i out = quantize16(x, 0.0f, rounding, seed, offset, e0, &so);
-        *reinterpret_cast<v4i *>(qdx + e0) = out;
-        if (lane == 0) store_scale(sdx, rb * SC + cb, so);
+        if (!ADD) {
+            *reinterpret_cast<v4i *>(qdx + e0) = out;
+            if (lane == 0) store_scale(sdx, rb * SC + cb, so);
+        } else {
+            float y[16];
+            unpack16(out, (float)(ST)so, x);                       // dx as stored
+            if (ad.x1_dtype == JF_FP_F32) {
+#pragma unroll
+                for (int k = 0; k < 16; ++k) y[k] = __int_as_float(raw[k >> 2][k & 3]);
+            } else if (ad.x1_dtype == JF_FP_F16) {
+#pragma unroll
+                for (int k = 0; k < 16; ++k)
+                    y[k] = (float)__builtin_bit_cast(half_t, (uint16_t)((uint32_t)raw[k >> 3][(k >> 1) & 3] >> (16 * (k & 1))));
+            } else {
+#pragma unroll
+                for (int k = 0; k < 16; ++k)
+                    y[k] = __uint_as_float(((uint32_t)raw[k >> 3][(k >> 1) & 3] >> (16 * (k & 1))) << 16);
+            }
+#pragma unroll
+            for (int k = 0; k < 16; ++k) y[k] = y[k] + x[k];
+            const size_t b0 = (size_t)rb * QB * C + cb * QB;       // the block's first element
+            if (ad.y1_dtype == JF_FP_F32) store_block_rows(cpatch, y, reinterpret_cast<float *>(ad.y1) + b0, C, lane);
+            else if (ad.y1_dtype == JF_FP_F16) store_block_rows(cpatch, y, reinterpret_cast<half_t *>(ad.y1) + b0, C, lane);
+            else store_block_rows(cpatch, y, reinterpret_cast<__bf16 *>(ad.y1) + b0, C, lane);
+            float s2;
+            const v4i c2 = quantize16(y, 0.0f, ad.rounding, ad.seed, ad.offset, e0, &s2);
+            *reinterpret_cast<v4i *>(ad.q + e0) = c2;
+            if (lane == 0) store_scale(reinterpret_cast<ST *>(ad.s), rb * SC + cb, s2);
+        }
         __builtin_amdgcn_sched_barrier(0);
     });
 }
@@ -833,12 +923,8 @@ __global__ __launch_bounds__(1024) void layernorm_bwd_colsum_finish_kernel(const
 }
 
 // add.py:29-162 / add_mean_var.py:28-177
-// The fp32 sum leaves through a wave-private LDS patch: in the layout the arithmetic uses (lane l: row l/2, 16 columns)
-// a store instruction would write 64 separate 16-byte pieces; read back as "lane l: row 8i + l/8, columns 4*(l%8) .. +3"
-// each of the four store instructions writes 8 whole 128-byte rows of the block (measured on an fp32 copy of 8192x1600:
-// 17.0 against 22.9 us; the mapping of the loads makes no difference).
+// The sum leaves through a wave-private LDS patch in whole rows (store_block_rows).
 // rowsum / rowsq: [C/32][R] (a wave stores the 32 consecutive rows of its block).
-constexpr int ADD_PITCH = QB + 4;                  // floats per patch row (16-byte aligned rows, rotated over the banks)
 template <typename T, typename ST, typename OT>
 __global__ __launch_bounds__(NT) void add_kernel(const T *x1, const int8_t *q2, const ST *s2, int R, int C,
                                                  int rounding, uint64_t seed, uint64_t offset, OT *y1, int8_t *q,
@@ -854,34 +940,7 @@ __global__ __launch_bounds__(NT) void add_kernel(const T *x1, const int8_t *q2, 
         unpack16(*reinterpret_cast<const v4i *>(q2 + pos.e0), load_scale(s2, pos.rb * SC + pos.cb), b);
 #pragma unroll
         for (int k = 0; k < 16; ++k) a[k] = a[k] + b[k];
-        {
-            float *w = ypatch + (lane >> 1) * ADD_PITCH + (lane & 1) * 16;
-#pragma unroll
-            for (int k = 0; k < 4; ++k) *reinterpret_cast<v4f *>(w + 4 * k) = v4f{a[4 * k], a[4 * k + 1], a[4 * k + 2], a[4 * k + 3]};
-            __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
-            __builtin_amdgcn_wave_barrier();
-            __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
-            if (sizeof(OT) == 4) {
-                float *dst = reinterpret_cast<float *>(y1) + (size_t)(pos.rb * QB + (lane >> 3)) * C + pos.cb * QB + (lane & 7) * 4;
-#pragma unroll
-                for (int i = 0; i < 4; ++i)
-                    *reinterpret_cast<v4f *>(dst + (size_t)(8 * i) * C) =
-                        *reinterpret_cast<const v4f *>(ypatch + (8 * i + (lane >> 3)) * ADD_PITCH + (lane & 7) * 4);
-            } else {
-                // 16-bit sum (rounded to nearest even from the fp32 sum): a row of the block is 64 bytes, a store
-                // instruction writes 16 whole rows (lane l: row 16i + l/4, columns 8*(l%4) .. +7)
-                OT *dst = y1 + (size_t)(pos.rb * QB + (lane >> 2)) * C + pos.cb * QB + (lane & 3) * 8;
-#pragma unroll
-                for (int i = 0; i < 2; ++i) {
-                    const float *r = ypatch + (16 * i + (lane >> 2)) * ADD_PITCH + (lane & 3) * 8;
-                    const v4f lo = *reinterpret_cast<const v4f *>(r), hi = *reinterpret_cast<const v4f *>(r + 4);
-                    OT h[8] = {(OT)lo.x, (OT)lo.y, (OT)lo.z, (OT)lo.w, (OT)hi.x, (OT)hi.y, (OT)hi.z, (OT)hi.w};
-                    *reinterpret_cast<v4i *>(dst + (size_t)(16 * i) * C) = *reinterpret_cast<v4i *>(h);
-                }
-            }
-            __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
-            __builtin_amdgcn_wave_barrier();                       // the patch may be rewritten
-        }
+        store_block_rows(ypatch, a, y1 + (size_t)pos.rb * QB * C + pos.cb * QB, C, lane);
         if (rowsum) {
             float t1 = 0.0f, t2 = 0.0f;
 #pragma unroll
@@ -1106,6 +1165,74 @@ size_t jf_layernorm_bwd_workspace_bytes(int R, int C)
     return ((size_t)2 * R * (C / QB) + (size_t)2 * lnb_groups(R) * C) * sizeof(float);
 }
 
+}  // extern "C"
+
+// rows of up to 2048 columns: one pass over the inputs, the strip's codes held in registers.  add != nullptr: the residual
+// add that follows happens in the same kernel (qdx / sdx are not written).
+static int launch_layernorm_bwd_strip(const int8_t *qx, const void *sx, const int8_t *qg, const void *sg, const float *gamma,
+                                      const float *mean, const float *rstd, int R, int C, int scale_dtype, int rounding,
+                                      uint64_t seed, uint64_t offset, int8_t *qdx, void *sdx, float *dgamma, float *dbeta,
+                                      void *workspace, const LnAddArgs *add, hipStream_t st)
+{
+    const bool want_dw = dgamma || dbeta;
+    const int SC = C / QB;
+    float *sdg = (float *)workspace, *sdb = sdg + (size_t)(R / QB) * C;      // [R/32][C] each: fits the workspace size
+    const size_t patch = add ? LNS_PATCH_ADD : want_dw ? COLSUM_PATCH : 0;
+    const size_t lds = ((size_t)C + 2 * SC * QB + 2 * 8 * QB + 2 * QB + LNS_WAVES * patch) * sizeof(float);
+    const LnAddArgs ad = add ? *add : LnAddArgs{};
+    int dev = 0;
+    if (hipGetDevice(&dev) != hipSuccess || dev < 0 || dev >= MAX_DEVICES) return JF_ERR_DEVICE;
+#define JF_LNS(ST, DW, ADD)                                                                                            \
+    do {                                                                                                               \
+        auto kern = layernorm_bwd_strip_kernel<ST, DW, ADD>;                                                           \
+        static std::atomic<bool> opted_in[MAX_DEVICES] = {};      /* more than 64 KiB of LDS: once per device */        \
+        if (lds > 64 * 1024 && !opted_in[dev].load(std::memory_order_acquire)) {                                       \
+            hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void *>(kern),                                   \
+                                               hipFuncAttributeMaxDynamicSharedMemorySize, 160 * 1024);                \
+            if (e != hipSuccess) return (int)e;                                                                        \
+            opted_in[dev].store(true, std::memory_order_release);                                                      \
+        }                                                                                                              \
+        hipLaunchKernelGGL(kern, dim3(R / QB), dim3(WAVE * LNS_WAVES), lds, st, qx, (const ST *)sx, qg,                \
+                           (const ST *)sg, gamma, mean, rstd, R, C, rounding, seed, offset, qdx, (ST *)sdx,            \
+                           DW ? sdg : nullptr, DW ? sdb : nullptr, ad);                                                \
+    } while (0)
+#define JF_LNS_DW(ST, ADD) do { if (want_dw) JF_LNS(ST, true, ADD); else JF_LNS(ST, false, ADD); } while (0)
+    if (scale_dtype == JF_SCALE_F16) { if (add) JF_LNS_DW(half_t, true); else JF_LNS_DW(half_t, false); }
+    else { if (add) JF_LNS_DW(float, true); else JF_LNS_DW(float, false); }
+#undef JF_LNS_DW
+#undef JF_LNS
+    if (want_dw)
+        hipLaunchKernelGGL(layernorm_bwd_colsum_finish_kernel, dim3(SC, 2), dim3(1024), 0, st, sdg, sdb, R / QB, C, dgamma, dbeta);
+    return (int)hipGetLastError();
+}
+
+extern "C" {
+
+int jf_layernorm_bwd_add(const int8_t *qx, const void *sx, const int8_t *qg, const void *sg, const float *gamma,
+                         const float *mean, const float *rstd, int R, int C, int scale_dtype, int rounding, uint64_t seed,
+                         uint64_t offset, const void *x1, int x1_dtype, int add_rounding, uint64_t add_seed,
+                         uint64_t add_offset, void *y1, int y1_dtype, int8_t *q, void *s, float *dgamma, float *dbeta,
+                         void *workspace, size_t workspace_bytes, jf_stream_t stream)
+{
+    int rc = check_block_tensor(qx, sx, R, C, scale_dtype);
+    if (rc) return rc;
+    if ((rc = check_block_tensor(qg, sg, R, C, scale_dtype))) return rc;
+    if (!gamma || !mean || !rstd || !x1 || !y1 || !q || !s) return JF_ERR_NULL;
+    if (!rounding_ok(rounding) || !rounding_ok(add_rounding)) return JF_ERR_ENUM;
+    if (x1_dtype < JF_FP_F16 || x1_dtype > JF_FP_BF16 || y1_dtype < JF_FP_F16 || y1_dtype > JF_FP_BF16) return JF_ERR_ENUM;
+    if (!aligned16(gamma) || !aligned16(x1) || !aligned16(y1) || !aligned16(q)) return JF_ERR_ALIGN;
+    if (C / QB > LNS_WAVES * LNS_BPW) return JF_ERR_SHAPE;         // wider rows: jf_layernorm_bwd, then jf_add
+    if (!workspace || workspace_bytes < jf_layernorm_bwd_workspace_bytes(R, C)) return JF_ERR_WORKSPACE;
+    if (!aligned16(workspace)) return JF_ERR_ALIGN;
+    if (!device_is_gfx950()) return JF_ERR_DEVICE;
+    LnAddArgs ad;
+    ad.x1 = x1; ad.y1 = y1; ad.q = q; ad.s = s;
+    ad.x1_dtype = x1_dtype; ad.y1_dtype = y1_dtype; ad.rounding = add_rounding;
+    ad.seed = add_seed; ad.offset = add_offset;
+    return launch_layernorm_bwd_strip(qx, sx, qg, sg, gamma, mean, rstd, R, C, scale_dtype, rounding, seed, offset, nullptr,
+                                      nullptr, dgamma, dbeta, workspace, &ad, (hipStream_t)stream);
+}
+
 int jf_layernorm_bwd(const int8_t *qx, const void *sx, const int8_t *qg, const void *sg, const float *gamma,
                      const float *mean, const float *rstd, int R, int C, int scale_dtype, int rounding, uint64_t seed,
                      uint64_t offset, int8_t *qdx, void *sdx, float *dgamma, float *dbeta, void *workspace,
@@ -1123,33 +1250,9 @@ int jf_layernorm_bwd(const int8_t *qx, const void *sx, const int8_t *qg, const v
     hipStream_t st = (hipStream_t)stream;
     const bool want_dw = dgamma || dbeta;
     const int SC = C / QB, groups = lnb_groups(R);
-    if (SC <= LNS_WAVES * LNS_BPW) {
-        // rows of up to 2048 columns: one pass over the inputs, the strip's codes held in registers
-        float *sdg = (float *)workspace, *sdb = sdg + (size_t)(R / QB) * C;      // [R/32][C] each: fits the size above
-        const size_t lds = ((size_t)C + 2 * SC * QB + 2 * 8 * QB + 2 * QB + (want_dw ? LNS_WAVES * COLSUM_PATCH : 0)) * sizeof(float);
-        int dev = 0;
-        if (hipGetDevice(&dev) != hipSuccess || dev < 0 || dev >= MAX_DEVICES) return JF_ERR_DEVICE;
-#define JF_LNS(ST, DW)                                                                                                 \
-        do {                                                                                                           \
-            auto kern = layernorm_bwd_strip_kernel<ST, DW>;                                                            \
-            static std::atomic<bool> opted_in[MAX_DEVICES] = {};  /* more than 64 KiB of LDS: once per device */        \
-            if (lds > 64 * 1024 && !opted_in[dev].load(std::memory_order_acquire)) {                                   \
-                hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void *>(kern),                               \
-                                                   hipFuncAttributeMaxDynamicSharedMemorySize, 160 * 1024);            \
-                if (e != hipSuccess) return (int)e;                                                                    \
-                opted_in[dev].store(true, std::memory_order_release);                                                  \
-            }                                                                                                          \
-            hipLaunchKernelGGL(kern, dim3(R / QB), dim3(WAVE * LNS_WAVES), lds, st, qx, (const ST *)sx, qg,            \
-                               (const ST *)sg, gamma, mean, rstd, R, C, rounding, seed, offset, qdx, (ST *)sdx,        \
-                               DW ? sdg : nullptr, DW ? sdb : nullptr);                                                \
-        } while (0)
-        if (scale_dtype == JF_SCALE_F16) { if (want_dw) JF_LNS(half_t, true); else JF_LNS(half_t, false); }
-        else { if (want_dw) JF_LNS(float, true); else JF_LNS(float, false); }
-#undef JF_LNS
-        if (want_dw)
-            hipLaunchKernelGGL(layernorm_bwd_colsum_finish_kernel, dim3(SC, 2), dim3(1024), 0, st, sdg, sdb, R / QB, C, dgamma, dbeta);
-        return (int)hipGetLastError();
-    }
+    if (SC <= LNS_WAVES * LNS_BPW)
+        return launch_layernorm_bwd_strip(qx, sx, qg, sg, gamma, mean, rstd, R, C, scale_dtype, rounding, seed, offset, qdx,
+                                          sdx, dgamma, dbeta, workspace, nullptr, st);
     const size_t smem = ((size_t)C + 2 * QB + 16 * QB) * sizeof(float);   // gamma, c1, c2 and the row-sum partials in LDS
     if (smem > LDS_VECTOR_LIMIT) return JF_ERR_SHAPE;
     float *part1 = (float *)workspace, *part2 = part1 + (size_t)R * SC;

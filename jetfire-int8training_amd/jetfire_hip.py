@@ -28,7 +28,7 @@ EXPORTS = [
     "jf_error_string", "jf_igemm_workspace_bytes", "jf_igemm_s32", "jf_igemm_block_acc", "jf_igemm_block_fp",
     "jf_igemm_splitk_plan", "jf_igemm_block_fp_workspace_bytes", "jf_igemm_block_q_gelu", "jf_igemm_block_fp_noalloc", "jf_igemm_block_q_gelu_bwd",
     "jf_igemm_block_q", "jf_quantize", "jf_dequantize", "jf_transpose_s8", "jf_rowstats", "jf_layernorm_fwd",
-    "jf_layernorm_bwd_workspace_bytes", "jf_layernorm_bwd", "jf_gelu_fwd", "jf_gelu_bwd", "jf_add", "jf_calibrate", "jf_wall_clock_khz", "jf_igemm_phase_record", "jf_rowstats_finish",
+    "jf_layernorm_bwd_workspace_bytes", "jf_layernorm_bwd", "jf_layernorm_bwd_add", "jf_gelu_fwd", "jf_gelu_bwd", "jf_add", "jf_calibrate", "jf_wall_clock_khz", "jf_igemm_phase_record", "jf_rowstats_finish",
     "jf_igemm_block_q_dequant", "jf_quantize_slabs",
 ]
 
@@ -71,6 +71,8 @@ def lib():
         L.jf_layernorm_bwd.argtypes = [_p, _p, _p, _p, _p, _p, _p, _i, _i, _i, _i, _u64, _u64, _p, _p, _p, _p, _p, _sz, _p]
         L.jf_gelu_fwd.argtypes = [_p, _p, _i, _i, _i, _i, _f, _p, _p, _p]
         L.jf_gelu_bwd.argtypes = [_p, _p, _p, _p, _i, _i, _i, _i, _i, _u64, _u64, _p, _p, _p]
+        L.jf_layernorm_bwd_add.argtypes = [_p, _p, _p, _p, _p, _p, _p, _i, _i, _i, _i, _u64, _u64, _p, _i, _i, _u64, _u64,
+                                           _p, _i, _p, _p, _p, _p, _p, _sz, _p]
         L.jf_add.argtypes = [_p, _i, _p, _p, _i, _i, _i, _i, _u64, _u64, _p, _i, _p, _p, _p, _p, _p]
         L.jf_wall_clock_khz.argtypes = []
         L.jf_calibrate.argtypes = [_i, _i, _i, _i, _i, _i, _p, _p, _p]
@@ -462,6 +464,42 @@ def layernorm_bwd(qx, sx, qg, sg, gamma, mean, rstd, rounding=ROUND_NEAREST, wan
                                  rounding, seed, offset, _ptr(qdx), _ptr(sdx), _ptr(dgamma), _ptr(dbeta), _ptr(ws), nbytes,
                                  _stream()))
     return qdx, sdx, dgamma, dbeta
+
+
+def layernorm_bwd_add(qx, sx, qg, sg, gamma, mean, rstd, x1, rounding=ROUND_NEAREST, add_rounding=ROUND_TRUNC,
+                      want_dbeta=True, out_dtype=torch.float32, seed=None, offset=None, add_seed=None, add_offset=None):
+    """layernorm_bwd followed by add(x1, dx codes, dx scales): (y1, q, s, dgamma, dbeta), the bits the two calls give
+    (noise offsets are drawn in their order).  Rows of up to 2048 columns run as one kernel that never stores dx; wider
+    rows make the two calls."""
+    R, Cc, code = _block_tensor(qx, sx, "x")
+    R2, C2, code2 = _block_tensor(qg, sg, "g")
+    if (R2, C2, code2) != (R, Cc, code):
+        raise RuntimeError("x and g must have the same shape and scale dtype")
+    _vec(gamma, Cc, "gamma")
+    _vec(mean, R, "mean")
+    _vec(rstd, R, "rstd")
+    _need(x1, None, "x1")
+    if x1.dtype not in _FP_CODE or tuple(x1.shape) != (R, Cc):
+        raise RuntimeError("x1 must be a float tensor of the same shape as x")
+    if out_dtype not in _FP_CODE:
+        raise RuntimeError("out_dtype must be float32, float16 or bfloat16")
+    seed, offset = _rng(rounding, R * Cc, seed, offset, qx.device)
+    add_seed, add_offset = _rng(add_rounding, R * Cc, add_seed, add_offset, qx.device)
+    if Cc // QB > 64:
+        qdx, sdx, dgamma, dbeta = layernorm_bwd(qx, sx, qg, sg, gamma, mean, rstd, rounding, want_dbeta, seed, offset)
+        return add(x1, qdx, sdx, add_rounding, seed=add_seed, offset=add_offset, out_dtype=out_dtype) + (dgamma, dbeta)
+    nbytes = lib().jf_layernorm_bwd_workspace_bytes(R, Cc)
+    ws = torch.empty(nbytes, dtype=torch.int8, device=qx.device)
+    y1 = torch.empty((R, Cc), dtype=out_dtype, device=qx.device)
+    q = torch.empty_like(qx)
+    s = torch.empty_like(sx)
+    dgamma = torch.empty(Cc, dtype=torch.float32, device=qx.device)
+    dbeta = torch.empty(Cc, dtype=torch.float32, device=qx.device) if want_dbeta else None
+    check(lib().jf_layernorm_bwd_add(_ptr(qx), _ptr(sx), _ptr(qg), _ptr(sg), _ptr(gamma), _ptr(mean), _ptr(rstd), R, Cc,
+                                     code, rounding, seed, offset, _ptr(x1), _FP_CODE[x1.dtype], add_rounding, add_seed,
+                                     add_offset, _ptr(y1), _FP_CODE[out_dtype], _ptr(q), _ptr(s), _ptr(dgamma), _ptr(dbeta),
+                                     _ptr(ws), nbytes, _stream()))
+    return y1, q, s, dgamma, dbeta
 
 
 def gelu_fwd(q, s, approx=GELU_ERF, amax_eps=5e-5):

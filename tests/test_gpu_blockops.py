@@ -235,6 +235,36 @@ def test_add(jf, oracle, dtype, mode):
     assert np.allclose(m, wy.mean(-1), atol=1e-5) and np.allclose(rstd.cpu().numpy(), 1 / np.sqrt(wy.var(-1)), rtol=1e-4)
 
 
+@pytest.mark.parametrize("R,C", [(64, 96), (96, 1600), (32, 2048), (64, 2080)])
+@pytest.mark.parametrize("x1_dtype,out_dtype,scale_dtype", [(torch.float32, torch.float32, torch.float32),
+                                                            (torch.bfloat16, torch.bfloat16, torch.float16),
+                                                            (torch.float16, torch.float32, torch.float16),
+                                                            (torch.float32, torch.bfloat16, torch.float32)])
+def test_layernorm_backward_with_the_residual_add(jf, R, C, x1_dtype, out_dtype, scale_dtype):
+    """One kernel for LayerNorm backward + the residual add that follows it in the recipe (rows of up to 2048 columns;
+    2080 columns make the two calls inside the wrapper): the same bits as the two calls, which are checked against the
+    CPU checker one by one above."""
+    g = torch.Generator().manual_seed(R + C)
+    x = torch.randn(R, C, generator=g).cuda()
+    dy = (torch.randn(R, C, generator=g) * 1e-2).cuda()
+    gamma = (1 + 0.1 * torch.randn(C, generator=g)).cuda()
+    x1 = (torch.randn(R, C, generator=g) * 1e-2).to(x1_dtype).cuda()
+    qx, sx = jf.quantize(x, scale_dtype=scale_dtype)
+    qg, sg = jf.quantize(dy, jf.ROUND_STOCHASTIC, scale_dtype, seed=4, offset=0)
+    mean, rstd = jf.rowstats(qx, sx)
+    for want_dbeta in (True, False):
+        for r1, r2 in ((jf.ROUND_STOCHASTIC, jf.ROUND_STOCHASTIC_TRUNC), (jf.ROUND_NEAREST, jf.ROUND_TRUNC)):
+            qdx, sdx, dg, db = jf.layernorm_bwd(qx, sx, qg, sg, gamma, mean, rstd, r1, want_dbeta, seed=7, offset=3)
+            wy, wq, ws = jf.add(x1, qdx, sdx, r2, seed=8, offset=5, out_dtype=out_dtype)
+            y1, q, s, dg2, db2 = jf.layernorm_bwd_add(qx, sx, qg, sg, gamma, mean, rstd, x1, r1, r2, want_dbeta, out_dtype,
+                                                      seed=7, offset=3, add_seed=8, add_offset=5)
+            assert y1.dtype == out_dtype and torch.equal(y1, wy)
+            assert torch.equal(q, wq) and torch.equal(s, ws)
+            assert torch.equal(dg, dg2)
+            assert (db is None and db2 is None) or torch.equal(db, db2)
+    assert int(q.abs().max()) > 100                                 # a real block tensor came out
+
+
 @pytest.mark.parametrize("out_dtype", [torch.bfloat16, torch.float16])
 @pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
 def test_add_with_a_16_bit_sum(jf, oracle, dtype, out_dtype):
