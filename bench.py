@@ -319,6 +319,13 @@ def nonlinear_extras(jf, torch):
     put("add_8192x1600", t(lambda: jf.add(x, qx, sx, jf.ROUND_TRUNC)), 10 * n)
     put("add_sr_8192x1600", t(lambda: jf.add(x, qx, sx, jf.ROUND_STOCHASTIC_TRUNC, seed=1, offset=0)), 10 * n)
     put("add_meanvar_8192x1600", t(lambda: jf.rowstats_finish(*jf.add(x, qx, sx, jf.ROUND_TRUNC, with_stats=True)[3:], C)), 10 * n)
+    # LayerNorm backward with the residual add behind it in one kernel (what the recipe's backward runs), fp32 / bfloat16
+    # gradient in and out: codes of x and dy in; the fp gradient in; the sum and its codes out
+    xb = x.to(torch.bfloat16)
+    put("layernorm_bwd_add_sr_8192x1600", t(lambda: jf.layernorm_bwd_add(qx, sx, qg, sg, gamma, mean, rstd, x, jf.ROUND_STOCHASTIC,
+        jf.ROUND_STOCHASTIC_TRUNC, seed=1, offset=0, add_seed=2, add_offset=0)), 11 * n)
+    put("layernorm_bwd_add_sr_bf16_8192x1600", t(lambda: jf.layernorm_bwd_add(qx, sx, qg, sg, gamma, mean, rstd, xb, jf.ROUND_STOCHASTIC,
+        jf.ROUND_STOCHASTIC_TRUNC, out_dtype=torch.bfloat16, seed=1, offset=0, add_seed=2, add_offset=0)), 7 * n)
     R, C = TOKENS, 6400
     x = torch.randn(R, C, generator=g).cuda()
     dy = (torch.randn(R, C, generator=g) * 1e-3).cuda()
