@@ -311,6 +311,34 @@ def test_full_size_nonlinear_properties(jf, oracle):
     assert torch.equal(jf.transpose_s8(jf.transpose_s8(qy)), qy)
 
 
+def test_full_size_layernorm_backward_with_the_residual_add(jf, oracle):
+    """8192 x 1600, stochastic, binary16 scales, bfloat16 gradient in and out (what a block of the recipe runs): the
+    one-kernel form against the two calls at full size, and three strips of the two calls against the CPU checker."""
+    R, C = 8192, 1600
+    g = torch.Generator().manual_seed(5)
+    x = torch.randn(R, C, generator=g).cuda()
+    dy = (torch.randn(R, C, generator=g) * 1e-3).cuda()
+    gamma = (1 + 0.1 * torch.randn(C, generator=g)).cuda()
+    x1 = (torch.randn(R, C, generator=g) * 1e-3).to(torch.bfloat16).cuda()
+    qx, sx = jf.quantize(x, scale_dtype=torch.float16)
+    qg, sg = jf.quantize(dy, jf.ROUND_STOCHASTIC, torch.float16, seed=1, offset=0)
+    mean, rstd = jf.rowstats(qx, sx)
+    qdx, sdx, dg, db = jf.layernorm_bwd(qx, sx, qg, sg, gamma, mean, rstd, jf.ROUND_STOCHASTIC, True, seed=2, offset=11)
+    wy, wq, ws = jf.add(x1, qdx, sdx, jf.ROUND_STOCHASTIC_TRUNC, seed=3, offset=17, out_dtype=torch.bfloat16)
+    y1, q, s, dg2, db2 = jf.layernorm_bwd_add(qx, sx, qg, sg, gamma, mean, rstd, x1, jf.ROUND_STOCHASTIC,
+                                              jf.ROUND_STOCHASTIC_TRUNC, True, torch.bfloat16, seed=2, offset=11,
+                                              add_seed=3, add_offset=17)
+    assert torch.equal(y1, wy) and torch.equal(q, wq) and torch.equal(s, ws)
+    assert torch.equal(dg, dg2) and torch.equal(db, db2)
+    for r0 in (0, 4096, 8160):
+        sl, bl = slice(r0, r0 + 32), slice(r0 // 32, r0 // 32 + 1)
+        oy, oq, os_ = oracle.add(x1[sl].float().cpu().numpy(), qdx[sl].cpu().numpy(), sdx[bl].float().cpu().numpy(), True, 3,
+                                 17 + r0 * C // 8, True, False, "f16")
+        assert torch.equal(y1[sl].cpu(), torch.from_numpy(oy).to(torch.bfloat16)), r0
+        same(q[sl], oq, f"codes rows {r0}")
+        same(s[bl], os_, f"scales rows {r0}")
+
+
 def _random_block_shapes(n, seed):
     rng = np.random.default_rng(seed)
     for _ in range(n):
