@@ -194,10 +194,11 @@ def recipe_block(torch, only=None):
     of three; the difference, halved, is what a block costs inside a stack.  Parameter gradients are reset to None before
     every step, as an optimizer's zero_grad() does.  The INT8 stack takes a float32 input (an embedding's output) and
     carries a bfloat16 residual between blocks, as the reference does (INT8_GPT2/qmodel.py:228); the sum inside a block
-    stays float32."""
+    stays float32.  Both sides pay for their weights in every step: the INT8 stack quantises them again (its cache of weight
+    codes is cleared, as after an optimizer update), the bf16 blocks cast them."""
     import torch.nn.functional as F
     sys.path.insert(0, os.path.join(PKG, "Jetfire"))
-    from recipe import QStack
+    from recipe import QStack, weight_codes
     torch.manual_seed(0)
     B, T, C, H = 8, 1024, 1600, 25
     x = torch.randn(B, T, C, device="cuda", requires_grad=True)
@@ -236,6 +237,12 @@ def recipe_block(torch, only=None):
             return h0
         params = list(model.parameters())
 
+        def int8_step():
+            # a training step follows an optimizer update: the cached weight codes are stale and every weight is quantised
+            # again (the bf16 blocks cast their weights in every step as well)
+            weight_codes.clear()
+            model(x).backward(wr)
+
         def peak_mb(fn):
             # memory held at the end of the forward pass above what is held before it (saved activations + output)
             for q in params + [x, xr]:
@@ -251,13 +258,16 @@ def recipe_block(torch, only=None):
         if layers == 3 and not only:
             out["mem"] = (peak_mb(lambda: model(x)), peak_mb(lambda: ref_stack(xr, torch.bfloat16)))
         if only:                                                   # one of the two, 3 + 10 steps: a kernel trace of it
-            return round(t(lambda: model(x).backward(wr), params + [x]) if only == "int8"
+            return round(t(int8_step, params + [x]) if only == "int8"
                          else t(lambda: ref_stack(xr, torch.bfloat16).backward(wr), params + [xr]), 3)
-        out[layers] = (t(lambda: model(x).backward(wr), params + [x]),
+        if layers == 3:                                            # weight codes reused between steps (micro-batches of one update)
+            out["cached"] = t(lambda: model(x).backward(wr), params + [x])
+        out[layers] = (t(int8_step, params + [x]),
                        t(lambda: ref_stack(xr, torch.bfloat16).backward(wr), params + [xr]))
         del model
     return {"tokens": B * T, "int8_recipe_ms": round(out[1][0], 3), "torch_bf16_ms": round(out[1][1], 3),
             "stack_of_3_blocks": {"int8_recipe_ms": round(out[3][0], 3), "torch_bf16_ms": round(out[3][1], 3),
+                                  "int8_recipe_weight_codes_reused_ms": round(out["cached"], 3),
                                   "held_after_forward_MiB": {"int8_recipe": out["mem"][0], "torch_bf16": out["mem"][1]}},
             "per_block_inside_a_stack": {"int8_recipe_ms": round((out[3][0] - out[1][0]) / 2, 3),
                                          "torch_bf16_ms": round((out[3][1] - out[1][1]) / 2, 3)}}
