@@ -17,8 +17,9 @@
  *     block tensor's own row-major scale array (JF_SCALES_ROWMAJOR): sa[mb*(K/32)+kb]; output scales are
  *     sc[mb*(N/32)+nb]  (reference: …/igemm/igemm_BlockSquare32OutputIntQuantizeBiasRowCol.cu:110-111,
  *     187-188, 297-304; paths below are relative to JetfireGEMMKernel/BlockQuantize/cpp_extension/).
- *   - stochastic rounding draws Philox4x32-10 noise keyed by (seed, offset + flat output index / 8),
- *     16 bits per element, so results do not depend on the launch geometry.
+ *   - stochastic rounding draws Philox4x32 noise keyed by (seed, offset + flat output index / 8), 16 bits per
+ *     element, so results do not depend on the launch geometry.  The round count is a build-time choice
+ *     (JF_PHILOX_ROUNDS: 7 by default, 10 = the count of the reference's generators); jf_philox_rounds() reports it.
  */
 #ifndef JETFIRE_HIP_H
 #define JETFIRE_HIP_H
@@ -72,6 +73,10 @@ typedef void *jf_stream_t;
 
 const char *jf_error_string(int code);
 
+/* Rounds of the Philox4x32 generator this library was built with (reference: curandStatePhilox4_32_10 at
+ * igemm/igemm_BlockSquare32OutputIntQuantizeStochastic.cu:311, 10 rounds). */
+int jf_philox_rounds(void);
+
 /* Bytes of device scratch the GEMM entry points need for this problem: 0 for both layouts (a JF_B_KN operand is
  * staged as it lies in memory and transposed by the LDS read).  The workspace arguments of jf_igemm_s32,
  * jf_igemm_block_acc and jf_igemm_block_q are kept for callers written against an implementation that re-lays B out
@@ -111,7 +116,9 @@ int jf_igemm_block_fp(const int8_t *A, const int8_t *B, const void *sa, const vo
  * loops, harnesses that forbid hipMalloc.  No counterpart in the reference.  Same arguments, same arithmetic and the
  * same bits as jf_igemm_block_fp with the same splitk request, minus the workspace: the fp32 partial results of the K
  * split live in a buffer built into the library (JF_NOALLOC_SCRATCH_BYTES per GPU the library runs on, held until the
- * process ends).  Calls nothing that allocates or frees.  A problem whose K split needs more scratch
+ * process ends).  Calls nothing that allocates or frees -- with one proviso: the HIP runtime loads a library's device
+ * code (and with it this buffer) on the first call into the library on a device, so make one warm-up call of any
+ * entry point on that device before a capture or an allocation-free region begins.  A problem whose K split needs more scratch
  * (parts * M * N * 4 bytes, see jf_igemm_splitk_plan) is refused with JF_ERR_SCRATCH_LIMIT; splitk = 1 never needs any.
  * All calls on one GPU share that GPU's buffer: two calls that may overlap on one GPU (different streams, or threads
  * without ordering between them) race on it and must be serialised by the caller. */

@@ -63,7 +63,13 @@ __device__ __forceinline__ float wave_max(float v)
 // R = 7, the smallest round count the authors report as passing BigCrush (10 is their default with a safety margin):
 // the generator is the largest single cost of every stochastic-rounding kernel here, and its multiplies run at a
 // quarter of the vector ALU's rate.
-constexpr int PHILOX_ROUNDS = 7;
+// Build-time switch: -DJF_PHILOX_ROUNDS=10 gives the reference generator's round count (curandStatePhilox4_32_10,
+// tl.rand); jf_philox_rounds() reports what a library was built with, and the CPU checker follows it.
+#ifndef JF_PHILOX_ROUNDS
+#define JF_PHILOX_ROUNDS 7
+#endif
+constexpr int PHILOX_ROUNDS = JF_PHILOX_ROUNDS;
+static_assert(PHILOX_ROUNDS >= 7 && PHILOX_ROUNDS <= 10, "Philox4x32: 7 to 10 rounds");
 template <int ROUNDS>
 __device__ __forceinline__ void philox4x32(uint32_t c0, uint32_t c1, uint32_t c2, uint32_t c3,
                                            uint32_t k0, uint32_t k1, uint32_t out[4])

@@ -1015,6 +1015,8 @@ const char *jf_error_string(int code)
     }
 }
 
+int jf_philox_rounds(void) { return PHILOX_ROUNDS; }
+
 size_t jf_igemm_workspace_bytes(int M, int N, int K, int b_layout)
 {
     (void)M; (void)N; (void)K; (void)b_layout;                // both B layouts are read in place

@@ -29,7 +29,7 @@ EXPORTS = [
     "jf_igemm_splitk_plan", "jf_igemm_block_fp_workspace_bytes", "jf_igemm_block_q_gelu", "jf_igemm_block_fp_noalloc", "jf_igemm_block_q_gelu_bwd",
     "jf_igemm_block_q", "jf_quantize", "jf_dequantize", "jf_transpose_s8", "jf_rowstats", "jf_layernorm_fwd",
     "jf_layernorm_bwd_workspace_bytes", "jf_layernorm_bwd", "jf_layernorm_bwd_add", "jf_gelu_fwd", "jf_gelu_bwd", "jf_add", "jf_calibrate", "jf_wall_clock_khz", "jf_igemm_phase_record", "jf_rowstats_finish",
-    "jf_igemm_block_q_dequant", "jf_quantize_slabs",
+    "jf_igemm_block_q_dequant", "jf_quantize_slabs", "jf_philox_rounds",
 ]
 
 _lib = None

@@ -67,7 +67,16 @@ void jfo_philox4x32_10(const uint32_t ctr[4], const uint32_t key[2], uint32_t ou
 /* Rounds of the generator behind the rounding noise: 7, the smallest count Salmon et al. report as passing BigCrush
  * (the kernels pay for every round with two quarter-rate multiplies per 8 elements).  The round function and key
  * schedule are the ones the 10-round known answers pin. */
-#define JFO_NOISE_ROUNDS 7
+static int jfo_noise_rounds_now = 7;
+#define JFO_NOISE_ROUNDS jfo_noise_rounds_now
+
+/* The product library has a build-time round count (7 by default, 10 = the reference generator's); a test run sets the
+ * checker to what the library under test reports.  Returns the count in force afterwards. */
+int jfo_set_noise_rounds(int rounds)
+{
+    if (rounds >= 1 && rounds <= 10) jfo_noise_rounds_now = rounds;
+    return jfo_noise_rounds_now;
+}
 
 /*
  * Rounding noise for element `e` (flat row-major index r*C+c of the OUTPUT

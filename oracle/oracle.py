@@ -110,7 +110,15 @@ def philox4x32_10(ctr, key):
     return o
 
 
-NOISE_ROUNDS = 7            # rounds of the generator behind sr_noise (JFO_NOISE_ROUNDS)
+NOISE_ROUNDS = 7            # rounds of the generator behind sr_noise (JFO_NOISE_ROUNDS); see set_noise_rounds
+
+
+def set_noise_rounds(rounds):
+    """Follow the round count the library under test was built with (jf_philox_rounds())."""
+    global NOISE_ROUNDS
+    lib().jfo_set_noise_rounds.argtypes = [_i]
+    NOISE_ROUNDS = int(lib().jfo_set_noise_rounds(int(rounds)))
+    return NOISE_ROUNDS
 
 
 def philox4x32(ctr, key, rounds):

@@ -12,10 +12,17 @@ def pytest_configure(config):
     config.addinivalue_line("markers", "gpu: needs a real MI355X (run on the GPU box)")
 
 
+PKG = os.path.join(ROOT, "jetfire-int8training_amd")
+
+
 @pytest.fixture(scope="session")
 def oracle():
     from oracle import oracle as O
     O.lib()
+    lib = os.path.join(PKG, "libjetfire_hip.so")
+    if os.path.exists(lib):                      # the checker draws its rounding noise with the library's round count
+        import ctypes
+        O.set_noise_rounds(ctypes.CDLL(lib).jf_philox_rounds())
     return O
 
 PKG = os.path.join(ROOT, "jetfire-int8training_amd")

@@ -1,10 +1,11 @@
 """The benchmark configurations at their full sizes, through the C ABI, against the CPU oracle.
 
-Every kernel here is local to 32-row strips of its output (GEMM rows, block rows of the block-local kernels, LayerNorm
-rows), so a strip of the output computed by the oracle from the matching strip of the inputs is a complete, bit-exact
-check of that strip.  Each case checks three strips: the first, an interior one that does not start on a 128-row tile
-boundary, and the last; all columns of each, so ragged last column tiles (1600, 4800 and 2304 are not multiples of the
-128-wide tile) and every K depth are covered.  Bars as everywhere: codes, scales, INT32 and fp32 accumulators bit-exact.
+The GEMMs are compared over their WHOLE outputs, bit for bit: which workgroup computes which tile (and which part of a
+K split) depends on the shape of the launch, so a sample of rows would not notice a tile computed twice or not at all in
+the rows it leaves out.  The oracle needs about half a second per GPT-2 XL GEMM on 16 host threads.  The block-local
+kernels (LayerNorm, GELU) have no such map (a block's result depends on its own 32-row strip only) and are checked on
+three strips: the first, an interior one that does not start on a 128-row boundary, and the last, all columns of each.
+Bars as everywhere: codes, scales, INT32 and fp32 accumulators bit-exact.
 
 Shapes (M, N, K) per layer: forward (T, C_out, C_in), dgrad (T, C_in, C_out), wgrad (C_out, C_in, T).
 """
@@ -12,7 +13,7 @@ import numpy as np
 import pytest
 import torch
 
-from helpers import QB
+from helpers import QB, rand_codes, rand_scales
 
 pytestmark = pytest.mark.gpu
 
@@ -83,32 +84,30 @@ def check_linear_layer(jf, oracle, T, Cin, Cout, seed, outliers, gelu=None, gelu
     torch.cuda.synchronize()
     X, W, G, GT = (t.cpu().numpy() for t in (qx, qw, qg, qgT))
     SX, SW, SG = (t.cpu().numpy() for t in (sx, sw, sg))
-    SWt = cont(SW.T)
-    for r0 in strips(T):
-        rows, rb = slice(r0, r0 + QB), slice(r0 // QB, r0 // QB + 1)
-        wq, wsc = oracle.igemm_block_q(X[rows], W, cont(SX[rb].T), SWt, 0)
-        same(y[rows], wq, f"forward codes rows {r0}")
-        same(sy[rb], wsc, f"forward scales rows {r0}")
-        if gelu is not None:
-            wg, wgs = oracle.gelu_fwd(wq, wsc, gelu, eps)
-            same(fg[rows], wg, f"fused GELU codes rows {r0}")
-            same(fgs[rb], wgs, f"fused GELU scales rows {r0}")
-        acc = oracle.igemm_block_f32(G[rows], W, cont(SG[rb].T), SW, 1)
-        wq, wsc = oracle.requant(acc, stochastic=True, seed=seed + 1, offset=17 + r0 * Cin // 8)
-        same(dx[rows], wq, f"dgrad codes rows {r0}")
-        same(sdx[rb], wsc, f"dgrad scales rows {r0}")
-        if gelu_bwd:
-            wb, wbs = oracle.gelu_bwd(X[rows], SX[rb], wq, wsc, 0, True, seed + 2, 5 + r0 * Cin // 8)
-            same(fb[rows], wb, f"fused GELU backward codes rows {r0}")
-            same(fbs[rb], wbs, f"fused GELU backward scales rows {r0}")
-    for r0 in strips(Cout):
-        rows, rb = slice(r0, r0 + QB), slice(r0 // QB, r0 // QB + 1)
-        sa = cont(SG[:, rb])
-        same(dw[rows], oracle.igemm_block_f32(GT[rows], X, sa, SX, 1), f"wgrad rows {r0}")
-        want = oracle.igemm_block_f32_splitk(GT[rows], X, sa, SX, 1, parts, per)
-        same(dw_km[rows], want, f"wgrad in place, {parts} parts, rows {r0}")
-        with np.errstate(over="ignore"):
-            same(dw_km16[rows], want.astype(np.float16), f"wgrad in place fp16, rows {r0}")
+    # forward, every tile
+    wq, wsc = oracle.igemm_block_q(X, W, cont(SX.T), cont(SW.T), 0)
+    same(y, wq, "forward codes")
+    same(sy, wsc, "forward scales")
+    if gelu is not None:
+        wg, wgs = oracle.gelu_fwd(wq, wsc, gelu, eps)
+        same(fg, wg, "fused GELU codes")
+        same(fgs, wgs, "fused GELU scales")
+    # activation gradient, every tile
+    acc = oracle.igemm_block_f32(G, W, cont(SG.T), SW, 1)
+    wq, wsc = oracle.requant(acc, stochastic=True, seed=seed + 1, offset=17)
+    del acc
+    same(dx, wq, "dgrad codes")
+    same(sdx, wsc, "dgrad scales")
+    if gelu_bwd:
+        wb, wbs = oracle.gelu_bwd(X, SX, wq, wsc, 0, True, seed + 2, 5)
+        same(fb, wb, "fused GELU backward codes")
+        same(fbs, wbs, "fused GELU backward scales")
+    # weight gradient, every tile: one chain from the transposed copy, and the gradient in place with the library's K split
+    same(dw, oracle.igemm_block_f32(GT, X, SG, SX, 1), "wgrad")
+    want = oracle.igemm_block_f32_splitk(GT, X, SG, SX, 1, parts, per)
+    same(dw_km, want, f"wgrad in place, {parts} parts")
+    with np.errstate(over="ignore"):
+        same(dw_km16, want.astype(np.float16), "wgrad in place fp16")
 
 
 def test_cfg1_cpu_path_case(jf, oracle):
@@ -145,6 +144,86 @@ def test_cfg3_gpt2_xl_layer(jf, oracle, name, Cin, Cout, gelu):
     """fc also runs the forward with the GELU fused into the epilogue, fc2 the activation gradient with the GELU
     backward fused into the epilogue (the recipe's MLP path)."""
     check_linear_layer(jf, oracle, 8192, Cin, Cout, seed=0, outliers=True, gelu=gelu, gelu_bwd=name == "fc2")
+
+
+def test_cfg5_stress_cube(jf, oracle):
+    """M = N = K = 8192, heavy-tailed A (Student-t, 3 degrees of freedom), B ~ N(0, 0.02); the requantised output in
+    deterministic and in stochastic mode, every code and every scale."""
+    n = 8192
+    g = torch.Generator().manual_seed(0)
+    a = torch.randn(n, n, generator=g) / torch.sqrt(torch.randn(3, n, n, generator=g).pow_(2).mean(0))   # t(3) = z / sqrt(chi2_3 / 3)
+    b = torch.randn(n, n, generator=g) * 0.02
+    qa, sa = jf.quantize(a.cuda(), scale_dtype=torch.float32)
+    qb, sb = jf.quantize(b.cuda(), scale_dtype=torch.float32)
+    del a, b
+    print("cfg5 8192^3 deterministic + stochastic", flush=True)
+    y, sy = jf.igemm_block_q(qa, qb, sa.t(), sb.t(), jf.B_NK)
+    z, sz = jf.igemm_block_q(qa, qb, sa.t(), sb.t(), jf.B_NK, rounding=jf.ROUND_STOCHASTIC, seed=5, offset=11)
+    torch.cuda.synchronize()
+    A, B, SA, SB = (t.cpu().numpy() for t in (qa, qb, sa, sb))
+    acc = oracle.igemm_block_f32(A, B, cont(SA.T), cont(SB.T), 0)
+    wq, wsc = oracle.requant(acc)
+    same(y, wq, "deterministic codes")
+    same(sy, wsc, "deterministic scales")
+    wq, wsc = oracle.requant(acc, stochastic=True, seed=5, offset=11)
+    same(z, wq, "stochastic codes")
+    same(sz, wsc, "stochastic scales")
+
+
+# One odd-shaped launch per regime of the launcher's choice of wave priorities (by the number of 128 x 128 workgroups
+# against the 512 that are resident at once: up to one round; 1 to 1.5 rounds with short and with long tiles; 1.5 to 2;
+# more than 2), each with a number of tile rows that is not a multiple of the 8-row groups the tile order walks, a
+# workgroup count that is not a multiple of the 8 XCDs, and ragged last tiles in both directions.
+PACE_SHAPES = [
+    (11 * 128 - 32, 13 * 128 - 64, 512),        # 143 workgroups
+    (21 * 128 - 32, 29 * 128 - 96, 256),        # 609: 1.19 rounds, short tiles
+    (21 * 128 - 32, 29 * 128 - 96, 4096),       # 609: long tiles
+    (27 * 128 - 64, 33 * 128 - 32, 384),        # 891: 1.74 rounds
+    (37 * 128 - 96, 31 * 128 - 64, 160),        # 1147: 2.24 rounds
+]
+
+
+@pytest.mark.parametrize("M,N,K", PACE_SHAPES)
+@pytest.mark.parametrize("layout", [0, 1])
+def test_odd_shapes_in_every_pacing_regime(jf, oracle, M, N, K, layout):
+    tiles = ((M + 127) // 128) * ((N + 127) // 128)
+    assert tiles % 8 and ((M + 127) // 128) % 8
+    print(f"odd shape M={M} N={N} K={K} layout={layout} workgroups={tiles}", flush=True)
+    rng = np.random.default_rng(M + N + K + layout)
+    A = rand_codes(rng, (M, K))
+    B = rand_codes(rng, (K, N) if layout else (N, K))
+    sa = rand_scales(rng, (K // QB, M // QB), f16=False)
+    sb = rand_scales(rng, (K // QB, N // QB), f16=False)
+    dA, dB, dsa, dsb = (torch.from_numpy(t).cuda() for t in (A, B, sa, sb))
+    q, sc = jf.igemm_block_q(dA, dB, dsa, dsb, layout)
+    z, sz = jf.igemm_block_q(dA, dB, dsa, dsb, layout, rounding=jf.ROUND_STOCHASTIC, seed=9, offset=3)
+    fp = jf.igemm_block_fp(dA, dB, dsa, dsb, layout, torch.float32)
+    torch.cuda.synchronize()
+    acc = oracle.igemm_block_f32(A, B, sa, sb, layout)
+    same(fp, acc, "fp32 accumulators")
+    wq, wsc = oracle.requant(acc)
+    same(q, wq, "deterministic codes"); same(sc, wsc, "deterministic scales")
+    wq, wsc = oracle.requant(acc, stochastic=True, seed=9, offset=3)
+    same(z, wq, "stochastic codes"); same(sz, wsc, "stochastic scales")
+
+
+@pytest.mark.parametrize("M,N,K,req", [(11 * 128 - 32, 5 * 128 - 96, 4096, 0), (3 * 128, 7 * 128 - 32, 6144, 5),
+                                       (13 * 128 - 64, 3 * 128 - 32, 2048, 3)])
+def test_odd_shapes_with_a_k_split(jf, oracle, M, N, K, req):
+    """The weight-gradient form (A given as [K,M], B as [K,N]) with several parts: workgroups are ordered part-major
+    over the same tile map, every part of every tile must be computed exactly once."""
+    parts, per = jf.splitk_plan(M, N, K, req)
+    assert parts > 1 and (req == 0 or (parts * ((M + 127) // 128) * ((N + 127) // 128)) % 8)
+    print(f"odd split shape M={M} N={N} K={K} parts={parts}", flush=True)
+    rng = np.random.default_rng(M + N + K)
+    At = rand_codes(rng, (K, M))
+    B = rand_codes(rng, (K, N))
+    sa = rand_scales(rng, (K // QB, M // QB), f16=False)
+    sb = rand_scales(rng, (K // QB, N // QB), f16=False)
+    dA, dB, dsa, dsb = (torch.from_numpy(t).cuda() for t in (At, B, sa, sb))
+    got = jf.igemm_block_fp(dA, dB, dsa, dsb, jf.B_KN, torch.float32, a_layout=jf.A_KM, splitk=req)
+    torch.cuda.synchronize()
+    same(got, oracle.igemm_block_f32_splitk(cont(At.T), B, sa, sb, 1, parts, per), f"{parts} parts")
 
 
 def test_cfg4_layernorm_full_size(jf, oracle):

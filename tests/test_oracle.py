@@ -50,7 +50,7 @@ def test_philox_reduced_rounds(oracle, ctr, key, want):
     assert _philox_py(ctr, key, 10) == want
     for rounds in range(0, 11):
         assert oracle.philox4x32(ctr, key, rounds).tolist() == _philox_py(ctr, key, rounds)
-    assert oracle.NOISE_ROUNDS == 7
+    assert oracle.NOISE_ROUNDS in (7, 8, 9, 10)      # follows the library under test (7 unless built otherwise)
 
 
 def test_sr_noise_layout_and_range(oracle):

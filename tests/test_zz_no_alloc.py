@@ -39,6 +39,7 @@ def _both(jf, A, B, sa, sb, a_km, splitk, out_dtype):
     out = torch.full((M, N), float("nan"), dtype=out_dtype, device="cuda")
     torch.cuda.synchronize()
     before = torch.cuda.memory_allocated()
+    free_before = torch.cuda.mem_get_info()[0]                 # the device's own count: sees a hipMalloc inside the library too
     L = jf.lib()
     print(f"noalloc M={M} N={N} K={K} a_km={a_km} splitk={splitk} {out_dtype}", flush=True)
     rc = L.jf_igemm_block_fp_noalloc(dA.data_ptr(), dB.data_ptr(), dsa.data_ptr(), dsb.data_ptr(), out.data_ptr(), M, N, K,
@@ -47,6 +48,7 @@ def _both(jf, A, B, sa, sb, a_km, splitk, out_dtype):
     assert rc == 0, L.jf_error_string(rc)
     torch.cuda.synchronize()
     assert torch.cuda.memory_allocated() == before
+    assert torch.cuda.mem_get_info()[0] >= free_before, "device memory was allocated during the call"
     return want, out
 
 
