@@ -261,6 +261,16 @@ int jf_add(const void *x1, int x1_dtype, const int8_t *q2, const void *s2, int R
            int scale_dtype, int rounding, uint64_t seed, uint64_t offset,
            void *y1, int y1_dtype, int8_t *q, void *s, float *rowsum, float *rowsq, jf_stream_t stream);
 
+/* out[c] = sum over all rows of q[r,c] * s[r/32,c/32] (fp32): the column sums of a block tensor, i.e. the bias gradient
+ * of a linear layer from its quantised output gradient (sketched in the reference as G8.sum(0),
+ * JetfireGEMMKernel/BlockQuantize/QBlockLinear.py:63-66).  Arithmetic, in a fixed order: per 32-row strip rb the term
+ * float(exact integer sum of the strip's 32 codes of column c) * s[rb, c/32]; lane g of 32 adds the terms of strips
+ * g, g+32, ... in ascending order starting from +0; the 32 partial sums are added in ascending g.
+ * workspace: jf_block_colsum_workspace_bytes(R, C) bytes of device scratch (the strip terms). */
+size_t jf_block_colsum_workspace_bytes(int R, int C);
+int jf_block_colsum(const int8_t *q, const void *s, int R, int C, int scale_dtype, float *out, void *workspace,
+                    size_t workspace_bytes, jf_stream_t stream);
+
 /* mean[r] = (sum of rowsum[0..parts-1, r], ascending) / C;  rstd[r] = 1 / sqrt((sum of rowsq[:, r]) / C - mean[r]^2)
  * (no epsilon): the finishing step of int8_add_Ifp_Ig16_Ofp_Og_MeanVar (Jetfire/Nonlinear/add_mean_var.py:219-221), which
  * the reference computes with torch operators on the kernel's partial sums.  rowsum, rowsq: [parts, R] fp32 as written by

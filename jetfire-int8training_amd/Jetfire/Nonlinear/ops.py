@@ -1,8 +1,9 @@
-"""The Nonlinear operators: thin shape handling over the C ABI (ctypes binding in jetfire_hip.py).
+"""The Nonlinear operators: shape handling over the C++ extension (BlockQuantizeCUDA.jetfire, csrc/jf_ops_ext.cpp), which
+validates the tensors, allocates the outputs and enqueues the gfx950 kernels through the C ABI with the GIL released.
 
 All functions accept 2-D [M,N] or 3-D [BS,T,N] operands like the reference launchers and return tensors
 of matching rank; scales are float16 [.., M/32, N/32] unless the inputs carry float32 scales.
-Stochastic rounding draws its Philox (seed, offset) from jetfire_hip.philox, which follows
+Stochastic rounding draws its Philox (seed, offset) from the device's default torch generator, so it follows
 torch.manual_seed (the reference materialises a uniform_(-0.5,0.5) noise tensor, quantize.py:143-146).
 """
 import os
@@ -14,7 +15,9 @@ _PKG = os.path.dirname(os.path.dirname(os.path.dirname(os.path.abspath(__file__)
 if _PKG not in sys.path:
     sys.path.insert(0, _PKG)
 
-import jetfire_hip as _jf  # noqa: E402
+import BlockQuantizeCUDA as _BQC  # noqa: E402
+
+_jf = _BQC.jetfire      # the operators below, as C++ functions on 2-D tensors
 
 from .common import SCALE_MIN_THRES  # noqa: E402
 
@@ -51,7 +54,7 @@ def int8_quantize(x, QB, stochastic=False, scale_dtype=torch.float16):
     """x fp32/fp16/bf16 -> (int8 codes, scales).  Reference: quantize.py:128-164."""
     _check_qb(QB)
     sh = _Shape(x)
-    q, s = _jf.quantize(sh.flat(x), _jf.ROUND_STOCHASTIC if stochastic else _jf.ROUND_NEAREST, scale_dtype)
+    q, s, _ = _jf.quantize(sh.flat(x), _jf.ROUND_STOCHASTIC if stochastic else _jf.ROUND_NEAREST, scale_dtype)
     return sh.fold(q), sh.fold(s)
 
 
@@ -66,8 +69,9 @@ def int8_quantize_concat(xs, QB, stochastic=False, scale_dtype=torch.float16):
         if x.dim() != xs[0].dim() or x.shape[:-1] != xs[0].shape[:-1]:
             raise RuntimeError("tensors to concatenate must agree in all but the last dimension")
         f = x.reshape(-1, x.shape[-1])                             # a view whenever the leading dimensions can be merged
-        flat.append(f if f.stride(1) == 1 and (f.stride(0) * f.element_size()) % 16 == 0 and f.data_ptr() % 16 == 0
-                    else f.contiguous())
+        in_place = (f.stride(1) == 1 and f.stride(0) >= f.shape[1]     # (an expanded gradient has row stride 0: copied)
+                    and (f.stride(0) * f.element_size()) % 16 == 0 and f.data_ptr() % 16 == 0)
+        flat.append(f if in_place else f.contiguous())
     q, s = _jf.quantize_slabs(flat, _jf.ROUND_STOCHASTIC if stochastic else _jf.ROUND_NEAREST, scale_dtype)
     return sh.fold(q), sh.fold(s)
 
@@ -76,8 +80,7 @@ def int8_quantize_transpose(x, QB, stochastic=False, transpose_output_2d=False, 
     """As int8_quantize, plus the transposed codes [N, M].  Reference: quantize_transpose.py:131-171."""
     _check_qb(QB)
     sh = _Shape(x)
-    q, s, qt = _jf.quantize(sh.flat(x), _jf.ROUND_STOCHASTIC if stochastic else _jf.ROUND_NEAREST, scale_dtype,
-                            transpose=True)
+    q, s, qt = _jf.quantize(sh.flat(x), _jf.ROUND_STOCHASTIC if stochastic else _jf.ROUND_NEAREST, scale_dtype, True)
     if sh.batched and not transpose_output_2d:
         qt = qt.reshape(sh.bs, -1, qt.shape[-1])
     return sh.fold(q), sh.fold(s), qt
@@ -96,7 +99,7 @@ def int8_dequantize(x, s_x, QB):
     """(codes, scales) -> float32.  Reference: dequantize.py:86-116."""
     _check_qb(QB)
     sh = _Shape(x)
-    return sh.fold(_jf.dequantize(sh.flat(x), sh.flat(s_x)))
+    return sh.fold(_jf.dequantize(sh.flat(x), sh.flat(s_x), torch.float32))
 
 
 def int8_rowstats(x, s_x, QB, eps=1e-5):
@@ -189,7 +192,7 @@ def int8_add_Ifp_Ig16_Ofp_Og(x1, x2, s_x2, QB, stochastic=False, rounding="trunc
     `.to()`, qmodel.py:228); y2, s_y2 are those of the fp32 sum either way."""
     _check_qb(QB)
     sh = _Shape(x1)
-    y1, q, s = _jf.add(sh.flat(x1), sh.flat(x2), sh.flat(s_x2), _add_rounding(stochastic, rounding), out_dtype=out_dtype)
+    y1, q, s, _, _ = _jf.add(sh.flat(x1), sh.flat(x2), sh.flat(s_x2), _add_rounding(stochastic, rounding), False, out_dtype)
     return sh.fold(y1), sh.fold(q), sh.fold(s)
 
 
@@ -198,7 +201,15 @@ def int8_add_Ifp_Ig16_Ofp_Og_MeanVar(x1, x2, s_x2, QB, rounding="trunc", out_dty
     rstd = 1/sqrt(var), no epsilon (reference: add_mean_var.py:179-230, finishing step :219-221)."""
     _check_qb(QB)
     sh = _Shape(x1)
-    y1, q, s, rowsum, rowsq = _jf.add(sh.flat(x1), sh.flat(x2), sh.flat(s_x2), _add_rounding(False, rounding),
-                                      with_stats=True, out_dtype=out_dtype)
-    mean, rstd = _jf.rowstats_finish(rowsum, rowsq, y1.shape[-1])     # one launch instead of eight torch operators
+    # the statistics are finished by a second kernel inside the same call (the reference: eight torch operators)
+    y1, q, s, mean, rstd = _jf.add(sh.flat(x1), sh.flat(x2), sh.flat(s_x2), _add_rounding(False, rounding), True, out_dtype)
     return sh.fold(y1), sh.fold(q), sh.fold(s), sh.fold_vec(mean), sh.fold_vec(rstd)
+
+
+def int8_column_sums(g, s_g, QB):
+    """Column sums over all rows of the block tensor (g, s_g), float32 [N]: the bias gradient of a linear layer from its
+    quantised output gradient (sketched in the reference as G8.sum(0), QBlockLinear.py:63-66).  3-D operands are summed
+    over both leading dimensions."""
+    _check_qb(QB)
+    sh = _Shape(g)
+    return _jf.block_colsum(sh.flat(g), sh.flat(s_g))

@@ -2,7 +2,8 @@
 
   libjetfire_hip.so        hipcc, gfx950 only: the HIP kernels behind the C ABI of include/jetfire_hip.h
   BlockQuantizeCUDA*.so    host C++ (g++): the PyTorch extension with the reference's module name and
-                           function signatures (JetfireGEMMKernel/setup.py:13, bindings.cpp:6-35); it is
+                           function signatures (JetfireGEMMKernel/setup.py:13, bindings.cpp:6-35), plus the
+                           submodule BlockQuantizeCUDA.jetfire with every other operator of the path; it is
                            compiled as plain C++ (no device code, nothing for hipify to rewrite) and
                            calls the HIP side only through the C ABI.
 
@@ -58,6 +59,9 @@ def build_hip():
     return HIP_LIB
 
 
+TORCH_SOURCES = ["bqc_ext.cpp", "jf_ops_ext.cpp"]
+
+
 def build_torch():
     import torch
     from torch.utils import cpp_extension as ce
@@ -68,17 +72,27 @@ def build_torch():
         inc += ["-isystem", p]
     inc += ["-isystem", os.path.join(ROCM, "include"), "-I", sysconfig.get_paths()["include"]]
     torch_lib = os.path.join(os.path.dirname(torch.__file__), "lib")
-    cmd = [
-        "g++", "-O2", "-std=c++17", "-fPIC", "-shared", "-Wall", "-Wno-unused-variable",
+    cflags = [
+        "g++", "-O2", "-std=c++17", "-fPIC", "-Wall", "-Wno-unused-variable",
         "-D__HIP_PLATFORM_AMD__=1", "-DUSE_ROCM=1", "-DTORCH_EXTENSION_NAME=BlockQuantizeCUDA",
         "-DTORCH_API_INCLUDE_EXTENSION_H", f"-D_GLIBCXX_USE_CXX11_ABI={int(torch._C._GLIBCXX_USE_CXX11_ABI)}",
-    ] + inc + [
-        os.path.join(CSRC, "bqc_ext.cpp"), "-o", out,
+    ] + inc
+    objdir = os.path.join(HERE, "build")
+    os.makedirs(objdir, exist_ok=True)
+    jobs = []
+    for src in TORCH_SOURCES:                                    # side by side: each takes most of a minute in the torch headers
+        obj = os.path.join(objdir, os.path.splitext(src)[0] + ".o")
+        cmd = cflags + ["-c", os.path.join(CSRC, src), "-o", obj]
+        print("+", " ".join(cmd), flush=True)
+        jobs.append((cmd, obj, subprocess.Popen(cmd)))
+    for cmd, obj, proc in jobs:
+        if proc.wait() != 0:
+            raise subprocess.CalledProcessError(proc.returncode, cmd)
+    _run(["g++", "-shared", "-o", out] + [obj for _, obj, _ in jobs] + [
         "-L" + torch_lib, "-L" + HERE, "-L" + os.path.join(ROCM, "lib"),
         "-ltorch", "-ltorch_cpu", "-lc10", "-ltorch_hip", "-lc10_hip", "-ltorch_python", "-ljetfire_hip", "-lamdhip64",
         "-Wl,-rpath,$ORIGIN", "-Wl,-rpath," + torch_lib, "-Wl,-rpath," + os.path.join(ROCM, "lib"),
-    ]
-    _run(cmd)
+    ])
     return out
 
 

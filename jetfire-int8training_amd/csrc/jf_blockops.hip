@@ -922,6 +922,30 @@ __global__ __launch_bounds__(1024) void layernorm_bwd_colsum_finish_kernel(const
     }
 }
 
+// Column sums of a block tensor's 32-row strips (the bias gradient of a linear layer is the column sum of its output
+// gradient; the reference sketches it as G8.sum(0), JetfireGEMMKernel/BlockQuantize/QBlockLinear.py:63-66).
+// strip term t[rb][c] = float(sum of the 32 codes of column c in row block rb) * s[rb][c/32]: the integer sum is exact,
+// the product rounds once.  One wave: 256 columns (4 per lane, whole 256-byte row segments) of one strip, all 32 row
+// loads in flight at once.  The strips' terms are then added by layernorm_bwd_colsum_finish_kernel in its fixed order.
+template <typename ST>
+__global__ __launch_bounds__(NT) void colsum_strip_kernel(const int8_t *q, const ST *s, int R, int C, float *terms)
+{
+    const int lane = threadIdx.x & 63, SC = C / QB, CG = (C + 255) / 256;
+    const int item = blockIdx.x * WPB + (threadIdx.x >> 6);        // (strip, 256-column group)
+    if (item >= (R / QB) * CG) return;
+    const int rb = item / CG, c0 = (item - rb * CG) * 256 + lane * 4;
+    if (c0 >= C) return;
+    const int8_t *src = q + (size_t)rb * QB * C + c0;
+    int w[QB];
+#pragma unroll
+    for (int i = 0; i < QB; ++i) w[i] = *reinterpret_cast<const int *>(src + (size_t)i * C);
+    int a0 = 0, a1 = 0, a2 = 0, a3 = 0;
+#pragma unroll
+    for (int i = 0; i < QB; ++i) { a0 += (w[i] << 24) >> 24; a1 += (w[i] << 16) >> 24; a2 += (w[i] << 8) >> 24; a3 += w[i] >> 24; }
+    const float sc = load_scale(s, rb * SC + c0 / QB);
+    *reinterpret_cast<v4f *>(terms + (size_t)rb * C + c0) = v4f{(float)a0 * sc, (float)a1 * sc, (float)a2 * sc, (float)a3 * sc};
+}
+
 // add.py:29-162 / add_mean_var.py:28-177
 // The sum leaves through a wave-private LDS patch in whole rows (store_block_rows).
 // rowsum / rowsq: [C/32][R] (a wave stores the 32 consecutive rows of its block).
@@ -1361,6 +1385,33 @@ int jf_rowstats_finish(const float *rowsum, const float *rowsq, int R, int parts
     hipLaunchKernelGGL(rowstats_finish_kernel, dim3((R + RSF_ROWS - 1) / RSF_ROWS), dim3(256),
                        (size_t)parts * RSF_ROWS * 2 * sizeof(float), (hipStream_t)stream, rowsum, rowsq, R, parts, (float)C,
                        mean, rstd);
+    return (int)hipGetLastError();
+}
+
+size_t jf_block_colsum_workspace_bytes(int R, int C)
+{
+    if (R <= 0 || C <= 0) return 0;
+    return (size_t)(R / QB) * (size_t)C * sizeof(float);
+}
+
+int jf_block_colsum(const int8_t *q, const void *s, int R, int C, int scale_dtype, float *out, void *workspace,
+                    size_t workspace_bytes, jf_stream_t stream)
+{
+    int rc = check_block_tensor(q, s, R, C, scale_dtype);
+    if (rc) return rc;
+    if (!out) return JF_ERR_NULL;
+    if (!workspace || workspace_bytes < jf_block_colsum_workspace_bytes(R, C)) return JF_ERR_WORKSPACE;
+    if (!aligned16(workspace)) return JF_ERR_ALIGN;
+    if (!device_is_gfx950()) return JF_ERR_DEVICE;
+    hipStream_t st = (hipStream_t)stream;
+    float *terms = (float *)workspace;
+    const int items = (R / QB) * ((C + 255) / 256);
+    if (scale_dtype == JF_SCALE_F16)
+        hipLaunchKernelGGL(colsum_strip_kernel<half_t>, dim3((items + WPB - 1) / WPB), dim3(NT), 0, st, q, (const half_t *)s, R, C, terms);
+    else
+        hipLaunchKernelGGL(colsum_strip_kernel<float>, dim3((items + WPB - 1) / WPB), dim3(NT), 0, st, q, (const float *)s, R, C, terms);
+    hipLaunchKernelGGL(layernorm_bwd_colsum_finish_kernel, dim3(C / QB, 1), dim3(1024), 0, st, terms, (const float *)nullptr, R / QB, C,
+                       out, (float *)nullptr);
     return (int)hipGetLastError();
 }
 

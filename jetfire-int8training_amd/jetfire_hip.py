@@ -29,7 +29,7 @@ EXPORTS = [
     "jf_igemm_splitk_plan", "jf_igemm_block_fp_workspace_bytes", "jf_igemm_block_q_gelu", "jf_igemm_block_fp_noalloc", "jf_igemm_block_q_gelu_bwd",
     "jf_igemm_block_q", "jf_quantize", "jf_dequantize", "jf_transpose_s8", "jf_rowstats", "jf_layernorm_fwd",
     "jf_layernorm_bwd_workspace_bytes", "jf_layernorm_bwd", "jf_layernorm_bwd_add", "jf_gelu_fwd", "jf_gelu_bwd", "jf_add", "jf_calibrate", "jf_wall_clock_khz", "jf_igemm_phase_record", "jf_rowstats_finish",
-    "jf_igemm_block_q_dequant", "jf_quantize_slabs", "jf_philox_rounds",
+    "jf_igemm_block_q_dequant", "jf_quantize_slabs", "jf_philox_rounds", "jf_block_colsum", "jf_block_colsum_workspace_bytes",
 ]
 
 _lib = None
@@ -75,6 +75,9 @@ def lib():
                                            _p, _i, _p, _p, _p, _p, _p, _sz, _p]
         L.jf_add.argtypes = [_p, _i, _p, _p, _i, _i, _i, _i, _u64, _u64, _p, _i, _p, _p, _p, _p, _p]
         L.jf_wall_clock_khz.argtypes = []
+        L.jf_block_colsum_workspace_bytes.argtypes = [_i, _i]
+        L.jf_block_colsum_workspace_bytes.restype = _sz
+        L.jf_block_colsum.argtypes = [_p, _p, _i, _i, _i, _p, _p, _sz, _p]
         L.jf_calibrate.argtypes = [_i, _i, _i, _i, _i, _i, _p, _p, _p]
         missing = [name for name in EXPORTS if not hasattr(L, name)]
         if missing:
@@ -541,6 +544,16 @@ def add(x1, q2, s2, rounding=ROUND_TRUNC, with_stats=False, seed=None, offset=No
     check(lib().jf_add(_ptr(x1), _FP_CODE[x1.dtype], _ptr(q2), _ptr(s2), R, Cc, code, rounding, seed, offset,
                        _ptr(y1), _FP_CODE[out_dtype], _ptr(q), _ptr(s), _ptr(rs), _ptr(rq), _stream()))
     return (y1, q, s, rs, rq) if with_stats else (y1, q, s)
+
+
+def block_colsum(q, s):
+    """fp32 column sums of the block tensor (q, s) over all rows (the bias gradient of a linear layer)."""
+    R, Cc, code = _block_tensor(q, s, "x")
+    nbytes = lib().jf_block_colsum_workspace_bytes(R, Cc)
+    ws = torch.empty(nbytes, dtype=torch.int8, device=q.device)
+    out = torch.empty(Cc, dtype=torch.float32, device=q.device)
+    check(lib().jf_block_colsum(_ptr(q), _ptr(s), R, Cc, code, _ptr(out), _ptr(ws), nbytes, _stream()))
+    return out
 
 
 def rowstats_finish(rowsum, rowsq, n_cols):

@@ -624,6 +624,35 @@ void jfo_add(const float *x1, const int8_t *q2, const float *s2, int R, int C,
     }
 }
 
+/*
+ * Column sums of a block tensor: out[c] = sum over all rows of q[r][c] * s[r/32][c/32] -- the bias gradient of a
+ * linear layer from its quantised output gradient (the reference only sketches it: grad_bias = G8.sum(0),
+ * JetfireGEMMKernel/BlockQuantize/QBlockLinear.py:63-66, which forgets the scales).  The order is this library's
+ * definition (an fp32 sum has to have one): per 32-row strip the exact integer sum of the column's codes times the
+ * strip's scale (one rounding); partial sum g of 32 adds the strips g, g+32, ... ascending from +0; the 32 partial
+ * sums are added ascending.
+ */
+void jfo_block_colsum(const int8_t *q, const float *s, int R, int C, float *out)
+{
+    int SC = C / QB, strips = R / QB;
+    #pragma omp parallel for schedule(static)
+    for (int c = 0; c < C; ++c) {
+        float part[32];
+        for (int g = 0; g < 32; ++g) {
+            float acc = 0.0f;
+            for (int rb = g; rb < strips; rb += 32) {
+                int isum = 0;
+                for (int i = 0; i < QB; ++i) isum += q[(size_t)(rb * QB + i) * C + c];
+                acc = acc + (float)isum * s[rb * SC + c / QB];
+            }
+            part[g] = acc;
+        }
+        float t = part[0];
+        for (int g = 1; g < 32; ++g) t = t + part[g];
+        out[c] = t;
+    }
+}
+
 /* ------------------------------------------------------------------------- */
 /* Model of the division shortcut the device kernels use for x/s with a        */
 /* block-constant s:  r = 1/s (IEEE), q0 = x*r, e = fmaf(-q0, s, x),            */

@@ -74,6 +74,7 @@ def _declare(L):
     L.jfo_layernorm_fwd.argtypes = [_p, _p, _i, _i, _p, _p, _p, _p, _p, _p]
     L.jfo_layernorm_bwd.argtypes = [_p, _p, _p, _p, _i, _i, _p, _p, _p, _i, _u64, _u64, _p, _p, _p, _p]
     L.jfo_add.argtypes = [_p, _p, _p, _i, _i, _i, _u64, _u64, _i, _p, _p, _p, _p, _p]
+    L.jfo_block_colsum.argtypes = [_p, _p, _i, _i, _p]
 
 
 def _ptr(a):
@@ -374,3 +375,14 @@ def add(x1, q2, s2, stochastic=False, seed=0, offset=0, truncate=True, with_stat
     if with_stats:
         return y1, q, _scale_out(s, scale_dtype), rs, rq
     return y1, q, _scale_out(s, scale_dtype)
+
+
+def block_colsum(q, s):
+    """Column sums of the block tensor (q, s) in fp32, in the library's fixed order (the bias gradient of a linear layer)."""
+    q = _c(q, np.int8)
+    s = _c(s, np.float32)
+    R, C_ = q.shape
+    _chk(R, C_)
+    out = np.empty(C_, np.float32)
+    lib().jfo_block_colsum(_ptr(q), _ptr(s), R, C_, _ptr(out))
+    return out

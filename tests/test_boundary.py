@@ -374,3 +374,144 @@ def test_linear_backward_with_fused_gelu_backward():
                                                wgrad_splitk=0)
         assert tuple(f8.shape) == (BS, T, Cin) and tuple(fs.shape) == (BS, T // 32, Cin // 32)
         assert torch.equal(f8, d8) and torch.equal(fs, ds) and torch.equal(fw, gw)
+
+
+@pytest.mark.gpu
+def test_linear_package_with_bias(oracle):
+    """bias through the Linear functions (sketched in the reference, QBlockLinear.py:38-39, 63-66): the forward adds it in
+    the requantising epilogue with biasmax = max|bias| (…BiasRowCol.cu:313,357), bit-exact against the oracle; the GELU
+    and dequantising epilogues take it as well; the backward returns the bias gradient = column sums of the gradient."""
+    from Linear import int8_linear_backward, int8_linear_backward_gelu, int8_linear_forward, int8_linear_forward_gelu
+    from Nonlinear import int8_column_sums, int8_dequantize, int8_gelu_forward, int8_quantize
+    torch.manual_seed(17)
+    BS, T, Cin, Cout = 2, 96, 160, 224
+    x = torch.randn(BS, T, Cin, device="cuda")
+    w = torch.randn(Cout, Cin, device="cuda") * 0.02
+    bias = torch.randn(Cout, device="cuda") * 0.3
+    g = torch.randn(BS, T, Cout, device="cuda") * 1e-3
+    qx, sx = int8_quantize(x, 32)
+    qw, sw = int8_quantize(w, 32)
+    o8, so = int8_linear_forward(qx, sx, qw, sw, True, 32, bias=bias)
+    sx2 = sx.reshape(-1, Cin // 32)
+    b = bias.cpu().numpy()
+    wq, ws = oracle.igemm_block_q(qx.reshape(-1, Cin).cpu().numpy(), qw.cpu().numpy(),
+                                  np.ascontiguousarray(sx2.float().cpu().numpy().T), np.ascontiguousarray(sw.float().cpu().numpy().T),
+                                  0, bias=b, biasmax=float(np.abs(b).max()), scale_dtype="f16")
+    assert eq(o8.reshape(-1, Cout), wq) and eq(so.reshape(-1, Cout // 32), ws)
+    o8_nobias, _ = int8_linear_forward(qx, sx, qw, sw, True, 32)
+    assert not torch.equal(o8, o8_nobias)
+    ref = x.reshape(-1, Cin) @ w.t() + bias
+    got = int8_dequantize(o8, so, 32).reshape(-1, Cout)
+    assert torch.nn.functional.cosine_similarity(got.reshape(-1), ref.reshape(-1), dim=0) > 0.999
+    # the unquantised output and the fused GELU see the same biased accumulator
+    ofp = int8_linear_forward(qx, sx, qw, sw, False, 32, bias=bias)
+    assert torch.equal(ofp, int8_dequantize(o8, so, 32).half())
+    f8, fs, fg8, fgs = int8_linear_forward_gelu(qx, sx, qw, sw, 32, bias=bias)
+    g8, gs = int8_gelu_forward(o8, so, 32)
+    assert torch.equal(f8, o8) and torch.equal(fs, so) and torch.equal(fg8, g8) and torch.equal(fgs, gs)
+    # bias gradient
+    qg, sg = int8_quantize(g, 32, stochastic=True)
+    torch.manual_seed(3)
+    gx8, gsx, gw = int8_linear_backward(qx, sx, qg, sg, None, qw, sw, 32)
+    torch.manual_seed(3)
+    gx8b, gsxb, gwb, gb = int8_linear_backward(qx, sx, qg, sg, None, qw, sw, 32, bias_grad=True)
+    assert torch.equal(gx8, gx8b) and torch.equal(gsx, gsxb) and torch.equal(gw, gwb)
+    want = oracle.block_colsum(qg.reshape(-1, Cout).cpu().numpy(), sg.reshape(-1, Cout // 32).float().cpu().numpy())
+    assert gb.dtype == torch.float32 and np.array_equal(gb.cpu().numpy().view(np.uint32), want.view(np.uint32))
+    assert torch.equal(gb, int8_column_sums(qg, sg, 32))
+    ref_gb = int8_dequantize(qg, sg, 32).reshape(-1, Cout).double().sum(0)
+    assert torch.allclose(gb.double(), ref_gb, rtol=1e-4, atol=1e-7)
+    out = int8_linear_backward(qx, sx, qg, sg, None, qw, sw, 32, dgrad_quantize=False, bias_grad=True)
+    assert len(out) == 3 and torch.equal(out[2], gb)
+    pre8, spre = int8_quantize(torch.randn(BS, T, Cin, device="cuda"), 32)
+    out = int8_linear_backward_gelu(qx, sx, qg, sg, qw, sw, pre8, spre, 32, bias_grad=True)
+    assert len(out) == 4 and torch.equal(out[3], gb)
+    with pytest.raises(RuntimeError, match="elements"):
+        int8_linear_forward(qx, sx, qw, sw, True, 32, bias=bias[:-1])
+
+
+@pytest.mark.gpu
+def test_packages_run_through_the_cpp_extension(oracle):
+    """Every operator of Linear / Nonlinear is a function of the C++ extension (BlockQuantizeCUDA and its submodule
+    `jetfire`): the ctypes binding of the C ABI, which the kernel tests use, gives the same bits on the same (seed, offset),
+    and the extension rejects bad operands itself."""
+    import BlockQuantizeCUDA as BQC
+    import jetfire_hip as jf
+    import Linear.linear as L
+    import Nonlinear.ops as N
+    J = BQC.jetfire
+    assert N._jf is J and L._jf is J and L.BQC is BQC
+    for mod in (N, L):
+        assert "jetfire_hip" not in vars(mod), "the packages must not call the ctypes binding"
+    torch.manual_seed(5)
+    R, C = 128, 160
+    x = torch.randn(R, C, device="cuda")
+    q, s, qT = J.quantize(x, J.ROUND_STOCHASTIC, torch.float16, True, 0.0, 9, 4)
+    q2, s2, qT2 = jf.quantize(x, jf.ROUND_STOCHASTIC, torch.float16, transpose=True, seed=9, offset=4)
+    assert torch.equal(q, q2) and torch.equal(s, s2) and torch.equal(qT, qT2)
+    g, sg, _ = J.quantize(torch.randn(R, C, device="cuda") * 1e-3, J.ROUND_NEAREST, torch.float16)
+    a = J.gelu_bwd(q, s, g, sg, J.GELU_TANH, J.ROUND_STOCHASTIC, 3, 8)
+    b = jf.gelu_bwd(q, s, g, sg, jf.GELU_TANH, jf.ROUND_STOCHASTIC, seed=3, offset=8)
+    assert torch.equal(a[0], b[0]) and torch.equal(a[1], b[1])
+    mean, rstd = J.rowstats(q, s, 1e-5)
+    gamma = 1 + 0.1 * torch.randn(C, device="cuda")
+    x1 = torch.randn(R, C, device="cuda").bfloat16()
+    a = J.layernorm_bwd_add(q, s, g, sg, gamma, mean, rstd, x1, J.ROUND_STOCHASTIC, J.ROUND_STOCHASTIC_TRUNC, True, torch.bfloat16,
+                            1, 0, 2, 4)
+    b = jf.layernorm_bwd_add(q, s, g, sg, gamma, mean, rstd, x1, jf.ROUND_STOCHASTIC, jf.ROUND_STOCHASTIC_TRUNC, True, torch.bfloat16,
+                             seed=1, offset=0, add_seed=2, add_offset=4)
+    for u, v in zip(a, b):
+        assert torch.equal(u, v)
+    y1, qa, sa, m2, r2 = J.add(x1, q, s, J.ROUND_TRUNC, True, torch.float32)
+    y1b, qab, sab, rs, rq = jf.add(x1, q, s, jf.ROUND_TRUNC, with_stats=True)
+    mb, rb = jf.rowstats_finish(rs, rq, C)
+    assert torch.equal(y1, y1b) and torch.equal(qa, qab) and torch.equal(m2, mb) and torch.equal(r2, rb)
+    # no seed given: counters come from the device's generator, under its mutex, and advance
+    torch.manual_seed(21)
+    before = BQC.philox_peek(0)
+    J.quantize(x, J.ROUND_STOCHASTIC)
+    assert BQC.philox_peek(0) == (21, before[1] + R * C // 8)
+    # operand errors are the extension's own
+    with pytest.raises(RuntimeError, match="int8"):
+        J.gelu_fwd(x, s)
+    with pytest.raises(RuntimeError, match="scale shape"):
+        J.gelu_fwd(q, s[:1])
+    with pytest.raises(RuntimeError, match="rounding"):
+        J.quantize(x, 7)
+    with pytest.raises(RuntimeError, match="contiguous"):
+        J.dequantize(q.t(), s)
+    with pytest.raises(RuntimeError, match="float32 vector"):
+        J.layernorm_fwd(q, s, gamma.half(), None, mean, rstd)
+    with pytest.raises(RuntimeError, match="come together"):
+        J.igemm_block_q(q, q, s.t(), s.t(), J.B_NK, gamma, None)
+
+
+def test_expanded_gradient_is_copied_not_rejected():
+    """int8_quantize_concat reads slabs where they lie only when their rows do not overlap: an expanded gradient (row stride
+    0) is made contiguous first (CPU check of the rule; the tensors never reach a kernel here)."""
+    import Nonlinear.ops as N
+    seen = {}
+
+    class Fake:
+        ROUND_NEAREST, ROUND_STOCHASTIC = 0, 1
+
+        @staticmethod
+        def quantize_slabs(flat, rounding, scale_dtype):
+            seen["flat"] = flat
+            R = flat[0].shape[0]
+            Ct = sum(f.shape[1] for f in flat)
+            return torch.zeros(R, Ct, dtype=torch.int8), torch.zeros(R // 32, Ct // 32, dtype=scale_dtype)
+
+    real = N._jf
+    N._jf = Fake
+    try:
+        a = torch.randn(64, 32)
+        b = torch.randn(1, 32).expand(64, 32)                       # stride (0, 1)
+        c = torch.randn(64, 96)[:, 32:64]                            # a column slab of a wider tensor: read in place
+        q, s = N.int8_quantize_concat([a, b, c], 32)
+    finally:
+        N._jf = real
+    fa, fb, fc = seen["flat"]
+    assert fb.stride(0) == 32 and fb.is_contiguous() and torch.equal(fb, b)
+    assert fa.data_ptr() == a.data_ptr() and fc.data_ptr() == c.data_ptr() and fc.stride(0) == 96
+    assert tuple(q.shape) == (64, 96) and tuple(s.shape) == (2, 3)

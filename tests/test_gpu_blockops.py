@@ -361,3 +361,18 @@ def test_random_shapes(jf, oracle, R, C, f16, approx):
     test_gelu_fwd_bwd(jf, oracle, R, C, approx, 5e-5 if approx == 0 else 0.0, f16)
     test_rowstats_layernorm(jf, oracle, R, C, f16)
     test_quantize(jf, oracle, R, C, "stochastic", f16)
+
+
+@pytest.mark.parametrize("R,C", [(32, 32), (96, 160), (2080, 288), (8192 + 64, 1600), (12288, 768)])
+@pytest.mark.parametrize("f16", [True, False])
+def test_block_column_sums(jf, oracle, R, C, f16):
+    """jf_block_colsum (the bias gradient) against the oracle's restatement of its summation order, bit for bit; shapes
+    with fewer strips than partial sums, strip counts that are not multiples of 32 or 256, widths that are not multiples
+    of the 256 columns a wave takes."""
+    rng = np.random.default_rng(R + C)
+    q = rand_codes(rng, (R, C), sparse=0.1)
+    s = rand_scales(rng, (R // QB, C // QB), f16=f16)
+    ds = torch.from_numpy(s).cuda()
+    got = jf.block_colsum(torch.from_numpy(q).cuda(), ds.half() if f16 else ds)
+    want = oracle.block_colsum(q, s)
+    assert np.array_equal(got.cpu().numpy().view(np.uint32), want.view(np.uint32))

@@ -470,3 +470,31 @@ def test_add_closed_form(oracle):
     mean = rs.sum(axis=0) / Cc
     var = rq.sum(axis=0) / Cc - mean ** 2
     assert np.allclose(var, w64.var(axis=1), rtol=1e-4)
+
+
+def test_block_column_sums(oracle):
+    """Column sums of a block tensor (the bias gradient): against float64 sums of the dequantised tensor; exactly, where
+    every step of the fixed order is exact (scales that are powers of two: terms and partial sums are small integers
+    times a power of two); and against an independent numpy restatement of the order (strip terms, 32 interleaved
+    partial sums, ascending) on general data."""
+    rng = np.random.default_rng(41)
+    for R, Cc in ((32, 32), (96, 160), (1120, 64), (8192 + 32, 96)):
+        q, s = _rand_block_tensor(rng, R, Cc, 0.3)
+        got = oracle.block_colsum(q, s)
+        deq = q.astype(np.float64) * expand_scales(s).astype(np.float64)
+        assert np.allclose(got, deq.sum(axis=0), rtol=2e-5, atol=1e-5 * np.abs(deq).sum(axis=0).max())
+        # the order, restated with numpy float32 scalars
+        strips = R // 32
+        terms = q.reshape(strips, 32, Cc).astype(np.int64).sum(axis=1).astype(np.float32) * np.repeat(s, 32, axis=1)
+        parts = np.zeros((32, Cc), np.float32)
+        for g in range(32):
+            for rb in range(g, strips, 32):
+                parts[g] = parts[g] + terms[rb]
+        want = parts[0].copy()
+        for g in range(1, 32):
+            want = want + parts[g]
+        assert np.array_equal(got.view(np.uint32), want.view(np.uint32))
+        # exact case
+        s2 = np.exp2(rng.integers(-6, 3, size=s.shape)).astype(np.float32)
+        exact = (q.astype(np.int64) * expand_scales(s2).astype(np.float64)).sum(axis=0)
+        assert np.array_equal(oracle.block_colsum(q, s2).astype(np.float64), exact)
