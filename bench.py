@@ -115,8 +115,8 @@ def dominant_kernel_roofline(jf, torch, ops, iters=200):
     return {"bound": "mfma", "kernel": "igemm_nt_kernel<EPI_Q,f32> fc forward 8192x6400x1600",
             "achieved": round(achieved, 2), "peak": INT8_PEAK_TOPS, "unit": "TOP/s",
             "frac": round(achieved / INT8_PEAK_TOPS, 4), "avg_launch_us": round(avg_s * 1e6, 2),
-            "launches": iters, "traffic": PROFILED_TRAFFIC_BYTES, "traffic_source": PROFILED_TRAFFIC_SOURCE,
-            "phases": phases}
+            "launches": iters, "traffic": PROFILED_TRAFFIC_BYTES, "traffic_carried_from_profile": True,
+            "traffic_source": PROFILED_TRAFFIC_SOURCE, "phases": phases}
 
 
 def fused_fc_gelu(jf, torch, ops):
@@ -186,8 +186,9 @@ def deep_k_weight_gradients(jf, torch):
     return out
 
 
-def recipe_block(torch, only=None):
-    """GPT-2 XL transformer blocks (1600 wide, 25 heads) forward + backward on 8 x 1024 tokens: the INT8 data-flow
+def recipe_block(torch, only=None, shape=(8, 1024, 1600, 25)):
+    """Transformer blocks forward + backward, by default GPT-2 XL's (1600 wide, 25 heads) on 8 x 1024 tokens; shape =
+    (12, 1024, 768, 12) is GPT-2 small's on 12288 tokens, where kernels are short and host overhead shows: the INT8 data-flow
     recipe (Jetfire/recipe.py: every linear layer, LayerNorm, GELU and residual add on INT8 block tensors, attention
     itself in fp16 through torch) next to the same blocks in plain torch bf16.  Measured for a stack of one block (which
     includes the stack's own begin / end: quantising the input, its row statistics, quantising the output gradient) and
@@ -200,7 +201,7 @@ def recipe_block(torch, only=None):
     sys.path.insert(0, os.path.join(PKG, "Jetfire"))
     from recipe import QStack, weight_codes
     torch.manual_seed(0)
-    B, T, C, H = 8, 1024, 1600, 25
+    B, T, C, H = shape
     x = torch.randn(B, T, C, device="cuda", requires_grad=True)
     w = torch.randn(B, T, C, device="cuda")
     xr, wr = x.detach().to(torch.bfloat16).requires_grad_(True), w.to(torch.bfloat16)
@@ -308,8 +309,28 @@ def nonlinear_extras(jf, torch):
     g = torch.Generator().manual_seed(0)
     S = torch.float32
     out = {}
-    def put(name, secs, nbytes):
+    COLD_BYTES = 320 << 20         # more than the 256 MiB Infinity Cache between two uses of the same bytes
+
+    def put(name, secs, nbytes, cold=None):
+        """cold = (fn(inputs), inputs): the same call timed again while rotating over as many clones of its input tensors
+        as it takes for COLD_BYTES of other operands to pass between two uses of a clone (outputs are fresh buffers in
+        either measurement), so that every byte comes from and goes to HBM: GB/s_cold / frac_cold.  The first figures
+        replay one set of inputs (<= 157 MB, cache-warm reads): an upper bound."""
         out[name] = {"GB/s": round(nbytes / secs / 1e9, 1), "us": round(secs * 1e6, 1), "frac_of_8TB/s": round(nbytes / secs / 8e12, 3)}
+        if cold is not None:
+            fn, inputs = cold
+            in_bytes = sum(t.numel() * t.element_size() for t in inputs)
+            sets = [inputs] + [tuple(t.clone() for t in inputs) for _ in range(max(2, -(-COLD_BYTES // max(in_bytes, 1))))]
+            state = {"i": 0}
+
+            def rotating():
+                fn(*sets[state["i"] % len(sets)])
+                state["i"] += 1
+            n = 2 * len(sets)
+            state["i"] = 0
+            secs_cold = t(rotating, n=n, replays=3)
+            out[name].update({"us_cold": round(secs_cold * 1e6, 1), "GB/s_cold": round(nbytes / secs_cold / 1e9, 1),
+                              "frac_cold": round(nbytes / secs_cold / 8e12, 3), "input_sets": len(sets)})
     R, C = TOKENS, 1600
     x = torch.randn(R, C, generator=g).cuda()
     dy = (torch.randn(R, C, generator=g) * 1e-3).cuda()
@@ -319,34 +340,85 @@ def nonlinear_extras(jf, torch):
     qg, sg = jf.quantize(dy, jf.ROUND_STOCHASTIC, S, seed=0, offset=0)
     mean, rstd = jf.rowstats(qx, sx)
     n = R * C
-    put("quantize_f32_8192x1600", t(lambda: jf.quantize(x, scale_dtype=S)), 5 * n)
-    put("quantize_transpose_sr_8192x1600", t(lambda: jf.quantize(x, jf.ROUND_STOCHASTIC, S, transpose=True, seed=1, offset=0)), 6 * n)
-    put("transpose_8192x1600", t(lambda: jf.transpose_s8(qx)), 2 * n)
-    put("layernorm_fwd_8192x1600", t(lambda: jf.layernorm_fwd(qx, sx, gamma, beta, mean, rstd)), 2 * n)
-    put("layernorm_bwd_sr_8192x1600", t(lambda: jf.layernorm_bwd(qx, sx, qg, sg, gamma, mean, rstd, jf.ROUND_STOCHASTIC, seed=1, offset=0)), 3 * n)
+    f = lambda x_: jf.quantize(x_, scale_dtype=S)
+    put("quantize_f32_8192x1600", t(lambda: f(x)), 5 * n, (f, (x,)))
+    f = lambda x_: jf.quantize(x_, jf.ROUND_STOCHASTIC, S, transpose=True, seed=1, offset=0)
+    put("quantize_transpose_sr_8192x1600", t(lambda: f(x)), 6 * n, (f, (x,)))
+    f = lambda q_: jf.transpose_s8(q_)
+    put("transpose_8192x1600", t(lambda: f(qx)), 2 * n, (f, (qx,)))
+    f = lambda q_, s_: jf.layernorm_fwd(q_, s_, gamma, beta, mean, rstd)
+    put("layernorm_fwd_8192x1600", t(lambda: f(qx, sx)), 2 * n, (f, (qx, sx)))
+    f = lambda q_, s_, g_, sg_: jf.layernorm_bwd(q_, s_, g_, sg_, gamma, mean, rstd, jf.ROUND_STOCHASTIC, seed=1, offset=0)
+    put("layernorm_bwd_sr_8192x1600", t(lambda: f(qx, sx, qg, sg)), 3 * n, (f, (qx, sx, qg, sg)))
     # residual add: fp32 in + codes in, fp32 out + codes out (the reference's default truncation; the backward's stochastic
     # form; the forward's form with the row partial sums and their finishing launch)
-    put("add_8192x1600", t(lambda: jf.add(x, qx, sx, jf.ROUND_TRUNC)), 10 * n)
-    put("add_sr_8192x1600", t(lambda: jf.add(x, qx, sx, jf.ROUND_STOCHASTIC_TRUNC, seed=1, offset=0)), 10 * n)
-    put("add_meanvar_8192x1600", t(lambda: jf.rowstats_finish(*jf.add(x, qx, sx, jf.ROUND_TRUNC, with_stats=True)[3:], C)), 10 * n)
+    f = lambda x_, q_, s_: jf.add(x_, q_, s_, jf.ROUND_TRUNC)
+    put("add_8192x1600", t(lambda: f(x, qx, sx)), 10 * n, (f, (x, qx, sx)))
+    f = lambda x_, q_, s_: jf.add(x_, q_, s_, jf.ROUND_STOCHASTIC_TRUNC, seed=1, offset=0)
+    put("add_sr_8192x1600", t(lambda: f(x, qx, sx)), 10 * n, (f, (x, qx, sx)))
+    f = lambda x_, q_, s_: jf.rowstats_finish(*jf.add(x_, q_, s_, jf.ROUND_TRUNC, with_stats=True)[3:], C)
+    put("add_meanvar_8192x1600", t(lambda: f(x, qx, sx)), 10 * n, (f, (x, qx, sx)))
     # LayerNorm backward with the residual add behind it in one kernel (what the recipe's backward runs), fp32 / bfloat16
     # gradient in and out: codes of x and dy in; the fp gradient in; the sum and its codes out
     xb = x.to(torch.bfloat16)
-    put("layernorm_bwd_add_sr_8192x1600", t(lambda: jf.layernorm_bwd_add(qx, sx, qg, sg, gamma, mean, rstd, x, jf.ROUND_STOCHASTIC,
-        jf.ROUND_STOCHASTIC_TRUNC, seed=1, offset=0, add_seed=2, add_offset=0)), 11 * n)
-    put("layernorm_bwd_add_sr_bf16_8192x1600", t(lambda: jf.layernorm_bwd_add(qx, sx, qg, sg, gamma, mean, rstd, xb, jf.ROUND_STOCHASTIC,
-        jf.ROUND_STOCHASTIC_TRUNC, out_dtype=torch.bfloat16, seed=1, offset=0, add_seed=2, add_offset=0)), 7 * n)
+    f = lambda q_, s_, g_, sg_, x_: jf.layernorm_bwd_add(q_, s_, g_, sg_, gamma, mean, rstd, x_, jf.ROUND_STOCHASTIC,
+                                                         jf.ROUND_STOCHASTIC_TRUNC, seed=1, offset=0, add_seed=2, add_offset=0)
+    put("layernorm_bwd_add_sr_8192x1600", t(lambda: f(qx, sx, qg, sg, x)), 11 * n, (f, (qx, sx, qg, sg, x)))
+    f = lambda q_, s_, g_, sg_, x_: jf.layernorm_bwd_add(q_, s_, g_, sg_, gamma, mean, rstd, x_, jf.ROUND_STOCHASTIC,
+                                                         jf.ROUND_STOCHASTIC_TRUNC, out_dtype=torch.bfloat16, seed=1, offset=0,
+                                                         add_seed=2, add_offset=0)
+    put("layernorm_bwd_add_sr_bf16_8192x1600", t(lambda: f(qx, sx, qg, sg, xb)), 7 * n, (f, (qx, sx, qg, sg, xb)))
+    f = lambda g_, sg_: jf.block_colsum(g_, sg_)
+    put("bias_gradient_colsum_8192x1600", t(lambda: f(qg, sg)), n, (f, (qg, sg)))
     R, C = TOKENS, 6400
     x = torch.randn(R, C, generator=g).cuda()
     dy = (torch.randn(R, C, generator=g) * 1e-3).cuda()
     qx, sx = jf.quantize(x, scale_dtype=S)
     qg, sg = jf.quantize(dy, jf.ROUND_STOCHASTIC, S, seed=0, offset=0)
     n = R * C
-    put("gelu_fwd_tanh_8192x6400", t(lambda: jf.gelu_fwd(qx, sx, jf.GELU_TANH, 0.0)), 2 * n)
-    put("gelu_fwd_erf_8192x6400", t(lambda: jf.gelu_fwd(qx, sx, jf.GELU_ERF, 5e-5)), 2 * n)
-    put("gelu_bwd_tanh_sr_8192x6400", t(lambda: jf.gelu_bwd(qx, sx, qg, sg, jf.GELU_TANH, jf.ROUND_STOCHASTIC, seed=1, offset=0)), 3 * n)
-    put("gelu_bwd_erf_sr_8192x6400", t(lambda: jf.gelu_bwd(qx, sx, qg, sg, jf.GELU_ERF, jf.ROUND_STOCHASTIC, seed=1, offset=0)), 3 * n)
+    del x, dy
+    f = lambda q_, s_: jf.gelu_fwd(q_, s_, jf.GELU_TANH, 0.0)
+    put("gelu_fwd_tanh_8192x6400", t(lambda: f(qx, sx)), 2 * n, (f, (qx, sx)))
+    f = lambda q_, s_: jf.gelu_fwd(q_, s_, jf.GELU_ERF, 5e-5)
+    put("gelu_fwd_erf_8192x6400", t(lambda: f(qx, sx)), 2 * n, (f, (qx, sx)))
+    f = lambda q_, s_, g_, sg_: jf.gelu_bwd(q_, s_, g_, sg_, jf.GELU_TANH, jf.ROUND_STOCHASTIC, seed=1, offset=0)
+    put("gelu_bwd_tanh_sr_8192x6400", t(lambda: f(qx, sx, qg, sg)), 3 * n, (f, (qx, sx, qg, sg)))
+    f = lambda q_, s_, g_, sg_: jf.gelu_bwd(q_, s_, g_, sg_, jf.GELU_ERF, jf.ROUND_STOCHASTIC, seed=1, offset=0)
+    put("gelu_bwd_erf_sr_8192x6400", t(lambda: f(qx, sx, qg, sg)), 3 * n, (f, (qx, sx, qg, sg)))
+    out["note"] = ("GB/s = algorithmic bytes / time.  The first figures replay one set of input tensors (reads served by the "
+                   "256 MiB Infinity Cache where they fit): an upper bound.  *_cold rotate over clones of the inputs so that every "
+                   "byte comes from HBM: the figure the 70 %-of-HBM target is judged on.")
     return out
+
+
+def host_call_overhead(jf, torch):
+    """Host microseconds per operator call on operands so small that the GPU never is the bottleneck (one 32 x 32 block):
+    the Python ctypes binding of the C ABI (what the Nonlinear package called before) against the C++ extension (what it
+    calls now), and the package-level functions on top of the extension."""
+    sys.path.insert(0, os.path.join(PKG, "Jetfire"))
+    import BlockQuantizeCUDA as BQC
+    from Nonlinear import int8_gelu_forward, int8_quantize
+    J = BQC.jetfire
+    x = torch.randn(32, 32, device="cuda")
+    q, s = jf.quantize(x)
+
+    def per_call(fn, n=2000):
+        for _ in range(50):
+            fn()
+        torch.cuda.synchronize()
+        t0 = time.perf_counter()
+        for _ in range(n):
+            fn()
+        dt = time.perf_counter() - t0
+        torch.cuda.synchronize()
+        return round(dt / n * 1e6, 2)
+    return {"gelu_fwd": {"ctypes_binding_us": per_call(lambda: jf.gelu_fwd(q, s)), "cpp_extension_us": per_call(lambda: J.gelu_fwd(q, s)),
+                         "Nonlinear.int8_gelu_forward_us": per_call(lambda: int8_gelu_forward(q, s, 32))},
+            "quantize": {"ctypes_binding_us": per_call(lambda: jf.quantize(x)), "cpp_extension_us": per_call(lambda: J.quantize(x)),
+                         "Nonlinear.int8_quantize_us": per_call(lambda: int8_quantize(x, 32))},
+            "quantize_stochastic": {"ctypes_binding_us": per_call(lambda: jf.quantize(x, jf.ROUND_STOCHASTIC)),
+                                    "cpp_extension_us": per_call(lambda: J.quantize(x, J.ROUND_STOCHASTIC))},
+            "note": "wall time of back-to-back calls on one 32x32 block (launch-bound on the host side), 2000 calls"}
 
 
 def calibration(jf, torch):
@@ -569,7 +641,9 @@ def main():
         print(json.dumps({"calibration": calibration(jf, torch)}))
         return
     if a.block_only:
-        print(json.dumps({"xl_block_forward_backward": recipe_block(torch)}))
+        print(json.dumps({"xl_block_forward_backward": recipe_block(torch),
+                          "gpt2_small_block_forward_backward": recipe_block(torch, shape=(12, 1024, 768, 12)),
+                          "host_call_overhead": host_call_overhead(jf, torch)}))
         return
     if a.stack_only:
         print(json.dumps({"stack_of_3_blocks_ms": recipe_block(torch, only=a.stack_only)}))
@@ -621,13 +695,21 @@ def main():
         "roofline": roof,
     }
     if not a.no_extras:
-        out["calibration"] = calibration(jf, torch)
+        out["calibration"] = cal = calibration(jf, torch)
+        # the dominant kernel against what any kernel with these semantics can reach (the register-only K-block stream at
+        # the clock it sustains on changing operands, and, in cycles, at an unchanged clock)
+        roof["frac_of_calibrated_ceiling"] = round(roof["achieved"] / cal["ceiling_TOPs_k_block_stream_changing_operands"], 3)
+        stream_cycles = [r["cycles"] for r in cal["rows"] if r["case"] == "gemm_k_block_stream" and r["waves_per_simd"] == 4]
+        if stream_cycles:
+            roof["frac_of_calibrated_ceiling_in_cycles"] = round(stream_cycles[0] / roof["phases"]["simd_cycles_per_block_product"], 3)
         out["other_configurations"] = other_configurations(jf, torch)
         out["memory_bound_kernels"] = nonlinear_extras(jf, torch)
         out["deep_k_weight_gradients"] = deep_k_weight_gradients(jf, torch)
         out["fc_forward_with_gelu"] = fused_fc_gelu(jf, torch, ops)
         out["fc2_dgrad_with_gelu_backward"] = fused_fc2_dgrad_gelu_bwd(jf, torch, ops)
         out["xl_block_forward_backward"] = recipe_block(torch)
+        out["gpt2_small_block_forward_backward"] = recipe_block(torch, shape=(12, 1024, 768, 12))
+        out["host_call_overhead"] = host_call_overhead(jf, torch)
     if not a.no_cpu:
         out["cpu_baseline"] = cpu_baseline(ops, a.cpu_rows)
     print(json.dumps(out))

@@ -12,12 +12,12 @@ def ref_block(x, blk):
     C = x.shape[-1]
     B, T, _ = x.shape
     h = F.layer_norm(x, (C,), blk.ln_1, None, 0.0)
-    qkv = h @ blk.w_qkv.t()
+    qkv = F.linear(h, blk.w_qkv, blk.b_qkv)
     q, k, v = (t.view(B, T, blk.n_head, C // blk.n_head).transpose(1, 2) for t in qkv.split(C, dim=2))
     y = F.scaled_dot_product_attention(q, k, v, is_causal=True).transpose(1, 2).contiguous().view(B, T, C)
-    x = x + y @ blk.w_attn_proj.t()
+    x = x + F.linear(y, blk.w_attn_proj, blk.b_attn_proj)
     h = F.layer_norm(x, (C,), blk.ln_2, None, 0.0)
-    return x + F.gelu(h @ blk.w_fc.t()) @ blk.w_mlp_proj.t()
+    return x + F.linear(F.gelu(F.linear(h, blk.w_fc, blk.b_fc)), blk.w_mlp_proj, blk.b_mlp_proj)
 
 
 def cos(a, b):
@@ -50,6 +50,47 @@ def test_one_block_matches_fp32_reference():
     for n, p in model.named_parameters():
         assert got[n].shape == p.shape and got[n].dtype == p.dtype
         assert cos(got[n], p.grad) > 0.97, n
+
+
+def test_block_with_linear_biases_matches_fp32_reference():
+    """QBlock(bias=True): the four biases enter in the GEMM epilogues and their gradients are the column sums of the
+    layers' quantised output gradients; against the fp32 block with the same biases."""
+    from recipe import QStack
+    torch.manual_seed(4)
+    B, T, C, H = 2, 128, 256, 4
+    model = QStack(1, C, H, bias=True).cuda()
+    names = [n for n, _ in model.named_parameters()]
+    assert sum(".b_" in n for n in names) == 4
+    with torch.no_grad():
+        for n, p in model.named_parameters():
+            if p.dim() == 1:
+                p.add_((0.3 if ".b_" in n else 0.1) * torch.randn_like(p))
+    x = torch.randn(B, T, C, device="cuda", requires_grad=True)
+    w = torch.randn(B, T, C, device="cuda")
+    out = model(x)
+    (out * w).sum().backward()
+    got = {n: p.grad.clone() for n, p in model.named_parameters()}
+    gx = x.grad.clone()
+    for p in model.parameters():
+        p.grad = None
+    x2 = x.detach().clone().requires_grad_(True)
+    ref = ref_block(x2, model.blocks[0])
+    (ref * w).sum().backward()
+    assert cos(out, ref) > 0.999
+    assert cos(gx, x2.grad) > 0.99
+    for n, p in model.named_parameters():
+        assert got[n].shape == p.shape and got[n].dtype == p.dtype
+        assert cos(got[n], p.grad) > (0.99 if ".b_" in n else 0.97), (n, cos(got[n], p.grad))
+    # without the biases the output differs: they are really applied
+    with torch.no_grad():
+        saved = [p.clone() for n, p in model.named_parameters() if ".b_" in n]
+        for n, p in model.named_parameters():
+            if ".b_" in n:
+                p.zero_()
+        assert cos(model(x), ref) < 0.999
+        for (n, p), v in zip([(n, p) for n, p in model.named_parameters() if ".b_" in n], saved):
+            p.copy_(v)
+        assert torch.equal(model(x), out)                          # cached bias operands follow the parameter's version
 
 
 def test_xl_width_block_matches_fp32_reference():
