@@ -603,20 +603,23 @@ __global__ __launch_bounds__(NT) void layernorm_bwd_stats_kernel(const int8_t *q
     }
 }
 
-// 64-lane sum, every lane returns it (data-parallel-primitive moves; a fixed tree)
+// 64-lane sum, every lane returns it (data-parallel-primitive forms of v_add_f32; a fixed tree: pairs, quads, eights,
+// rows of 16, then row 1 += row 0 and row 3 += row 2, then rows 2-3 += rows 0-1; asm for the reason given at wave_max)
 __device__ __forceinline__ float wave_sum(float v)
 {
-    auto step = [](float x, auto ctrl_c, auto rows_c) {
-        const int t = __builtin_amdgcn_update_dpp(0, __float_as_int(x), decltype(ctrl_c)::value, decltype(rows_c)::value, 0xF, false);
-        return x + __int_as_float(t);
-    };
-    using all = std::integral_constant<int, 0xF>;
-    v = step(v, std::integral_constant<int, 0xB1>{}, all{});
-    v = step(v, std::integral_constant<int, 0x4E>{}, all{});
-    v = step(v, std::integral_constant<int, 0x141>{}, all{});
-    v = step(v, std::integral_constant<int, 0x140>{}, all{});      // every lane: the sum of its 16-lane row
-    v = step(v, std::integral_constant<int, 0x142>{}, std::integral_constant<int, 0xA>{});   // rows 1, 3 += row 0, 2
-    v = step(v, std::integral_constant<int, 0x143>{}, std::integral_constant<int, 0xC>{});   // rows 2, 3 += row 1
+    asm volatile("s_nop 1\n\t"
+                 "v_add_f32_dpp %0, %0, %0 quad_perm:[1,0,3,2] row_mask:0xf bank_mask:0xf\n\t"
+                 "s_nop 1\n\t"
+                 "v_add_f32_dpp %0, %0, %0 quad_perm:[2,3,0,1] row_mask:0xf bank_mask:0xf\n\t"
+                 "s_nop 1\n\t"
+                 "v_add_f32_dpp %0, %0, %0 row_half_mirror row_mask:0xf bank_mask:0xf\n\t"
+                 "s_nop 1\n\t"
+                 "v_add_f32_dpp %0, %0, %0 row_mirror row_mask:0xf bank_mask:0xf\n\t"
+                 "s_nop 1\n\t"
+                 "v_add_f32_dpp %0, %0, %0 row_bcast:15 row_mask:0xa bank_mask:0xf\n\t"
+                 "s_nop 1\n\t"
+                 "v_add_f32_dpp %0, %0, %0 row_bcast:31 row_mask:0xc bank_mask:0xf\n\t"
+                 : "+v"(v));
     return __int_as_float(__builtin_amdgcn_readlane(__float_as_int(v), 63));
 }
 

@@ -39,22 +39,26 @@ template <typename ST> __device__ __forceinline__ void store_scale(ST *p, int i,
 
 // ---------------------------------------------------------------------------------------------
 // 64-lane max reduction of NON-NEGATIVE values; every lane returns the maximum (it comes back through a scalar
-// register, so the compiler knows it is wave-uniform).  Data-parallel-primitive moves inside the vector ALU:
-// a shuffle through the LDS crossbar would cost six dependent LDS round trips.
+// register, so the compiler knows it is wave-uniform).  Data-parallel-primitive forms of v_max_f32 inside the vector
+// ALU: a shuffle through the LDS crossbar would cost six dependent LDS round trips.  Written as asm: from the
+// update_dpp builtin the compiler makes a copy, a v_mov_b32_dpp and two v_max_f32 per step (36 instructions where 6 do;
+// every block-wise kernel runs this once per block and lane).  A DPP operand read needs two wait states behind the
+// vector instruction that wrote the register: the s_nop between the dependent steps.
 __device__ __forceinline__ float wave_max(float v)
 {
-    auto step = [](float x, auto ctrl_c, auto rows_c) {
-        const int t = __builtin_amdgcn_update_dpp(__float_as_int(x), __float_as_int(x), decltype(ctrl_c)::value,
-                                                  decltype(rows_c)::value, 0xF, false);
-        return fmaxf(x, __int_as_float(t));
-    };
-    using all = std::integral_constant<int, 0xF>;
-    v = step(v, std::integral_constant<int, 0xB1>{}, all{});     // quad_perm [1,0,3,2]
-    v = step(v, std::integral_constant<int, 0x4E>{}, all{});     // quad_perm [2,3,0,1]
-    v = step(v, std::integral_constant<int, 0x141>{}, all{});    // row_half_mirror: max of 8
-    v = step(v, std::integral_constant<int, 0x140>{}, all{});    // row_mirror: max of the 16-lane row, in all its lanes
-    v = step(v, std::integral_constant<int, 0x142>{}, std::integral_constant<int, 0xA>{});   // row_bcast15 into rows 1, 3
-    v = step(v, std::integral_constant<int, 0x143>{}, std::integral_constant<int, 0xC>{});   // row_bcast31 into rows 2, 3
+    asm volatile("s_nop 1\n\t"
+                 "v_max_f32_dpp %0, %0, %0 quad_perm:[1,0,3,2] row_mask:0xf bank_mask:0xf\n\t"
+                 "s_nop 1\n\t"
+                 "v_max_f32_dpp %0, %0, %0 quad_perm:[2,3,0,1] row_mask:0xf bank_mask:0xf\n\t"
+                 "s_nop 1\n\t"
+                 "v_max_f32_dpp %0, %0, %0 row_half_mirror row_mask:0xf bank_mask:0xf\n\t"     // max of 8
+                 "s_nop 1\n\t"
+                 "v_max_f32_dpp %0, %0, %0 row_mirror row_mask:0xf bank_mask:0xf\n\t"          // max of the 16-lane row, in all its lanes
+                 "s_nop 1\n\t"
+                 "v_max_f32_dpp %0, %0, %0 row_bcast:15 row_mask:0xa bank_mask:0xf\n\t"        // rows 1, 3: with the row before
+                 "s_nop 1\n\t"
+                 "v_max_f32_dpp %0, %0, %0 row_bcast:31 row_mask:0xc bank_mask:0xf\n\t"        // rows 2, 3: with rows 0-1; lane 63 has all
+                 : "+v"(v));
     return __int_as_float(__builtin_amdgcn_readlane(__float_as_int(v), 63));
 }
 

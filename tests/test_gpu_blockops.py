@@ -376,3 +376,45 @@ def test_block_column_sums(jf, oracle, R, C, f16):
     got = jf.block_colsum(torch.from_numpy(q).cuda(), ds.half() if f16 else ds)
     want = oracle.block_colsum(q, s)
     assert np.array_equal(got.cpu().numpy().view(np.uint32), want.view(np.uint32))
+
+
+@pytest.mark.parametrize("approx,eps", [(0, 5e-5), (1, 0.0), (0, 0.0)])
+@pytest.mark.parametrize("f16", [True, False])
+def test_gelu_fwd_on_one_sided_and_degenerate_blocks(jf, oracle, approx, eps, f16):
+    """Blocks whose absmax is not where random data puts it: only negative codes, on one side of the minimum of x*Phi(x)
+    (at x = -0.75) or straddling it, a single code, the byte -128, far tails where the outputs are a few units of 2^-24,
+    all zeros, a zero scale, scales from 1e-4 to 40."""
+    rng = np.random.default_rng(77 + approx)
+    blocks, scales = [], []
+
+    def add(codes, scale):
+        b = np.asarray(codes, dtype=np.int8)
+        blocks.append(np.resize(b, (QB, QB)) if b.size != QB * QB else b.reshape(QB, QB))
+        scales.append(scale)
+    for scale in (0.0059, 0.01, 0.0387, 0.1, 0.75, 3.0, 1e-4, 40.0):
+        ks = min(int(0.7518 / scale), 127)
+        add(rng.integers(-127, 0, QB * QB), scale)                           # negative only
+        add(rng.integers(-max(ks, 1), 1, QB * QB), scale)                    # up to the split
+        add(rng.integers(-127, -min(ks + 1, 127) + 1, QB * QB), scale)       # beyond the split
+        add([-min(ks, 127) or -1, -min(ks + 1, 127)], scale)                 # the two codes around the minimum
+        add([-127, -124], scale)                                             # two far-tail codes
+        add([-128, -127, 5], scale)                                          # the byte -128
+        add([int(rng.integers(-127, 128))], scale)                           # one code
+        add(rng.integers(-127, 128, QB * QB), scale)
+        add(np.where(rng.random(QB * QB) < 0.9, 0, rng.integers(-127, 0, QB * QB)), scale)
+    add(np.zeros(QB * QB), 1.0)
+    add(rng.integers(-127, 128, QB * QB), 0.0)
+    n = len(blocks)
+    cols = 8
+    rows = -(-n // cols)
+    while len(blocks) < rows * cols:
+        add(rng.integers(-127, 128, QB * QB), 0.5)
+    q = np.block([[blocks[r * cols + c] for c in range(cols)] for r in range(rows)])
+    s = np.array(scales, np.float32).reshape(rows, cols)
+    if f16:
+        s = s.astype(np.float16).astype(np.float32)
+    ds = torch.from_numpy(s).cuda()
+    qy, sy = jf.gelu_fwd(torch.from_numpy(q).cuda(), ds.half() if f16 else ds, approx, eps)
+    wq, ws = oracle.gelu_fwd(q, s, approx, eps, scale_dtype="f16" if f16 else "f32")
+    same(sy, ws, "scales")
+    same(qy, wq, "codes")
