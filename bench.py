@@ -98,7 +98,7 @@ def dominant_kernel_roofline(jf, torch, ops, iters=200):
     # the same launch once more, right behind the timed ones (the clock has settled), with the kernel's profiling build:
     # when each workgroup's phases began and ended and the shader clock its main loop ran at
     tiles = ((M + 127) // 128) * ((N + 127) // 128)
-    ph = jf.igemm_phases(lambda: jf.igemm_block_q(o["qx"], o["qw"], o["sxT"], o["swT"], jf.B_NK), tiles)
+    _, _, ph = jf.igemm_phases(o["qx"], o["qw"], o["sxT"], o["swT"], jf.B_NK)
     us, mhz = ph["us"], float(ph["k_loop_MHz"].mean())
     span_us = float(us[:, 5].max())
     products = (M // 32) * (N // 32) * (K // 32)              # 32x32x32 block products = MFMA instructions

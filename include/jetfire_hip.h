@@ -278,40 +278,6 @@ int jf_block_colsum(const int8_t *q, const void *s, int R, int C, int scale_dtyp
 int jf_rowstats_finish(const float *rowsum, const float *rowsq, int R, int parts, int C, float *mean, float *rstd,
                        jf_stream_t stream);
 
-/* Phase recording (no counterpart in the reference; a profiling aid for bench.py).  While a buffer is set, every
- * jf_igemm_block_q call with fp32 scales launches a profiling build of its kernel in which workgroup w (w <
- * capacity_workgroups; a workgroup computes one 128x128 output tile) stores 8 64-bit words at phases[8*w]:
- *   [0] start  [1] main loop begins  [2] main loop ends  [3] epilogue begins  [4] blocks requantised  [5] end
- *       (ticks of the constant-rate wall clock, jf_wall_clock_khz)
- *   [6] the hardware id register of its first wave (which CU it ran on)
- *   [7] shader-clock cycles its main loop took ([7] / ([2]-[1]) = the clock the shader ran at under this load).
- * `phases` is device memory of 8 * capacity_workgroups words; NULL ends the recording.  Process-wide, meant for one
- * thread measuring one launch at a time; results are the same bits as the normal build's. */
-int jf_igemm_phase_record(unsigned long long *phases, int capacity_workgroups);
-
-/* Calibration (no counterpart in the reference; used by bench.py for the roofline discussion): launches `workgroups` x
- * `threads` (128, 256, 384 or 512) threads; per iteration every wave runs 4 work items from registers, an item being
- *   JF_CAL_UNIFORM: [one 32x32x32 INT8 MFMA if with_mfma] + [valu_per_mfma independent v_fmac_f32]
- *                   supported (with_mfma, valu_per_mfma): (1,0) (0,32) (1,32) (0,16) (1,16);
- *   JF_CAL_SPLIT:   the MFMA in the first half of a workgroup's waves, 32 v_fmac_f32 in the second half (1, 32): with
- *                   512 threads the two kinds of wave share each SIMD;
- *   JF_CAL_STREAM:  the GEMM's K-block instruction stream (1, 32): MFMA with the constant accumulator input, then 16
- *                   subtractions and 16 v_fmac_f32 on the previous product;
- *   JF_CAL_STREAM_DATA: the same stream (1, 32) on operands that change with every MFMA and use all 8 bits, and a
- *                   scale with a full mantissa: the clock rate the stream sustains when the datapaths toggle as on
- *                   real tensors (launch it long enough, tens of milliseconds, for the clock to settle).
- * `scratch`: a device buffer of at least 4 bytes (never written in practice).  `clocks` (may be NULL): 2 x workgroups
- * 64-bit words; workgroup w's first wave stores the shader-clock cycles and the wall-clock ticks (constant rate,
- * hipDeviceAttributeWallClockRate) it ran for, which gives the clock the shader ran at under this load. */
-#define JF_CAL_UNIFORM 0
-#define JF_CAL_SPLIT   1
-#define JF_CAL_STREAM  2
-#define JF_CAL_STREAM_DATA 3
-int jf_calibrate(int mode, int with_mfma, int valu_per_mfma, int iters, int workgroups, int threads, float *scratch,
-                 unsigned long long *clocks, jf_stream_t stream);
-/* Ticks per millisecond of the wall clock above on the current device (0 or negative: not available). */
-int jf_wall_clock_khz(void);
-
 #ifdef __cplusplus
 }
 #endif

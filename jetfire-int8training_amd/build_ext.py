@@ -1,6 +1,9 @@
 """Builds the native parts in-tree (no JIT cache, so the artefacts travel with the source tree):
 
   libjetfire_hip.so        hipcc, gfx950 only: the HIP kernels behind the C ABI of include/jetfire_hip.h
+  libjetfire_prof.so       hipcc, gfx950 only: measurement aids (include/jetfire_prof.h): the phase-recording build of
+                           the GEMM kernel (the same source, -DJF_PROF_LIB) and register-only calibration loops;
+                           used by the benchmark, not by the operators
   BlockQuantizeCUDA*.so    host C++ (g++): the PyTorch extension with the reference's module name and
                            function signatures (JetfireGEMMKernel/setup.py:13, bindings.cpp:6-35), plus the
                            submodule BlockQuantizeCUDA.jetfire with every other operator of the path; it is
@@ -19,7 +22,9 @@ CSRC = os.path.join(HERE, "csrc")
 HIP_LIB = os.path.join(HERE, "libjetfire_hip.so")
 ROCM = os.environ.get("ROCM_PATH", "/opt/rocm")
 
-HIP_SOURCES = ["jf_gemm.hip", "jf_blockops.hip", "jf_calib.hip"]
+HIP_SOURCES = ["jf_gemm.hip", "jf_blockops.hip"]
+PROF_LIB = os.path.join(HERE, "libjetfire_prof.so")
+PROF_SOURCES = [("jf_gemm.hip", ["-DJF_PROF_LIB"], "jf_gemm_prof.o"), ("jf_calib.hip", [], "jf_calib.o")]
 HIP_FLAGS = [
     "--offload-arch=gfx950", "-O3", "-std=c++17", "-fPIC", "-shared",
     "-ffp-contract=off",                                         # roundings are exactly the ones written
@@ -46,16 +51,22 @@ def build_hip():
     hipcc = os.path.join(ROCM, "bin", "hipcc")
     objdir = os.path.join(HERE, "build")
     os.makedirs(objdir, exist_ok=True)
-    jobs = []
+    jobs, prof_jobs = [], []
     for src in HIP_SOURCES:
         obj = os.path.join(objdir, os.path.splitext(src)[0] + ".o")
         cmd = [hipcc] + flags + ["-c", os.path.join(CSRC, src), "-o", obj]
         print("+", " ".join(cmd), flush=True)
         jobs.append((cmd, obj, subprocess.Popen(cmd)))
-    for cmd, obj, proc in jobs:
+    for src, extra, name in PROF_SOURCES:
+        obj = os.path.join(objdir, name)
+        cmd = [hipcc] + flags + extra + ["-c", os.path.join(CSRC, src), "-o", obj]
+        print("+", " ".join(cmd), flush=True)
+        prof_jobs.append((cmd, obj, subprocess.Popen(cmd)))
+    for cmd, obj, proc in jobs + prof_jobs:
         if proc.wait() != 0:
             raise subprocess.CalledProcessError(proc.returncode, cmd)
     _run([hipcc, "--offload-arch=gfx950", "-shared", "-fPIC", "-o", HIP_LIB] + [obj for _, obj, _ in jobs])
+    _run([hipcc, "--offload-arch=gfx950", "-shared", "-fPIC", "-o", PROF_LIB] + [obj for _, obj, _ in prof_jobs])
     return HIP_LIB
 
 

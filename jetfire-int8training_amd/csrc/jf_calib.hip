@@ -6,6 +6,7 @@
 // wall clock it ran for, so that a result can be stated in cycles as well as in nanoseconds: "the two pipes add up"
 // can then be told apart from "the clock dropped under the combined load".
 #include "jf_device.hpp"
+#include "../../include/jetfire_prof.h"
 
 namespace jf {
 

@@ -925,15 +925,18 @@ __global__ __launch_bounds__(256) void splitk_reduce_kernel(const float *part, s
     }
 }
 
+// compute units of the current device (asked once per device; 256 if the query fails)
 static int cu_count()
 {
-    static const int n = [] {
-        int dev = 0, cus = 0;
-        if (hipGetDevice(&dev) != hipSuccess || hipDeviceGetAttribute(&cus, hipDeviceAttributeMultiprocessorCount, dev) != hipSuccess || cus <= 0)
-            cus = 256;
-        return cus;
-    }();
-    return n;
+    static std::atomic<int> known[MAX_DEVICES] = {};
+    int dev = 0;
+    if (hipGetDevice(&dev) != hipSuccess || dev < 0 || dev >= MAX_DEVICES) return 256;
+    int cus = known[dev].load(std::memory_order_relaxed);
+    if (cus == 0) {
+        if (hipDeviceGetAttribute(&cus, hipDeviceAttributeMultiprocessorCount, dev) != hipSuccess || cus <= 0) cus = 256;
+        known[dev].store(cus, std::memory_order_relaxed);
+    }
+    return cus;
 }
 
 // K split of the fp-output GEMM.  request 1: none; request > 1: that many parts (fewer if K is short); request 0: as
@@ -972,17 +975,15 @@ template <int EPI, typename ST> static int launch_gemm(const GemmArgs &a, hipStr
             }
             return JF_ERR_UNSUPPORTED;
         }
+#ifdef JF_PROF_LIB
         if constexpr (EPI == EPI_Q && std::is_same<ST, float>::value) {
-            if (a.phases)                                     // a recording buffer is set: the profiling build
+            if (a.phases)                                     // the profiling library: the PROF build of the same kernel
                 return b_kn ? launch_gemm_cfg<EPI, ST, 2, 4, 2, 2, 1, 0, 1>(a, st) : launch_gemm_cfg<EPI, ST, 2, 4, 2, 2, 0, 0, 1>(a, st);
         }
+#endif
         return b_kn ? launch_gemm_cfg<EPI, ST, 2, 4, 2, 2, 1>(a, st) : launch_gemm_cfg<EPI, ST, 2, 4, 2, 2, 0>(a, st);
     }
 }
-
-// recording buffer of the profiling build (process-wide; set and cleared by jf_igemm_phase_record)
-static std::atomic<unsigned long long *> phase_buffer{nullptr};
-static std::atomic<int> phase_buffer_capacity{0};
 
 static int check_gemm_common(const void *A, const void *B, const void *C, int M, int N, int K, int b_layout)
 {
@@ -997,6 +998,21 @@ static int check_gemm_common(const void *A, const void *B, const void *C, int M,
 
 using namespace jf;
 
+// element strides (K block, tile block) of a scale operand with `blocks` tile blocks
+static bool scale_strides(int layout, int K, int blocks, int &ks, int &is)
+{
+    if (layout == JF_SCALES_KMAJOR) { ks = blocks; is = 1; return true; }
+    if (layout == JF_SCALES_ROWMAJOR) { ks = 1; is = K / QB; return true; }
+    return false;
+}
+
+// scale arrays need the natural alignment of their element type (binary16 scales are fetched one element at a time)
+static bool scale_ptr_ok(const void *p, int scale_dtype)
+{
+    return (reinterpret_cast<uintptr_t>(p) & (scale_dtype == JF_SCALE_F32 ? 3u : 1u)) == 0;
+}
+
+#ifndef JF_PROF_LIB
 extern "C" {
 
 const char *jf_error_string(int code)
@@ -1049,20 +1065,6 @@ int jf_igemm_block_acc(const int8_t *A, const int8_t *B, int32_t *acc, int M, in
         if ((rc = launch_gemm<EPI_S32, float>(a, (hipStream_t)stream, kn))) return rc;
     }
     return JF_OK;
-}
-
-// element strides (K block, tile block) of a scale operand with `blocks` tile blocks
-static bool scale_strides(int layout, int K, int blocks, int &ks, int &is)
-{
-    if (layout == JF_SCALES_KMAJOR) { ks = blocks; is = 1; return true; }
-    if (layout == JF_SCALES_ROWMAJOR) { ks = 1; is = K / QB; return true; }
-    return false;
-}
-
-// scale arrays need the natural alignment of their element type (binary16 scales are fetched one element at a time)
-static bool scale_ptr_ok(const void *p, int scale_dtype)
-{
-    return (reinterpret_cast<uintptr_t>(p) & (scale_dtype == JF_SCALE_F32 ? 3u : 1u)) == 0;
 }
 
 int jf_igemm_splitk_plan(int M, int N, int K, int splitk, int *splits, int *kb_per_split)
@@ -1195,10 +1197,6 @@ int jf_igemm_block_q(const int8_t *A, const int8_t *B, const void *sa, const voi
     if (!scale_strides(sa_layout, K, M / QB, a.sa_ks, a.sa_is) || !scale_strides(sb_layout, K, N / QB, a.sb_ks, a.sb_is))
         return JF_ERR_ENUM;
     hipStream_t st = (hipStream_t)stream;
-    if (scale_dtype == JF_SCALE_F32) {
-        a.phases = phase_buffer.load(std::memory_order_acquire);
-        a.phase_capacity = phase_buffer_capacity.load(std::memory_order_acquire);
-    }
     return scale_dtype == JF_SCALE_F16 ? launch_gemm<EPI_Q, half_t>(a, st, kn) : launch_gemm<EPI_Q, float>(a, st, kn);
 }
 
@@ -1222,16 +1220,6 @@ int jf_igemm_block_q_dequant(const int8_t *A, const int8_t *B, const void *sa, c
         return JF_ERR_ENUM;
     hipStream_t st = (hipStream_t)stream;
     return scale_dtype == JF_SCALE_F16 ? launch_gemm<EPI_QD, half_t>(a, st, kn) : launch_gemm<EPI_QD, float>(a, st, kn);
-}
-
-int jf_igemm_phase_record(unsigned long long *phases, int capacity_workgroups)
-{
-    if (phases && capacity_workgroups <= 0) return JF_ERR_SHAPE;
-    if (!phases) capacity_workgroups = 0;
-    phase_buffer_capacity.store(0, std::memory_order_release);
-    phase_buffer.store(phases, std::memory_order_release);
-    phase_buffer_capacity.store(capacity_workgroups, std::memory_order_release);
-    return JF_OK;
 }
 
 int jf_igemm_block_q_gelu(const int8_t *A, const int8_t *B, const void *sa, const void *sb, const float *bias,
@@ -1289,3 +1277,31 @@ int jf_transpose_s8(const int8_t *in, int R, int C, int8_t *out, jf_stream_t str
 }
 
 }  // extern "C"
+#else   // JF_PROF_LIB: libjetfire_prof.so
+
+#include "../../include/jetfire_prof.h"
+
+// jf_igemm_block_q with fp32 scales through the PROF instantiation of the kernel: same arithmetic, same bits, plus the
+// per-workgroup phase record (include/jetfire_prof.h).
+extern "C" int jf_prof_igemm_block_q(const int8_t *A, const int8_t *B, const float *sa, const float *sb, const float *bias,
+                                     const float *biasmax, int8_t *C, float *sc, int M, int N, int K, int b_layout,
+                                     int sa_layout, int sb_layout, int rounding, uint64_t seed, uint64_t offset,
+                                     unsigned long long *phases, int capacity_workgroups, jf_stream_t stream)
+{
+    int rc = check_gemm_common(A, B, C, M, N, K, b_layout);
+    if (rc) return rc;
+    if (!sa || !sb || !sc || !phases) return JF_ERR_NULL;
+    if (capacity_workgroups <= 0) return JF_ERR_SHAPE;
+    if (rounding != JF_ROUND_NEAREST && rounding != JF_ROUND_STOCHASTIC) return JF_ERR_ENUM;
+    const bool kn = b_layout == JF_B_KN;
+    GemmArgs a = {};
+    a.A = A; a.B = B; a.sa = sa; a.sb = sb; a.C = C; a.sc = sc; a.bias = bias; a.biasmax = biasmax;
+    a.M = M; a.N = N; a.K = K; a.lda = K; a.ldb = kn ? N : K; a.rounding = rounding; a.seed = seed; a.offset = offset;
+    if (!scale_strides(sa_layout, K, M / QB, a.sa_ks, a.sa_is) || !scale_strides(sb_layout, K, N / QB, a.sb_ks, a.sb_is))
+        return JF_ERR_ENUM;
+    a.phases = phases;
+    a.phase_capacity = capacity_workgroups;
+    return launch_gemm<EPI_Q, float>(a, (hipStream_t)stream, kn);
+}
+
+#endif  // JF_PROF_LIB

@@ -28,7 +28,7 @@ EXPORTS = [
     "jf_error_string", "jf_igemm_workspace_bytes", "jf_igemm_s32", "jf_igemm_block_acc", "jf_igemm_block_fp",
     "jf_igemm_splitk_plan", "jf_igemm_block_fp_workspace_bytes", "jf_igemm_block_q_gelu", "jf_igemm_block_fp_noalloc", "jf_igemm_block_q_gelu_bwd",
     "jf_igemm_block_q", "jf_quantize", "jf_dequantize", "jf_transpose_s8", "jf_rowstats", "jf_layernorm_fwd",
-    "jf_layernorm_bwd_workspace_bytes", "jf_layernorm_bwd", "jf_layernorm_bwd_add", "jf_gelu_fwd", "jf_gelu_bwd", "jf_add", "jf_calibrate", "jf_wall_clock_khz", "jf_igemm_phase_record", "jf_rowstats_finish",
+    "jf_layernorm_bwd_workspace_bytes", "jf_layernorm_bwd", "jf_layernorm_bwd_add", "jf_gelu_fwd", "jf_gelu_bwd", "jf_add", "jf_rowstats_finish",
     "jf_igemm_block_q_dequant", "jf_quantize_slabs", "jf_philox_rounds", "jf_block_colsum", "jf_block_colsum_workspace_bytes",
 ]
 
@@ -57,7 +57,6 @@ def lib():
         L.jf_igemm_splitk_plan.argtypes = [_i, _i, _i, _i, C.POINTER(C.c_int), C.POINTER(C.c_int)]
         L.jf_igemm_block_fp_workspace_bytes.argtypes = [_i, _i, _i, _i, _i]
         L.jf_igemm_block_fp_workspace_bytes.restype = _sz
-        L.jf_igemm_phase_record.argtypes = [_p, _i]
         L.jf_rowstats_finish.argtypes = [_p, _p, _i, _i, _i, _p, _p, _p]
         L.jf_igemm_block_q.argtypes = [_p, _p, _p, _p, _p, _p, _p, _p, _i, _i, _i, _i, _i, _i, _i, _i, _u64, _u64, _p, _sz, _p]
         L.jf_quantize.argtypes = [_p, _i, _i, _i, _p, _p, _p, _i, _i, _u64, _u64, _f, _p]
@@ -74,16 +73,33 @@ def lib():
         L.jf_layernorm_bwd_add.argtypes = [_p, _p, _p, _p, _p, _p, _p, _i, _i, _i, _i, _u64, _u64, _p, _i, _i, _u64, _u64,
                                            _p, _i, _p, _p, _p, _p, _p, _sz, _p]
         L.jf_add.argtypes = [_p, _i, _p, _p, _i, _i, _i, _i, _u64, _u64, _p, _i, _p, _p, _p, _p, _p]
-        L.jf_wall_clock_khz.argtypes = []
         L.jf_block_colsum_workspace_bytes.argtypes = [_i, _i]
         L.jf_block_colsum_workspace_bytes.restype = _sz
         L.jf_block_colsum.argtypes = [_p, _p, _i, _i, _i, _p, _p, _sz, _p]
-        L.jf_calibrate.argtypes = [_i, _i, _i, _i, _i, _i, _p, _p, _p]
         missing = [name for name in EXPORTS if not hasattr(L, name)]
         if missing:
             raise RuntimeError(f"{LIB_PATH} does not export {missing}")
         _lib = L
     return _lib
+
+
+PROF_LIB_PATH = os.path.join(_HERE, "libjetfire_prof.so")
+PROF_EXPORTS = ["jf_prof_igemm_block_q", "jf_calibrate", "jf_wall_clock_khz"]
+_prof = None
+
+
+def prof_lib():
+    """The measurement library (include/jetfire_prof.h); only the benchmark and its tests load it."""
+    global _prof
+    if _prof is None:
+        if not os.path.exists(PROF_LIB_PATH):
+            raise RuntimeError(f"{PROF_LIB_PATH} is missing: build it with `python {os.path.join(_HERE, 'build_ext.py')} hip`")
+        L = C.CDLL(PROF_LIB_PATH)
+        L.jf_prof_igemm_block_q.argtypes = [_p, _p, _p, _p, _p, _p, _p, _p, _i, _i, _i, _i, _i, _i, _i, _u64, _u64, _p, _i, _p]
+        L.jf_calibrate.argtypes = [_i, _i, _i, _i, _i, _i, _p, _p, _p]
+        L.jf_wall_clock_khz.argtypes = []
+        _prof = L
+    return _prof
 
 
 def check(rc):
@@ -574,9 +590,9 @@ CAL_UNIFORM, CAL_SPLIT, CAL_STREAM, CAL_STREAM_DATA = 0, 1, 2, 3
 
 
 def calibrate(with_mfma, valu_per_mfma, iters=2000, workgroups_per_cu=4, threads=256, mode=CAL_UNIFORM, launches=3):
-    """Runs the register-only calibration kernel (see jf_calibrate in the header) and returns a dict: seconds per launch
-    (events), the number of work items it ran (workgroups * waves * iters * 4; for CAL_SPLIT: items of the MFMA waves),
-    the resident waves per SIMD, and the shader clock in MHz the kernel ran at (cycles / wall-clock time, from the
+    """Runs the register-only calibration kernel (jf_calibrate of the measurement library) and returns a dict: seconds per
+    launch (events), the number of work items it ran (workgroups * waves * iters * 4; for CAL_SPLIT: items of the MFMA
+    waves), the resident waves per SIMD, and the shader clock in MHz the kernel ran at (cycles / wall-clock time, from the
     per-workgroup readings of the last launch)."""
     props = torch.cuda.get_device_properties(0)
     cus = props.multi_processor_count
@@ -584,8 +600,8 @@ def calibrate(with_mfma, valu_per_mfma, iters=2000, workgroups_per_cu=4, threads
     waves = threads // 64
     scratch = torch.zeros(16, dtype=torch.float32, device="cuda")
     clocks = torch.zeros(2 * wgs, dtype=torch.int64, device="cuda")
-    run = lambda: check(lib().jf_calibrate(mode, with_mfma, valu_per_mfma, iters, wgs, threads, _ptr(scratch), _ptr(clocks),
-                                           _stream()))
+    run = lambda: check(prof_lib().jf_calibrate(mode, with_mfma, valu_per_mfma, iters, wgs, threads, _ptr(scratch), _ptr(clocks),
+                                                _stream()))
     run()
     e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
     e0.record()
@@ -600,34 +616,36 @@ def calibrate(with_mfma, valu_per_mfma, iters=2000, workgroups_per_cu=4, threads
             "shader_MHz": float(c[0] / c[1]) * wall_hz / 1e6, "simds": cus * 4}
 
 
-def igemm_phases(fn, workgroups):
-    """Runs fn() (one jf_igemm_block_q call with fp32 scales) under the library's phase recording and returns, per
-    workgroup (one 128x128 output tile each), a dict of numpy arrays: 'us' [workgroups, 6] (start, main loop begins, main
-    loop ends, epilogue begins, blocks requantised, end; microseconds since the first workgroup started), 'cu' (an id
-    of the CU it ran on), 'k_loop_MHz' (shader clock during its main loop) and 'k_loop_cycles'."""
+def igemm_phases(A, B, sa, sb, b_layout=B_KN, rounding=ROUND_NEAREST, seed=0, offset=0):
+    """igemm_block_q (fp32 scales) through the phase-recording build of its kernel (measurement library).  Returns
+    (q, sc, phases): the same codes and scales, and per workgroup (one 128x128 output tile each) a dict of numpy arrays:
+    'us' [workgroups, 6] (start, main loop begins, main loop ends, epilogue begins, blocks requantised, end; microseconds
+    since the first workgroup started), 'cu' (an id of the CU it ran on), 'k_loop_MHz' (shader clock during its main
+    loop) and 'k_loop_cycles'."""
     import numpy as np
-    buf = torch.zeros(workgroups * 8, dtype=torch.int64, device="cuda")
-    check(lib().jf_igemm_phase_record(_ptr(buf), workgroups))
-    try:
-        fn()
-        torch.cuda.synchronize()
-    finally:
-        check(lib().jf_igemm_phase_record(None, 0))
+    M, N, K, _, _ = _gemm_operands(A, B, b_layout)
+    code, la, lb = _gemm_scales(sa, sb, M, N, K)
+    if code != SCALE_F32:
+        raise RuntimeError("igemm_phases: fp32 scales only")
+    workgroups = ((M + 127) // 128) * ((N + 127) // 128)
+    buf = torch.zeros(workgroups * 8, dtype=torch.int64, device=A.device)
+    out = torch.empty((M, N), dtype=torch.int8, device=A.device)
+    sc = torch.empty((M // QB, N // QB), dtype=torch.float32, device=A.device)
+    check(prof_lib().jf_prof_igemm_block_q(_ptr(A), _ptr(B), _ptr(sa), _ptr(sb), None, None, _ptr(out), _ptr(sc), M, N, K,
+                                           b_layout, la, lb, rounding, seed, offset, _ptr(buf), workgroups, _stream()))
+    torch.cuda.synchronize()
     w = buf.view(workgroups, 8).cpu().numpy()
     hz = _wall_clock_hz()
     t = w[:, :6].astype(np.float64)
-    if (t[:, 5] <= 0).any():
-        raise RuntimeError("igemm_phases: the call launched fewer workgroups than asked for, or no profiling build")
     us = (t - t[:, 0].min()) / hz * 1e6
     hw = w[:, 6]
-    return {"us": us, "cu": hw & 0xFF00 | ((hw >> 16) & 0xFF),
-            "k_loop_cycles": w[:, 7].astype(np.float64),
-            "k_loop_MHz": w[:, 7] / np.maximum(t[:, 2] - t[:, 1], 1.0) * hz / 1e6}
+    return out, sc, {"us": us, "cu": hw & 0xFF00 | ((hw >> 16) & 0xFF), "k_loop_cycles": w[:, 7].astype(np.float64),
+                     "k_loop_MHz": w[:, 7] / np.maximum(t[:, 2] - t[:, 1], 1.0) * hz / 1e6}
 
 
 def _wall_clock_hz():
     """Rate of the constant clock the kernel's wall-clock readings count in."""
-    khz = lib().jf_wall_clock_khz()
+    khz = prof_lib().jf_wall_clock_khz()
     if khz <= 0:
         raise RuntimeError("jf_wall_clock_khz: the device does not report a wall clock rate")
     return khz * 1e3

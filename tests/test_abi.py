@@ -6,8 +6,8 @@ import re
 ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
 
 
-def _declared():
-    text = open(os.path.join(ROOT, "include", "jetfire_hip.h")).read()
+def _declared(header="jetfire_hip.h"):
+    text = open(os.path.join(ROOT, "include", header)).read()
     text = re.sub(r"/\*.*?\*/", "", text, flags=re.S)
     return sorted(set(re.findall(r"\b(jf_[a-z0-9_]+)\s*\(", text)))
 
@@ -22,6 +22,18 @@ def test_header_symbols_are_exported():
 
 def test_binding_lists_every_symbol(jf):
     assert sorted(jf.EXPORTS) == _declared()
+
+
+def test_measurement_library_is_separate(jf):
+    """The measurement aids live in their own library and header: the product library exports only what jetfire_hip.h
+    declares (the reference's interfaces and the allocation-free entry point)."""
+    names = _declared("jetfire_prof.h")
+    assert sorted(jf.PROF_EXPORTS) == names and len(names) == 3
+    prof = ctypes.CDLL(os.path.join(ROOT, "jetfire-int8training_amd", "libjetfire_prof.so"))
+    main = ctypes.CDLL(os.path.join(ROOT, "jetfire-int8training_amd", "libjetfire_hip.so"))
+    for n in names:
+        assert hasattr(prof, n), n
+        assert not hasattr(main, n), f"{n} belongs to the measurement library"
 
 
 def test_argument_errors_without_gpu(jf):

@@ -465,23 +465,19 @@ def test_gemm_with_fused_dequantisation(jf, oracle, M, N, K, layout, f16):
 
 @pytest.mark.gpu
 def test_phase_recording_build_gives_the_same_bits_and_ordered_phases(jf):
-    """The profiling build of the requantising GEMM (jf_igemm_phase_record) stores the same codes and scales as the
-    normal build, and every workgroup's phase stamps are in order with a plausible shader clock."""
+    """The profiling build of the requantising GEMM (jf_prof_igemm_block_q of the measurement library) stores the same
+    codes and scales as the product library's kernel, and every workgroup's phase stamps are in order with a plausible
+    shader clock."""
     g = torch.Generator().manual_seed(5)
     M, N, K = 384, 416, 256                                     # 3 x 4 tiles, the last tile column a quarter full
     A = torch.randint(-127, 128, (M, K), generator=g, dtype=torch.int8).cuda()
     B = torch.randint(-127, 128, (N, K), generator=g, dtype=torch.int8).cuda()
     sa = (torch.rand(K // 32, M // 32, generator=g) * 0.01 + 1e-3).cuda()
     sb = (torch.rand(K // 32, N // 32, generator=g) * 0.01 + 1e-3).cuda()
-    q0, s0 = jf.igemm_block_q(A, B, sa, sb, jf.B_NK)
-    out = {}
-
-    def call():
-        out["q"], out["s"] = jf.igemm_block_q(A, B, sa, sb, jf.B_NK)
-    ph = jf.igemm_phases(call, 12)
-    assert torch.equal(out["q"], q0) and torch.equal(out["s"], s0)
-    us = ph["us"]
-    assert us.shape == (12, 6) and (us[:, 1:] >= us[:, :-1]).all() and us[:, 5].max() < 1e4
-    assert ((ph["k_loop_MHz"] > 300) & (ph["k_loop_MHz"] < 3500)).all()
-    q1, s1 = jf.igemm_block_q(A, B, sa, sb, jf.B_NK)            # recording is off again
-    assert torch.equal(q1, q0) and torch.equal(s1, s0)
+    for rounding, kw in ((jf.ROUND_NEAREST, {}), (jf.ROUND_STOCHASTIC, dict(seed=3, offset=8))):
+        q0, s0 = jf.igemm_block_q(A, B, sa, sb, jf.B_NK, rounding=rounding, **kw)
+        q, s, ph = jf.igemm_phases(A, B, sa, sb, jf.B_NK, rounding=rounding, **kw)
+        assert torch.equal(q, q0) and torch.equal(s, s0)
+        us = ph["us"]
+        assert us.shape == (12, 6) and (us[:, 1:] >= us[:, :-1]).all() and us[:, 5].max() < 1e4
+        assert ((ph["k_loop_MHz"] > 300) & (ph["k_loop_MHz"] < 3500)).all()
