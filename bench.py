@@ -370,6 +370,10 @@ def nonlinear_extras(jf, torch):
     put("layernorm_bwd_add_sr_bf16_8192x1600", t(lambda: f(qx, sx, qg, sg, xb)), 7 * n, (f, (qx, sx, qg, sg, xb)))
     f = lambda g_, sg_: jf.block_colsum(g_, sg_)
     put("bias_gradient_colsum_8192x1600", t(lambda: f(qg, sg)), n, (f, (qg, sg)))
+    # what a plain device copy of the same bytes reaches under the same two measurements (1 + 1 bytes per element, the
+    # traffic of LayerNorm / GELU forward): the ceiling of this method at this size, beside the 8 TB/s the fractions use
+    f = lambda q_: torch.empty_like(q_).copy_(q_)
+    put("reference_copy_s8_8192x1600", t(lambda: f(qx)), 2 * n, (f, (qx,)))
     R, C = TOKENS, 6400
     x = torch.randn(R, C, generator=g).cuda()
     dy = (torch.randn(R, C, generator=g) * 1e-3).cuda()
@@ -377,6 +381,8 @@ def nonlinear_extras(jf, torch):
     qg, sg = jf.quantize(dy, jf.ROUND_STOCHASTIC, S, seed=0, offset=0)
     n = R * C
     del x, dy
+    f = lambda q_: torch.empty_like(q_).copy_(q_)
+    put("reference_copy_s8_8192x6400", t(lambda: f(qx)), 2 * n, (f, (qx,)))
     f = lambda q_, s_: jf.gelu_fwd(q_, s_, jf.GELU_TANH, 0.0)
     put("gelu_fwd_tanh_8192x6400", t(lambda: f(qx, sx)), 2 * n, (f, (qx, sx)))
     f = lambda q_, s_: jf.gelu_fwd(q_, s_, jf.GELU_ERF, 5e-5)

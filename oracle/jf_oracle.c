@@ -367,30 +367,35 @@ float jfo_expf(float x)
     return p;
 }
 
-/* erfc(z) for z >= 0: the Chebyshev-fitted form of Numerical Recipes (erfcc),
- * fractional error < 1.2e-7 in exact arithmetic. */
-float jfo_erfc_pos(float z)
+/* Phi(-x) = erfc(x/sqrt2)/2 for x >= 0: 0.5 / (1 + b1 x + ... + b6 x^6)^16, Abramowitz & Stegun 7.1.28 (|error| <= 3e-7
+ * on erf) with the coefficients rescaled to x/sqrt2; with float rounding (the sixteenth power amplifies the rounding of
+ * its base sixteen times) the absolute error stays below 1e-6.  The reciprocal is three Newton steps from an
+ * integer-subtraction seed, so that host and device evaluate the same bits without an IEEE division or an exponential. */
+float jfo_phi_neg(float x)
 {
-    float t = 1.0f / fmaf(0.5f, z, 1.0f);
-    float p = 0.17087277f;
-    p = fmaf(p, t, -0.82215223f);
-    p = fmaf(p, t, 1.48851587f);
-    p = fmaf(p, t, -1.13520398f);
-    p = fmaf(p, t, 0.27886807f);
-    p = fmaf(p, t, -0.18628806f);
-    p = fmaf(p, t, 0.09678418f);
-    p = fmaf(p, t, 0.37409196f);
-    p = fmaf(p, t, 1.00002368f);
-    p = fmaf(p, t, -1.26551223f);
-    float e = fmaf(-z, z, p);
-    return t * jfo_expf(e);
+    float p = 5.38297490e-06f;
+    p = fmaf(p, x, 4.88906371e-05f);
+    p = fmaf(p, x, 3.80035744e-05f);
+    p = fmaf(p, x, 3.27762635e-03f);
+    p = fmaf(p, x, 2.11410057e-02f);
+    p = fmaf(p, x, 4.98673469e-02f);
+    float u = fmaf(p, x, 1.0f);
+    u = u * u; u = u * u; u = u * u; u = u * u;
+    u = fminf(u, 1.2676506e30f);                      /* 2^100 */
+    int32_t bits; memcpy(&bits, &u, 4);
+    bits = 0x7EF311C7 - bits;
+    float r; memcpy(&r, &bits, 4);
+    for (int i = 0; i < 3; ++i) {
+        float e = fmaf(-u, r, 1.0f);
+        r = fmaf(r, e, r);
+    }
+    return 0.5f * r;
 }
 
 /* Phi(x) = (1+erf(x/sqrt2))/2  (gelu_fwd.py:81) */
 float jfo_norm_cdf(float x)
 {
-    float z = fabsf(x) * 0.707106781f;
-    float h = 0.5f * jfo_erfc_pos(z);
+    float h = jfo_phi_neg(fabsf(x));
     return x > 0.0f ? 1.0f - h : h;
 }
 

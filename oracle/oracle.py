@@ -62,7 +62,7 @@ def _declare(L):
     L.jfo_igemm_block_acc.argtypes = [_p, _p, _p, _i, _i, _i, _i]
     L.jfo_igemm_block_f32.argtypes = [_p, _p, _p, _p, _p, _i, _i, _i, _i, _i]
     L.jfo_requant.argtypes = [_p, _i, _i, _p, _f, _i, _u64, _u64, _p, _p]
-    for name in ("jfo_expf", "jfo_erfc_pos", "jfo_norm_cdf", "jfo_tanhf"):
+    for name in ("jfo_expf", "jfo_phi_neg", "jfo_norm_cdf", "jfo_tanhf"):
         getattr(L, name).argtypes = [_f]
         getattr(L, name).restype = _f
     for name in ("jfo_gelu", "jfo_dgelu"):
@@ -267,8 +267,8 @@ def expf(x):
     return _vec("jfo_expf", x)
 
 
-def erfc_pos(x):
-    return _vec("jfo_erfc_pos", x)
+def phi_neg(x):
+    return _vec("jfo_phi_neg", x)
 
 
 def norm_cdf(x):
