@@ -28,8 +28,8 @@ INT8_PEAK_TOPS = 5000.0      # MI355X dense INT8 MFMA peak, tera-ops/s
 # HBM-side bytes per launch of the fc forward GEMM, from the rocprofv3 --pmc runs summarised in
 # profiles/igemm_fc_forward_pmc.md (FETCH_SIZE and WRITE_SIZE, each scaled by a copy of known size): a property of the
 # kernel, carried over from that profile, not re-measured by this run (counters need the profiler attached)
-PROFILED_TRAFFIC_BYTES = 150.2e6
-PROFILED_TRAFFIC_SOURCE = "profiles/igemm_fc_forward_pmc.md (97.3 MB fetched + 52.8 MB written; algorithmic 75.9 MB)"
+PROFILED_TRAFFIC_BYTES = 160.3e6
+PROFILED_TRAFFIC_SOURCE = "profiles/igemm_fc_forward_pmc.md (101.0 MB fetched + 59.3 MB written; algorithmic 75.9 MB)"
 TOKENS = 8192
 LAYERS = [("qkv", 1600, 4800), ("proj", 1600, 1600), ("fc", 1600, 6400), ("fc2", 6400, 1600)]
 

@@ -71,7 +71,7 @@ struct GemmArgs {
     uint64_t seed2, offset2;   // noise of the GELU backward's own requantisation   (EPI_QB)
     int rounding2;        // JF_ROUND_NEAREST / JF_ROUND_STOCHASTIC   (EPI_QB)
     int pace;             // PACE_*: wave priorities that order the resident workgroups of a CU (set by the launcher, see there)
-    unsigned long long *phases;   // PROF kernels: 8 words per workgroup (jf_igemm_phase_record), first phase_capacity workgroups
+    unsigned long long *phases;   // PROF kernels: 8 words per workgroup (jf_prof_igemm_block_q), first phase_capacity workgroups
     int phase_capacity;
 };
 
@@ -109,8 +109,8 @@ constexpr int WBM = 2, WBN = 1;
 static int cu_count();
 
 // PROF = 1: the first wave of every workgroup also records when the workgroup's phases began and ended (wall clock) and
-// how many shader cycles its main loop took: a profiling build of the same code, launched only while a recording buffer
-// is set (jf_igemm_phase_record).
+// how many shader cycles its main loop took: a profiling build of the same code, instantiated only in the measurement
+// library (jf_prof_igemm_block_q).
 template <int EPI, typename ST, int WGM, int WGN, int NSTAGE, int WGPC, int BKN, int AKM = 0, int PROF = 0>
 __global__ __launch_bounds__(64 * WGM * WGN, WGPC * WGM * WGN / 4) void igemm_nt_kernel(GemmArgs p_in)
 {
