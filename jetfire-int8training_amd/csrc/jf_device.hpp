@@ -284,14 +284,15 @@ __device__ __forceinline__ float phi_neg(float x)
     p = __builtin_fmaf(p, x, 4.98673469e-02f);
     float u = __builtin_fmaf(p, x, 1.0f);
     u = u * u; u = u * u; u = u * u; u = u * u;
-    u = fminf(u, 1.2676506e30f);                      // 2^100: keeps the seed below in range (Phi(-x) < 4e-31 there)
+    u = fminf(u, 1.2676506e30f);                      // 2^100 (x > 12.4): keeps the seed below in range; the result is 0 there
     float r = __int_as_float(0x7EF311C7 - __float_as_int(u));     // 1/u to 12 %; each step squares the error
 #pragma unroll
     for (int i = 0; i < 3; ++i) {
         const float e = __builtin_fmaf(-u, r, 1.0f);
         r = __builtin_fmaf(r, e, r);
     }
-    return 0.5f * r;
+    // beyond the clamp Phi(-x) < 4e-31 is returned as 0, so that x * Phi(-x) vanishes for huge x as the function does
+    return u < 1.2676506e30f ? 0.5f * r : 0.0f;
 }
 
 __device__ __forceinline__ float norm_cdf(float x)
@@ -403,6 +404,21 @@ __device__ __forceinline__ void gather16(const float *table, v4i p, float x[16])
         x[4 * i + 3] = table[w[i] >> 24];
     }
 }
+// The largest of a lane's 16 codes (signed bytes): one SDWA instruction per code (the operand's byte, sign-extended).
+__device__ __forceinline__ int max_code16(v4i p)
+{
+    int m = -128;
+#define JF_MAXB(W, B) asm("v_max_i32_sdwa %0, sext(%1), %2 dst_sel:DWORD dst_unused:UNUSED_PAD src0_sel:BYTE_" #B " src1_sel:DWORD" \
+                          : "=v"(m) : "v"(W), "v"(m))
+#define JF_MAXW(W) JF_MAXB(W, 0); JF_MAXB(W, 1); JF_MAXB(W, 2); JF_MAXB(W, 3)
+    JF_MAXW(p.x); JF_MAXW(p.y); JF_MAXW(p.z); JF_MAXW(p.w);
+#undef JF_MAXW
+#undef JF_MAXB
+    return m;
+}
+// max |gelu(x)| over x <= 0 is 0.169972 (erf form, at x = -0.7516) and 0.170041 (tanh form, at x = -0.7525) in this
+// library's arithmetic (checked over the whole negative axis on the host); the bound leaves 6e-5 above both.
+constexpr float GELU_NEG_BOUND = 0.1701f;
 __device__ __forceinline__ void table_done()
 {
     __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
@@ -419,12 +435,24 @@ __device__ __forceinline__ v4i gelu_fwd_block(v4i c, float sc, float f0, float a
     fill_code_table(tab, lane, sc, f0, [](float v, float &a, float &b) { gelu_pair<APPROX>(v, a, b); });
     // The outputs take at most 256 distinct values too, so the requantisation (exact division, rounding, clamp) is
     // done on the table, 4 entries per lane, once the block's absmax is known; an element costs two gathers.
-    float x[16];
-    gather16(tab, c, x);
-    float m = 0.0f;
+    // The block's absmax.  x * Phi(x) rises with x > 0 (from one code to the next by at least 1/127 of itself, five
+    // orders of magnitude above the table's rounding errors), so among the positive codes present the largest code has
+    // the largest table entry, and no entry of a code <= 0 exceeds GELU_NEG_BOUND in magnitude at any scale.  A lane
+    // therefore looks up the entry of its own largest code only; if the wave's maximum of those reaches the bound it
+    // is the block's absmax.  Otherwise (no positive code, all of them tiny, a scale that overflows) every element's
+    // entry is looked at.
+    const int cl = max_code16(c);
+    const float tl = tab[cl & 0xFF];
+    float amax0 = wave_max(cl > 0 ? tl : 0.0f);
+    if (!(amax0 >= GELU_NEG_BOUND && amax0 < __builtin_inff())) {   // uniform
+        float x[16];
+        gather16(tab, c, x);
+        float m = 0.0f;
 #pragma unroll
-    for (int k = 0; k < 16; ++k) m = fmaxf(m, fabsf(x[k]));
-    const float amax = wave_max(m) + amax_eps;
+        for (int k = 0; k < 16; ++k) m = fmaxf(m, fabsf(x[k]));
+        amax0 = wave_max(m);
+    }
+    const float amax = amax0 + amax_eps;
     float scale = 0.0f;
     v4i codes = {0, 0, 0, 0};
     if (amax > 0.0f) {                                         // uniform
@@ -441,12 +469,24 @@ __device__ __forceinline__ v4i gelu_fwd_block(v4i c, float sc, float f0, float a
         __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
         __builtin_amdgcn_wave_barrier();
         __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
-        const unsigned char *q8 = reinterpret_cast<const unsigned char *>(qtab);
-        const uint32_t wd[4] = {(uint32_t)c.x, (uint32_t)c.y, (uint32_t)c.z, (uint32_t)c.w};
+        // entry address = table + the code's byte: one SDWA add per element (the operand's byte, zero-extended)
+        typedef __attribute__((address_space(3))) unsigned char lds_u8;
+        const uint32_t q8 = (uint32_t)(uintptr_t)(lds_u8 *)qtab;
+        const int wd[4] = {c.x, c.y, c.z, c.w};
         int o[4];
 #pragma unroll
-        for (int i = 0; i < 4; ++i)
-            o[i] = (int)pack4(q8[wd[i] & 0xFF], q8[(wd[i] >> 8) & 0xFF], q8[(wd[i] >> 16) & 0xFF], q8[wd[i] >> 24]);
+        for (int i = 0; i < 4; ++i) {
+            uint32_t a0, a1, a2, a3;
+#define JF_ADDB(DST, B) asm("v_add_u32_sdwa %0, %1, %2 dst_sel:DWORD dst_unused:UNUSED_PAD src0_sel:BYTE_" #B " src1_sel:DWORD" \
+                            : "=v"(DST) : "v"(wd[i]), "v"(q8))
+            JF_ADDB(a0, 0); JF_ADDB(a1, 1); JF_ADDB(a2, 2); JF_ADDB(a3, 3);
+#undef JF_ADDB
+            const uint32_t b0 = *(const lds_u8 *)(uintptr_t)a0, b1 = *(const lds_u8 *)(uintptr_t)a1;
+            const uint32_t b2 = *(const lds_u8 *)(uintptr_t)a2, b3 = *(const lds_u8 *)(uintptr_t)a3;
+            // four zero-extended bytes into one word with three byte permutes
+            o[i] = (int)__builtin_amdgcn_perm(__builtin_amdgcn_perm(b3, b2, 0x0c0c0400u), __builtin_amdgcn_perm(b1, b0, 0x0c0c0400u),
+                                              0x05040100u);
+        }
         codes = v4i{o[0], o[1], o[2], o[3]};
     }
     table_done();

@@ -389,7 +389,8 @@ float jfo_phi_neg(float x)
         float e = fmaf(-u, r, 1.0f);
         r = fmaf(r, e, r);
     }
-    return 0.5f * r;
+    /* beyond the clamp (x > 12.4, Phi(-x) < 4e-31) the result is 0, so that x * Phi(-x) vanishes for huge x */
+    return u < 1.2676506e30f ? 0.5f * r : 0.0f;
 }
 
 /* Phi(x) = (1+erf(x/sqrt2))/2  (gelu_fwd.py:81) */

@@ -383,7 +383,8 @@ def test_block_column_sums(jf, oracle, R, C, f16):
 def test_gelu_fwd_on_one_sided_and_degenerate_blocks(jf, oracle, approx, eps, f16):
     """Blocks whose absmax is not where random data puts it: only negative codes, on one side of the minimum of x*Phi(x)
     (at x = -0.75) or straddling it, a single code, the byte -128, far tails where the outputs are a few units of 2^-24,
-    all zeros, a zero scale, scales from 1e-4 to 40."""
+    all zeros, a zero scale, scales from 1e-4 to 40; blocks whose largest positive output lies just below or above the
+    largest magnitude a negative input can produce."""
     rng = np.random.default_rng(77 + approx)
     blocks, scales = [], []
 
@@ -402,6 +403,15 @@ def test_gelu_fwd_on_one_sided_and_degenerate_blocks(jf, oracle, approx, eps, f1
         add([int(rng.integers(-127, 128))], scale)                           # one code
         add(rng.integers(-127, 128, QB * QB), scale)
         add(np.where(rng.random(QB * QB) < 0.9, 0, rng.integers(-127, 0, QB * QB)), scale)
+        # the largest positive output on either side of 0.1701 (x = 0.279), where the kernel changes how it finds the
+        # block's absmax, with negative codes on both sides of the minimum; one positive element among negative ones
+        kp = min(int(0.279 / scale), 126)
+        for top in (kp, kp + 1):
+            if top >= 1:
+                add(np.where(rng.random(QB * QB) < 0.5, rng.integers(1, top + 1, QB * QB), rng.integers(-127, 0, QB * QB)), scale)
+        lone = rng.integers(-127, 0, QB * QB)
+        lone[int(rng.integers(0, QB * QB))] = int(rng.integers(1, 128))
+        add(lone, scale)
     add(np.zeros(QB * QB), 1.0)
     add(rng.integers(-127, 128, QB * QB), 0.0)
     n = len(blocks)

@@ -376,6 +376,27 @@ def test_gelu_and_derivative_vs_torch(oracle, approx, name):
     assert np.max(np.abs(oracle.dgelu(x, approx) - xt.grad.numpy())) < 2e-6
 
 
+@pytest.mark.parametrize("approx", [0, 1])
+def test_gelu_table_properties_the_forward_kernel_relies_on(oracle, approx):
+    """The GELU forward kernel finds a block's absmax from the table entry of its largest positive code when that entry
+    is at least 0.1701.  That is exact if (a) the entries of the positive codes 1..127 rise with the code at every
+    scale, and (b) no input <= 0 gives an output above 0.1701 in magnitude.  Both are properties of this library's
+    arithmetic (the oracle's function has the device's bits), checked here for every binary16 scale, 40000 binary32
+    scales over the whole exponent range and two million points of the negative axis."""
+    rng = np.random.default_rng(5)
+    codes = np.arange(1, 128, dtype=np.float32)
+    scales = np.concatenate([np.arange(1, 0x7C00, dtype=np.uint16).view(np.float16).astype(np.float32),
+                             np.exp(rng.uniform(np.log(1e-44), np.log(2.6e36), 40000)).astype(np.float32)])
+    for chunk in np.array_split(scales, 16):
+        x = (codes[None, :] * chunk[:, None]).astype(np.float32)
+        y = oracle.gelu(x.ravel(), approx).reshape(x.shape)
+        assert np.isfinite(y).all() and (np.diff(y, axis=1) >= 0).all() and (y >= 0).all()
+    neg = -np.linspace(0.0, 40.0, 2_000_001).astype(np.float32)
+    assert np.abs(oracle.gelu(neg, approx)).max() < 0.17005
+    tails = -np.exp(rng.uniform(np.log(1e-44), np.log(3e38), 200000)).astype(np.float32)
+    assert np.abs(oracle.gelu(tails, approx)).max() < 0.17005
+
+
 # ----------------------------------------------------------------------------- fused nonlinear ops
 def _rand_block_tensor(rng, R, Cc, scale=1.0):
     x = (rng.standard_normal((R, Cc)) * scale).astype(np.float32)
