@@ -185,94 +185,56 @@ __global__ __launch_bounds__(NT) void dequantize_kernel(const int8_t *q, const S
     }
 }
 
-// A wave that loads one block (1 KiB of codes), waits, computes and stores keeps far too few bytes in flight to
-// cover the memory latency, so the streaming kernels run their block loop with the codes and scales of the next PF
-// blocks already requested.  The PF request slots are named at compile time (the loop body is unrolled PF times, slot
-// s serving the iterations s, s + PF, ...): moving the slots' registers down a queue instead would make every
-// iteration wait for ALL outstanding loads (a register cannot be copied before its load has landed), which is no
-// prefetch at all.
-constexpr int PF = 3;
-// Walks the blocks blk0, blk0 + stride, ... of a wave without a division per block: (row block, column block) advance
-// by (stride / SC, stride % SC) with a carry.
-struct BlockWalk {
-    int rb, cb, drb, dcb, SC;
-    __device__ __forceinline__ BlockWalk(int blk0, int stride, int SC_) : SC(SC_)
-    {
-        rb = blk0 / SC; cb = blk0 - rb * SC;
-        drb = stride / SC; dcb = stride - drb * SC;
-    }
-    __device__ __forceinline__ void step()
-    {
-        rb += drb; cb += dcb;
-        if (cb >= SC) { cb -= SC; ++rb; }
-    }
-};
-// body(walk, slot) for every block of the walk while walk.rb < RB; slot = iteration number mod PF as a compile-time
-// constant.  The body takes the slot's data and then refills the slot (the block PF iterations ahead).  Whole groups
-// of PF blocks run in a loop without exits inside it (so that the slots' registers are the loop's own, not copies
-// made on the way round); the last, partial group follows.
-template <typename Body> __device__ __forceinline__ void for_each_block_pipelined(BlockWalk w, int RB, int blk0, int stride, Body body)
+// Code tensors leave the GELU kernels in whole 128-byte row pieces.  A wave works on one 32x32 block in the row layout
+// (lane l: row l/2, 16 bytes), in which a store instruction touches 32 rows with 32 bytes each: a quarter of each
+// 128-byte line.  Out of the caches that costs a third of the bandwidth (a copy of 8192x6400 bytes: 30 us when written
+// in that shape, 23 us read in that shape but written in whole lines, 21 us with both in whole lines).  So a wave
+// works through four adjacent blocks (a group; the last group of a row may be partial), leaves each block's codes in
+// a wave-private 32 x 128-byte patch in LDS (padded to 144 bytes per row) and then stores the group's 32 rows, 128
+// bytes each (lane l: rows l/8, l/8 + 8, .., bytes 16*(l%8) ..).  All blocks of a group are requested at once, so the
+// later ones arrive while the first is worked on; one group per wave and many workgroups beat fewer, longer-lived ones
+// with requests further ahead here (the dispatcher evens them out).
+constexpr int LINE_PITCH = 4 * QB + 16;
+__device__ __forceinline__ void group_put(unsigned char *patch, int lane, int j, v4i codes)
 {
-    const int nblk = RB * w.SC;
-    const int n = blk0 < nblk ? (nblk - blk0 + stride - 1) / stride : 0;     // blocks of this wave (uniform)
-    for (int i = n / PF; i > 0; --i) {
-        static_for<0, PF>([&](auto slot_c) {
-            body(w, slot_c);
-            w.step();
-        });
-    }
-    const int rem = n % PF;
-    static_for<0, PF - 1>([&](auto slot_c) {
-        if (decltype(slot_c)::value < rem) {
-            body(w, slot_c);
-            w.step();
-        }
-    });
+    *reinterpret_cast<v4i *>(patch + (lane >> 1) * LINE_PITCH + QB * j + 16 * (lane & 1)) = codes;
 }
-template <typename ST> struct CodeStream {
-    const int8_t *q;
-    const ST *s;
-    int C, RB, lane;
-    BlockWalk at;                 // the next block to request
-    v4i codes[PF];
-    float scale[PF];
-    template <int SLOT> __device__ __forceinline__ void request()
-    {
-        if (at.rb < RB) {
-            codes[SLOT] = *reinterpret_cast<const v4i *>(q + (size_t)(at.rb * QB + (lane >> 1)) * C + at.cb * QB + (lane & 1) * 16);
-            scale[SLOT] = load_scale(s, at.rb * at.SC + at.cb);
+__device__ __forceinline__ void group_store_lines(unsigned char *patch, int lane, int8_t *out, int rb, int cg, int C)
+{
+    __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
+    __builtin_amdgcn_wave_barrier();
+    __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
+    const int lcol = 16 * (lane & 7);
+    if (cg * 4 * QB + lcol < C) {
+#pragma unroll
+        for (int k = 0; k < 4; ++k) {
+            const int row = 8 * k + (lane >> 3);
+            *reinterpret_cast<v4i *>(out + (size_t)(rb * QB + row) * C + cg * 4 * QB + lcol) =
+                *reinterpret_cast<const v4i *>(patch + row * LINE_PITCH + lcol);
         }
-        at.step();
     }
-    __device__ __forceinline__ CodeStream(const int8_t *q_, const ST *s_, int R, int C_, int stride, int lane_, int blk0)
-        : q(q_), s(s_), C(C_), RB(R / QB), lane(lane_), at(blk0, stride, C_ / QB)
-    {
-        static_for<0, PF>([&](auto i) { request<decltype(i)::value>(); });
+    __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
+    __builtin_amdgcn_wave_barrier();                               // the patch may be rewritten
+}
+// The (up to) four blocks of group (rb, cg) of a block tensor, in the row layout, and their scales.
+template <typename ST>
+__device__ __forceinline__ void group_request(const int8_t *q, const ST *s, int C, int rb, int cg, int lane, v4i (&c)[4], float (&sc)[4])
+{
+    const int SC = C / QB;
+#pragma unroll
+    for (int j = 0; j < 4; ++j) {
+        // beyond the end of a row the last block is read again (and not used): four loads in a straight line, whose
+        // arrivals the compiler can then count one by one
+        const int cb = (cg * 4 + j < SC) ? cg * 4 + j : SC - 1;
+        c[j] = *reinterpret_cast<const v4i *>(q + (size_t)(rb * QB + (lane >> 1)) * C + cb * QB + (lane & 1) * 16);
+        sc[j] = load_scale(s, rb * SC + cb);
     }
-    // hands out the slot's block; refill() then requests the block PF iterations ahead into the same slot
-    template <int SLOT> __device__ __forceinline__ void take(v4i &c, float &sc) const { c = codes[SLOT]; sc = scale[SLOT]; }
-    template <int SLOT> __device__ __forceinline__ void refill() { request<SLOT>(); }
-};
-
-// The same walk for a per-row fp32 vector (mean, rstd): the lane's row of each block, requested PF blocks ahead.
-struct RowStream {
-    const float *v;
-    int RB, lane;
-    BlockWalk at;
-    float val[PF];
-    template <int SLOT> __device__ __forceinline__ void request()
-    {
-        if (at.rb < RB) val[SLOT] = v[at.rb * QB + (lane >> 1)];
-        at.step();
-    }
-    __device__ __forceinline__ RowStream(const float *v_, int R, int SC, int stride, int lane_, int blk0)
-        : v(v_), RB(R / QB), lane(lane_), at(blk0, stride, SC)
-    {
-        static_for<0, PF>([&](auto i) { request<decltype(i)::value>(); });
-    }
-    template <int SLOT> __device__ __forceinline__ float take() const { return val[SLOT]; }
-    template <int SLOT> __device__ __forceinline__ void refill() { request<SLOT>(); }
-};
+}
+static inline int grid_for_groups(int R, int C)
+{
+    const long groups = (long)(R / QB) * ((C / QB + 3) / 4), g = (groups + WPB - 1) / WPB;
+    return (int)(g < 256L * 16 ? g : 256L * 16);
+}
 
 // gelu_fwd.py:34-126
 template <int APPROX, typename ST>
@@ -281,54 +243,70 @@ __global__ __launch_bounds__(NT) void gelu_fwd_kernel(const int8_t *q, const ST 
 {
     __shared__ __attribute__((aligned(16))) float table[WPB][256];
     __shared__ __attribute__((aligned(16))) int qtable[WPB][64];      // 256 one-byte entries per wave
-    float *tab = table[threadIdx.x >> 6];
-    int *qtab = qtable[threadIdx.x >> 6];
-    const int lane = threadIdx.x & 63, SC = C / QB, RB = R / QB, stride = gridDim.x * WPB;
-    const int blk0 = __builtin_amdgcn_readfirstlane(blockIdx.x * WPB + (threadIdx.x >> 6));
-    CodeStream<ST> in(q, s, R, C, stride, lane, blk0);
+    __shared__ __attribute__((aligned(16))) unsigned char patches[WPB][QB * LINE_PITCH];
+    const int lane = threadIdx.x & 63, wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
+    float *tab = table[wave];
+    int *qtab = qtable[wave];
+    unsigned char *patch = patches[wave];
+    const int SC = C / QB, SG = (SC + 3) / 4, ngrp = (R / QB) * SG, stride = gridDim.x * WPB;
+    int g = blockIdx.x * WPB + wave;
+    if (g >= ngrp) return;
     float zero = 0.0f;
     asm volatile("" : "+v"(zero));                                 // evaluated on the device, like every other entry
     const float f0 = gelu<APPROX>(zero);
-    for_each_block_pipelined(BlockWalk(blk0, stride, SC), RB, blk0, stride, [&](const BlockWalk &w, auto slot_c) {
-        constexpr int SLOT = decltype(slot_c)::value;
-        const size_t e0 = (size_t)(w.rb * QB + (lane >> 1)) * C + w.cb * QB + (lane & 1) * 16;
-        v4i c; float sc;
-        in.template take<SLOT>(c, sc);
-        float scale;
-        const v4i codes = gelu_fwd_block<APPROX>(c, sc, f0, amax_eps, tab, qtab, lane, &scale);
-        in.template refill<SLOT>();                                // after the last use of c: the load lands in its registers
-        *reinterpret_cast<v4i *>(qy + e0) = codes;
-        if (lane == 0) store_scale(sy, w.rb * SC + w.cb, scale);
-    });
+    for (; g < ngrp; g += stride) {
+        const int rb = g / SG, cg = g - rb * SG;
+        v4i cur[4];
+        float csc[4];
+        group_request(q, s, C, rb, cg, lane, cur, csc);            // the later blocks arrive while the first is worked on
+#pragma unroll
+        for (int j = 0; j < 4; ++j) {
+            const int cb = cg * 4 + j;
+            if (cb < SC) {                                         // uniform
+                float scale;
+                group_put(patch, lane, j, gelu_fwd_block<APPROX>(cur[j], csc[j], f0, amax_eps, tab, qtab, lane, &scale));
+                if (lane == 0) store_scale(sy, rb * SC + cb, scale);
+            }
+        }
+        group_store_lines(patch, lane, qy, rb, cg, C);
+    }
 }
 
 // gelu_bwd.py:28-171
 template <int APPROX, typename ST>
-__global__ __launch_bounds__(NT) void gelu_bwd_kernel(const int8_t *qx, const ST *sx, const int8_t *qg, const ST *sg,
+__global__ __launch_bounds__(NT) __attribute__((amdgpu_waves_per_eu(5, 5))) void gelu_bwd_kernel(const int8_t *qx, const ST *sx, const int8_t *qg, const ST *sg,
                                                       int R, int C, int rounding, uint64_t seed, uint64_t offset,
                                                       int8_t *qy, ST *sy)
 {
     __shared__ __attribute__((aligned(16))) float table[WPB][256];
-    float *tab = table[threadIdx.x >> 6];
-    const int lane = threadIdx.x & 63, SC = C / QB, RB = R / QB, stride = gridDim.x * WPB;
-    const int blk0 = __builtin_amdgcn_readfirstlane(blockIdx.x * WPB + (threadIdx.x >> 6));
-    CodeStream<ST> inx(qx, sx, R, C, stride, lane, blk0), ing(qg, sg, R, C, stride, lane, blk0);
+    __shared__ __attribute__((aligned(16))) unsigned char patches[WPB][QB * LINE_PITCH];
+    const int lane = threadIdx.x & 63, wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
+    float *tab = table[wave];
+    unsigned char *patch = patches[wave];
+    const int SC = C / QB, SG = (SC + 3) / 4, ngrp = (R / QB) * SG, stride = gridDim.x * WPB;
+    int g = blockIdx.x * WPB + wave;
+    if (g >= ngrp) return;
     float zero = 0.0f;
     asm volatile("" : "+v"(zero));
     const float f0 = dgelu<APPROX>(zero);
-    for_each_block_pipelined(BlockWalk(blk0, stride, SC), RB, blk0, stride, [&](const BlockWalk &w, auto slot_c) {
-        constexpr int SLOT = decltype(slot_c)::value;
-        const size_t e0 = (size_t)(w.rb * QB + (lane >> 1)) * C + w.cb * QB + (lane & 1) * 16;
-        v4i cx, cg; float scx, scg;
-        inx.template take<SLOT>(cx, scx);
-        ing.template take<SLOT>(cg, scg);
-        float scale;
-        v4i codes = gelu_bwd_block<APPROX>(cx, scx, cg, scg, f0, tab, lane, rounding, seed, offset, e0, &scale);
-        inx.template refill<SLOT>();                               // after the last use of the slot's registers
-        ing.template refill<SLOT>();
-        *reinterpret_cast<v4i *>(qy + e0) = codes;
-        if (lane == 0) store_scale(sy, w.rb * SC + w.cb, scale);
-    });
+    for (; g < ngrp; g += stride) {
+        const int rb = g / SG, cg = g - rb * SG;
+        v4i cx[4], cgr[4];
+        float scx[4], scg[4];
+        group_request(qx, sx, C, rb, cg, lane, cx, scx);
+        group_request(qg, sg, C, rb, cg, lane, cgr, scg);
+#pragma unroll
+        for (int j = 0; j < 4; ++j) {
+            const int cb = cg * 4 + j;
+            if (cb < SC) {                                         // uniform
+                const size_t e0 = (size_t)(rb * QB + (lane >> 1)) * C + cb * QB + (lane & 1) * 16;
+                float scale;
+                group_put(patch, lane, j, gelu_bwd_block<APPROX>(cx[j], scx[j], cgr[j], scg[j], f0, tab, lane, rounding, seed, offset, e0, &scale));
+                if (lane == 0) store_scale(sy, rb * SC + cb, scale);
+            }
+        }
+        group_store_lines(patch, lane, qy, rb, cg, C);
+    }
 }
 
 // layernorm.py:74-190, with a real beta.  Arithmetic (this library's definition; the reference dequantises in binary16):
@@ -994,15 +972,6 @@ static inline int grid_for_blocks(int R, int C)
     return (int)(g < cap ? g : cap);
 }
 
-// kernels that keep several blocks in flight per wave and have per-kernel setup: no more workgroups than are resident
-static inline int grid_for_resident(int R, int C)
-{
-    const long nblk = (long)(R / QB) * (C / QB);
-    long g = (nblk + WPB - 1) / WPB;
-    const long cap = 256L * 8;
-    return (int)(g < cap ? g : cap);
-}
-
 static int check_block_tensor(const void *q, const void *s, int R, int C, int scale_dtype)
 {
     if (!q || !s) return JF_ERR_NULL;
@@ -1307,7 +1276,7 @@ int jf_gelu_fwd(const int8_t *q, const void *s, int R, int C, int scale_dtype, i
     if (approx != JF_GELU_ERF && approx != JF_GELU_TANH) return JF_ERR_ENUM;
     if (!aligned16(qy)) return JF_ERR_ALIGN;
     hipStream_t st = (hipStream_t)stream;
-    const int grid = grid_for_resident(R, C);
+    const int grid = grid_for_groups(R, C);
 #define JF_GF(A, ST) JF_LAUNCH((gelu_fwd_kernel<A, ST>), grid, 0, st, q, (const ST *)s, R, C, amax_eps, qy, (ST *)sy)
     if (scale_dtype == JF_SCALE_F16) {
         if (approx == JF_GELU_ERF) JF_GF(JF_GELU_ERF, half_t);
@@ -1329,7 +1298,7 @@ int jf_gelu_bwd(const int8_t *qx, const void *sx, const int8_t *qg, const void *
     if ((approx != JF_GELU_ERF && approx != JF_GELU_TANH) || !rounding_ok(rounding)) return JF_ERR_ENUM;
     if (!aligned16(qy)) return JF_ERR_ALIGN;
     hipStream_t st = (hipStream_t)stream;
-    const int grid = grid_for_resident(R, C);
+    const int grid = grid_for_groups(R, C);
 #define JF_GB(A, ST)                                                                                              \
     JF_LAUNCH((gelu_bwd_kernel<A, ST>), grid, 0, st, qx, (const ST *)sx, qg, (const ST *)sg, R, C, rounding, seed, \
               offset, qy, (ST *)sy)
