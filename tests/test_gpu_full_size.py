@@ -289,3 +289,34 @@ def test_cfg4_gelu_backward_full_size(jf, oracle, approx):
         wq, ws = oracle.gelu_fwd(X, SX, approx, eps)
         same(qy[rows], wq, f"forward codes rows {r0}")
         same(sy[rb], ws, f"forward scales rows {r0}")
+
+
+@pytest.mark.parametrize("approx", [0, 1])
+def test_gelu_whole_output_against_row_slices_and_more_groups_than_waves(jf, oracle, approx):
+    """A wave of the GELU kernels takes a group of four adjacent blocks, and at most 16384 waves are launched: 8192 x 8352
+    has 256 x 66 = 16896 groups (the last group of a row is a single block), so some waves take a second group.  The
+    whole outputs must equal what the same kernels give on 512-row slices (1056 groups each; the noise of a slice is
+    that of its rows in the whole tensor: offset + first row * C / 8), and two strips are checked against the oracle."""
+    R, C = 8192, 8352
+    g = torch.Generator().manual_seed(3)
+    f32 = torch.float32
+    qx, sx = jf.quantize(torch.randn(R, C, generator=g).cuda(), scale_dtype=f32)
+    qg, sg = jf.quantize((1e-3 * torch.randn(R, C, generator=g)).cuda(), jf.ROUND_STOCHASTIC, f32, seed=0, offset=0)
+    eps = 5e-5 if approx == 0 else 0.0
+    qy, sy = jf.gelu_fwd(qx, sx, approx, eps)
+    qd, sd = jf.gelu_bwd(qx, sx, qg, sg, approx, jf.ROUND_STOCHASTIC, seed=6, offset=4)
+    for r0 in range(0, R, 512):
+        rows, rb = slice(r0, r0 + 512), slice(r0 // QB, (r0 + 512) // QB)
+        py, ps = jf.gelu_fwd(qx[rows], sx[rb], approx, eps)
+        assert torch.equal(py, qy[rows]) and torch.equal(ps, sy[rb]), f"forward rows {r0}"
+        pd, ps = jf.gelu_bwd(qx[rows], sx[rb], qg[rows], sg[rb], approx, jf.ROUND_STOCHASTIC, seed=6, offset=4 + r0 * C // 8)
+        assert torch.equal(pd, qd[rows]) and torch.equal(ps, sd[rb]), f"backward rows {r0}"
+    for r0 in (0, R - QB):
+        rows, rb = slice(r0, r0 + QB), slice(r0 // QB, r0 // QB + 1)
+        X, SX, G, SG = (t.cpu().numpy() for t in (qx[rows], sx[rb], qg[rows], sg[rb]))
+        wq, ws = oracle.gelu_fwd(X, SX, approx, eps)
+        same(qy[rows], wq, f"forward codes rows {r0}")
+        same(sy[rb], ws, f"forward scales rows {r0}")
+        wq, ws = oracle.gelu_bwd(X, SX, G, SG, approx, True, 6, 4 + r0 * C // 8)
+        same(qd[rows], wq, f"backward codes rows {r0}")
+        same(sd[rb], ws, f"backward scales rows {r0}")
