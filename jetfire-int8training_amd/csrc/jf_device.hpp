@@ -65,8 +65,8 @@ __device__ __forceinline__ float wave_max(float v)
 // ---------------------------------------------------------------------------------------------
 // Philox4x32-R.  (Salmon et al., "Parallel random numbers: as easy as 1, 2, 3", SC'11.)  The rounding noise uses
 // R = 7, the smallest round count the authors report as passing BigCrush (10 is their default with a safety margin):
-// the generator is the largest single cost of every stochastic-rounding kernel here, and its multiplies run at a
-// quarter of the vector ALU's rate.
+// the generator is the largest single cost of every stochastic-rounding kernel here (its 64-bit multiplies take twice
+// the issue time of a plain fp32 instruction).
 // Build-time switch: -DJF_PHILOX_ROUNDS=10 gives the reference generator's round count (curandStatePhilox4_32_10,
 // tl.rand); jf_philox_rounds() reports what a library was built with, and the CPU checker follows it.
 #ifndef JF_PHILOX_ROUNDS
