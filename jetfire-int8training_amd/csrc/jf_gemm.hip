@@ -744,8 +744,8 @@ __global__ __launch_bounds__(64 * WGM * WGN, WGPC * WGM * WGN / 4) void igemm_nt
                 v4i codes = {0, 0, 0, 0};
                 float scale = 0.0f;
                 if (amax > 0.0f) {
-                    scale = amax / 127.0f;
                     BlockDivisor d(amax);
+                    scale = d.fast ? div_by_127_in_range(amax) : amax / 127.0f;      // (uniform)
                     float t[16];
                     if (p.bias) {
 #pragma unroll

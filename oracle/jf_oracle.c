@@ -674,6 +674,23 @@ float jfo_model_fast_div(float x, float s)
     return fmaf(e, r, q0);
 }
 
+/* Model of the device's division of a block maximum by 127 (q0 = a * rn(1/127), e = fmaf(-q0, 127, a),            */
+/* q = fmaf(e, rn(1/127), q0)): counts the mantissas, over the binades 2^lo .. 2^hi, for which it differs from the   */
+/* IEEE a / 127.0f that the functions above use.                                                                     */
+long jfo_model_div127_mismatches(int lo, int hi)
+{
+    const float r = 1.0f / 127.0f;
+    long bad = 0;
+    for (int ex = lo; ex <= hi; ++ex)
+        for (uint32_t m = 0; m < (1u << 23); ++m) {
+            uint32_t bits = ((uint32_t)(127 + ex) << 23) | m;
+            float a; memcpy(&a, &bits, 4);
+            float q0 = a * r, e = fmaf(-q0, 127.0f, a), q = fmaf(e, r, q0), w = a / 127.0f;
+            if (memcmp(&q, &w, 4) != 0) bad++;
+        }
+    return bad;
+}
+
 long jfo_model_fast_div_mismatches(const float *x, const float *s, long n)
 {
     long bad = 0;

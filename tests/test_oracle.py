@@ -345,6 +345,18 @@ def test_fast_division_model_equals_ieee(oracle):
         assert L.jfo_model_fast_div_mismatches(x.ctypes.data, s.ctypes.data, n) == 0
 
 
+def test_division_by_127_model_equals_ieee(oracle):
+    """amax / 127 as the kernels form it inside (2^-53, 2^66) (a multiplication by rn(1/127) corrected by two fmas) ==
+    the IEEE quotient: every mantissa of three binades (the arithmetic is the same in every binade while nothing
+    underflows) and of the two binades at either end of the range it is used on."""
+    L = oracle.lib()
+    L.jfo_model_div127_mismatches.argtypes = [C.c_int, C.c_int]
+    L.jfo_model_div127_mismatches.restype = C.c_long
+    assert L.jfo_model_div127_mismatches(-1, 1) == 0
+    assert L.jfo_model_div127_mismatches(-53, -52) == 0
+    assert L.jfo_model_div127_mismatches(65, 66) == 0
+
+
 # ----------------------------------------------------------------------------- elementary functions
 def test_exp_phi_cdf_tanh_vs_scipy(oracle):
     import scipy.special as sp
