@@ -347,7 +347,7 @@ template <int APPROX> __device__ __forceinline__ float dgelu(float x)
         float pdf = 0.398942280f * expf_det(-0.5f * (x * x));
         return __builtin_fmaf(x, pdf, norm_cdf(x));
     }
-    float x2 = x * x;
+    float x2 = fminf(x * x, 1e30f);                        // (keeps dinner finite: sech2 is exactly 0 long before, and 0 * inf is not)
     float inner = 0.797884561f * (x * __builtin_fmaf(0.044715f, x2, 1.0f));
     float t = tanhf_det(inner);
     float dinner = 0.797884561f * __builtin_fmaf(0.134145f, x2, 1.0f);
@@ -383,7 +383,7 @@ template <int APPROX> __device__ __forceinline__ void dgelu_pair(float x, float 
         neg = __builtin_fmaf(-x, pdf, h);
         return;
     }
-    const float x2 = x * x;
+    const float x2 = fminf(x * x, 1e30f);
     const float inner = 0.797884561f * (x * __builtin_fmaf(0.044715f, x2, 1.0f));
     const float t = tanhf_det(inner);
     const float dinner = 0.797884561f * __builtin_fmaf(0.134145f, x2, 1.0f);

@@ -426,7 +426,7 @@ float jfo_dgelu(float x, int approx)
         float pdf = 0.398942280f * jfo_expf(-0.5f * (x * x));
         return fmaf(x, pdf, jfo_norm_cdf(x));
     }
-    float x2 = x * x;
+    float x2 = fminf(x * x, 1e30f);      /* keeps dinner finite: sech2 is exactly 0 long before, and 0 * inf is not */
     float inner = 0.797884561f * (x * fmaf(0.044715f, x2, 1.0f));
     float t = jfo_tanhf(inner);
     float dinner = 0.797884561f * fmaf(0.134145f, x2, 1.0f);

@@ -386,6 +386,10 @@ def test_gelu_and_derivative_vs_torch(oracle, approx, name):
     yt.sum().backward()
     assert np.max(np.abs(oracle.gelu(x, approx) - yt.detach().numpy())) < 1.5e-6
     assert np.max(np.abs(oracle.dgelu(x, approx) - xt.grad.numpy())) < 2e-6
+    # far out: the function itself for x > 0, -0 for x < 0; the derivative 1 and 0 (no 0 * inf, no tail left of Phi)
+    big = np.array([50, 1e3, 1e10, 1e19, 1e20, 1e30, 3e38], dtype=np.float32)
+    assert np.array_equal(oracle.gelu(big, approx), big) and not oracle.gelu(-big, approx).any()
+    assert np.array_equal(oracle.dgelu(big, approx), np.ones_like(big)) and not oracle.dgelu(-big, approx).any()
 
 
 @pytest.mark.parametrize("approx", [0, 1])
