@@ -88,6 +88,32 @@ struct BlockPos {
     const int nblk = ((R) / QB) * SC;                                                      \
     for (int blk = blockIdx.x * WPB + (threadIdx.x >> 6); blk < nblk; blk += gridDim.x * WPB)
 
+// Codes leave in whole 128-byte lines.  In the row layout of a block (lane l: row l/2, 16 bytes) a store instruction
+// writes 32 rows x 32 bytes, a quarter of each line; out of the caches those quarter-line writes cost a third of the
+// bandwidth, also when the four waves of a workgroup write the four quarters at the same moment (copies of 8192 x 6400
+// bytes: 32 us that way, 23 us with the same reads and whole-line writes).  Kernels whose workgroup works on four adjacent
+// column blocks of one row block (a group; wave w: block 4*cg + w, idle beyond the end of the row) therefore exchange
+// the codes through a 32 x 128-byte patch in LDS (144 bytes per row) and wave w stores rows 8w .. 8w+7 of the group.
+// Two patches take turns, so one barrier per group is enough: a patch is rewritten two groups later, behind the
+// barrier of the group in between.  Every wave of the workgroup must make the call (it contains the barrier).
+constexpr int LINE_PITCH = 4 * QB + 16;
+struct GroupLineStore {
+    unsigned char *patches;       // [2][QB * LINE_PITCH], shared by the workgroup
+    int turn, lane, wave;
+    __device__ __forceinline__ GroupLineStore(unsigned char *p, int lane_, int wave_) : patches(p), turn(0), lane(lane_), wave(wave_) {}
+    __device__ __forceinline__ void store(v4i codes, int8_t *out, int rb, int cg, int C)
+    {
+        unsigned char *patch = patches + turn * (QB * LINE_PITCH);
+        turn ^= 1;
+        *reinterpret_cast<v4i *>(patch + (lane >> 1) * LINE_PITCH + QB * wave + 16 * (lane & 1)) = codes;
+        __syncthreads();
+        const int row = 8 * wave + (lane >> 3), lcol = 16 * (lane & 7);
+        if (cg * 4 * QB + lcol < C)
+            *reinterpret_cast<v4i *>(out + (size_t)(rb * QB + row) * C + cg * 4 * QB + lcol) =
+                *reinterpret_cast<const v4i *>(patch + row * LINE_PITCH + lcol);
+    }
+};
+
 // ------------------------------------------------------------------------------------------------
 // quantize.py:33-117 (and quantize_transpose.py:33-129 when qT != nullptr)
 // The input is up to QSRC_MAX column slabs lying side by side in the result: slab k is [R, end[k] - end[k-1]] with rows
@@ -98,7 +124,7 @@ struct BlockPos {
 __host__ __device__ static inline int quantize_groups(int R, int C, bool transposed)
 {
     const int RB = R / QB, SC = C / QB, G4 = (SC + WPB - 1) / WPB;
-    if (!transposed) return (RB * SC + WPB - 1) / WPB;
+    if (!transposed) return RB * G4;
     const int pairs = ((RB + 3) / 4) * G4;
     return 32 * ((pairs + 7) / 8);
 }
@@ -121,19 +147,25 @@ __global__ __launch_bounds__(NT) void quantize_kernel(QuantSrc src, int R, int C
     // written 32 bytes at a time by the workgroups of four consecutive row blocks: those four are made the workgroups
     // b, b+8, b+16, b+24, which the dispatcher deals to the same XCD one after the other, so that the four pieces of a
     // line meet in that XCD's L2 before the line leaves for memory (see quantize_groups() for the count).
-    const int nwg = qT ? quantize_groups(R, C, true) : (RB * SC + WPB - 1) / WPB;
+    const int nwg = quantize_groups(R, C, qT != nullptr);
+    __shared__ __attribute__((aligned(16))) unsigned char line_patches[2 * QB * LINE_PITCH];
+    GroupLineStore lines(line_patches, lane, wave);
     for (int wg = blockIdx.x; wg < nwg; wg += gridDim.x)
     {
-        int blk;
+        int rbq, cg;
         if (qT) {
             const int idx = (wg >> 5) * 8 + (wg & 7), j = (wg >> 3) & 3;     // (row-block quad, column group) and the row block of the quad
-            const int rbq = (idx / G4) * 4 + j, cbq = (idx % G4) * WPB + wave;
-            if (rbq >= RB || cbq >= SC) continue;                           // wave-uniform
-            blk = rbq * SC + cbq;
+            rbq = (idx / G4) * 4 + j; cg = idx % G4;
         } else {
-            blk = wg * WPB + wave;
-            if (blk >= RB * SC) continue;
+            rbq = wg / G4; cg = wg - rbq * G4;
         }
+        const int cbq = cg * WPB + wave;
+        const bool valid = rbq < RB && cbq < SC;                            // wave-uniform
+        if (!valid) {
+            if (!qT && rbq < RB) lines.store(v4i{0, 0, 0, 0}, q, rbq, cg, C);   // (the barrier; its bytes lie beyond the row's end)
+            continue;
+        }
+        const int blk = rbq * SC + cbq;
         BlockPos pos(blk, SC, C, lane);
         // the slab of this block (uniform over the wave; slabs are whole blocks wide)
         const T *x = reinterpret_cast<const T *>(src.x[0]);
@@ -145,7 +177,8 @@ __global__ __launch_bounds__(NT) void quantize_kernel(QuantSrc src, int R, int C
         Load16<T>::run(x + (size_t)pos.row * ldx + (pos.col - begin), v);
         float scale;
         v4i codes = quantize16(v, amax_eps, rounding, seed, offset, pos.e0, &scale);
-        *reinterpret_cast<v4i *>(q + pos.e0) = codes;
+        if (qT) *reinterpret_cast<v4i *>(q + pos.e0) = codes;
+        else lines.store(codes, q, rbq, cg, C);
         if (lane == 0) store_scale(s, pos.rb * SC + pos.cb, scale);
         if (qT) {
             unsigned char(*tp)[QB + 16] = tpatch[threadIdx.x >> 6];
@@ -194,7 +227,6 @@ __global__ __launch_bounds__(NT) void dequantize_kernel(const int8_t *q, const S
 // bytes each (lane l: rows l/8, l/8 + 8, .., bytes 16*(l%8) ..).  All blocks of a group are requested at once, so the
 // later ones arrive while the first is worked on; one group per wave and many workgroups beat fewer, longer-lived ones
 // with requests further ahead here (the dispatcher evens them out).
-constexpr int LINE_PITCH = 4 * QB + 16;
 __device__ __forceinline__ void group_put(unsigned char *patch, int lane, int j, v4i codes)
 {
     *reinterpret_cast<v4i *>(patch + (lane >> 1) * LINE_PITCH + QB * j + 16 * (lane & 1)) = codes;
@@ -327,10 +359,15 @@ __global__ __launch_bounds__(NT) void layernorm_fwd_kernel(const int8_t *q, cons
                                                            const float *beta, const float *mean, const float *rstd,
                                                            int R, int C, int8_t *qy, ST *sy)
 {
+    __shared__ __attribute__((aligned(16))) unsigned char line_patches[2 * QB * LINE_PITCH];
     const int lane = threadIdx.x & 63, wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
     const int SC = C / QB, RB = R / QB, S4 = (SC + WPB - 1) / WPB;
-    const int cb = (blockIdx.x % S4) * WPB + wave, grp = blockIdx.x / S4;
-    if (cb >= SC) return;                                          // a wave of the last, partial group of column blocks
+    const int cg = blockIdx.x % S4, grp = blockIdx.x / S4;
+    GroupLineStore lines(line_patches, lane, wave);
+    // a wave of the last, partial group of column blocks computes its neighbour's block again (and keeps none of it):
+    // it is needed for the whole-line stores of the group's rows
+    const bool mine = cg * WPB + wave < SC;
+    const int cb = mine ? cg * WPB + wave : SC - 1;
     const int col = cb * QB + (lane & 1) * 16;
     const int nrb = (RB - grp * CW_ROWS) < CW_ROWS ? (RB - grp * CW_ROWS) : CW_ROWS;      // uniform
     float g[16], bt[16];
@@ -365,10 +402,10 @@ __global__ __launch_bounds__(NT) void layernorm_fwd_kernel(const int8_t *q, cons
     }
 #pragma unroll
     for (int k = 0; k < CW_ROWS; ++k) {
-        if (k < nrb) {
+        if (k < nrb) {                                             // (uniform over the workgroup)
             const int rb = grp * CW_ROWS + k;
-            *reinterpret_cast<v4i *>(qy + (size_t)(rb * QB + (lane >> 1)) * C + col) = out[k];
-            if (lane == 0) store_scale(sy, rb * SC + cb, so[k]);
+            lines.store(out[k], qy, rb, cg, C);
+            if (mine && lane == 0) store_scale(sy, rb * SC + cb, so[k]);
         }
     }
 }
@@ -939,10 +976,20 @@ __global__ __launch_bounds__(NT) void add_kernel(const T *x1, const int8_t *q2, 
                                                  ST *s, float *rowsum, float *rowsq)
 {
     __shared__ __attribute__((aligned(16))) float ypatch_all[WPB][QB * ADD_PITCH];
+    __shared__ __attribute__((aligned(16))) unsigned char line_patches[2 * QB * LINE_PITCH];
     float *ypatch = ypatch_all[threadIdx.x >> 6];
-    JF_FOR_EACH_BLOCK(R, C)
+    const int lane = threadIdx.x & 63, wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
+    const int SC = C / QB, SG = (SC + WPB - 1) / WPB, ngrp = (R / QB) * SG;
+    GroupLineStore lines(line_patches, lane, wave);
+    // a workgroup: four adjacent column blocks of one row block (a group), so that the codes leave in whole lines
+    for (int grp = blockIdx.x; grp < ngrp; grp += gridDim.x)
     {
-        BlockPos pos(blk, SC, C, lane);
+        const int rbg = grp / SG, cg = grp - rbg * SG, cbg = cg * WPB + wave;
+        if (cbg >= SC) {                                           // (wave-uniform) beyond the row's end: the barrier only
+            lines.store(v4i{0, 0, 0, 0}, q, rbg, cg, C);
+            continue;
+        }
+        BlockPos pos(rbg * SC + cbg, SC, C, lane);
         float a[16], b[16];
         Load16<T>::run(x1 + pos.e0, a);
         unpack16(*reinterpret_cast<const v4i *>(q2 + pos.e0), load_scale(s2, pos.rb * SC + pos.cb), b);
@@ -961,7 +1008,7 @@ __global__ __launch_bounds__(NT) void add_kernel(const T *x1, const int8_t *q2, 
         }
         float scale;
         v4i codes = quantize16(a, 0.0f, rounding, seed, offset, pos.e0, &scale);
-        *reinterpret_cast<v4i *>(q + pos.e0) = codes;
+        lines.store(codes, q, rbg, cg, C);
         if (lane == 0) store_scale(s, pos.rb * SC + pos.cb, scale);
     }
 }
@@ -972,6 +1019,13 @@ static inline int grid_for_blocks(int R, int C)
     const long nblk = (long)(R / QB) * (C / QB);
     long g = (nblk + WPB - 1) / WPB;
     const long cap = 256L * 32;                    // 32 workgroups per CU is plenty of waves in flight
+    return (int)(g < cap ? g : cap);
+}
+
+// kernels whose workgroup takes a group of four adjacent column blocks of one row block per step
+static inline int grid_for_workgroup_groups(int R, int C)
+{
+    const long g = (long)(R / QB) * ((C / QB + WPB - 1) / WPB), cap = 256L * 32;
     return (int)(g < cap ? g : cap);
 }
 
@@ -1327,7 +1381,7 @@ int jf_add(const void *x1, int x1_dtype, const int8_t *q2, const void *s2, int R
     if (y1_dtype < JF_FP_F16 || y1_dtype > JF_FP_BF16) return JF_ERR_ENUM;
     if (!aligned16(x1) || !aligned16(y1) || !aligned16(q)) return JF_ERR_ALIGN;
     hipStream_t st = (hipStream_t)stream;
-    const int grid = grid_for_blocks(R, C);
+    const int grid = grid_for_workgroup_groups(R, C);
 #define JF_ADD(T, ST, OT)                                                                                         \
     JF_LAUNCH((add_kernel<T, ST, OT>), grid, 0, st, (const T *)x1, q2, (const ST *)s2, R, C, rounding, seed, offset, \
               (OT *)y1, q, (ST *)s, rowsum, rowsq)
